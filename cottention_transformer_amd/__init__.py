@@ -1,0 +1,19 @@
+"""MI355X-native cosine linear attention (causal, non-causal and recurrent-decode forms).
+
+The compute path is libcottention_hip.so (hand-written HIP for gfx950) behind the C ABI of
+include/cottention.h; this package is the torch-facing host side.  `Cuda_Kernel/` holds modules
+named like the reference's extension (`FastAttention2.kernel`, `FastAttention.forward/backward`,
+`Custom_Kernel.CustomAttention`) so its callers import them unchanged.
+"""
+from .ops import (causal_backward, causal_dot_product, decode_step, noncausal_backward,  # noqa: F401
+                  noncausal_dot_product)
+
+__all__ = ["causal_dot_product", "causal_backward", "noncausal_dot_product", "noncausal_backward", "decode_step",
+           "CustomAttention", "NonCausalAttention"]
+
+
+def __getattr__(name):
+    if name in ("CustomAttention", "NonCausalAttention"):
+        from . import autograd
+        return getattr(autograd, name)
+    raise AttributeError(name)

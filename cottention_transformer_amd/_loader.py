@@ -1,0 +1,53 @@
+"""ctypes binding of libcottention_hip.so (the C ABI declared in include/cottention.h).
+
+There is no CPU or PyTorch fallback behind these entry points: if the library cannot be built or
+loaded the import of this module's `lib()` raises.
+"""
+import ctypes
+import os
+
+_lib = None
+
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_HIP = 0, 1, 2, 3, 4
+F32, F64, F16, BF16 = 0, 1, 2, 3
+
+_vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+
+SIGNATURES = {
+    "cott_version": (_i, []),
+    "cott_last_error": (ctypes.c_char_p, []),
+    "cott_causal_workspace_bytes": (_sz, [_i] * 6),
+    "cott_causal_fwd": (_i, [_vp] * 4 + [_i] * 7 + [_vp, _sz, _vp]),
+    "cott_causal_bwd_workspace_bytes": (_sz, [_i] * 6),
+    "cott_causal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_noncausal_workspace_bytes": (_sz, [_i] * 6),
+    "cott_noncausal_fwd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_noncausal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_decode_step": (_i, [_vp] * 5 + [_i] * 5 + [_vp]),
+}
+
+
+def lib_path():
+    from . import build as _build
+    return _build.LIB_PATH
+
+
+def lib():
+    """The loaded library; built first if no shared object is present."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not os.path.exists(path):
+            from . import build as _build
+            _build.build()
+        handle = ctypes.CDLL(path)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)  # AttributeError here = header and library disagree
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def last_error():
+    return lib().cott_last_error().decode("utf-8", "replace")

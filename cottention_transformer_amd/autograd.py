@@ -1,0 +1,62 @@
+"""torch.autograd boundary: `CustomAttention` with the reference's signature, plus the
+non-causal counterpart.  Reference: Cuda_Kernel/Custom_Kernel.py:7-141."""
+import torch
+
+from . import ops
+
+_SUPPORTED = (torch.float32, torch.float64, torch.float16, torch.bfloat16)
+
+
+def _autocast_target(q, half_entry=False):
+    """Forward-time dtype rule of forward_<T>, Cuda_Kernel/combined_kernel_general.cu:377-389:
+    under autocast an fp32 Q is computed in the autocast type (fp16 only for the `float16` entry),
+    otherwise in Q's own type; K and V are converted to match."""
+    try:
+        enabled = torch.is_autocast_enabled("cuda")
+    except TypeError:  # older signature
+        enabled = torch.is_autocast_enabled()
+    if enabled and q.dtype == torch.float32:
+        return torch.float16 if half_entry else torch.bfloat16
+    return q.dtype
+
+
+class CustomAttention(torch.autograd.Function):
+    """O = causal cosine-attention core of (Q, K, V), tensors (N, H, S, D); apply(Q, K, V) -> O."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V):
+        if Q.dtype not in _SUPPORTED:
+            raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
+        Q, K, V = Q.contiguous(), K.contiguous(), V.contiguous()
+        ctx.save_for_backward(Q, K, V)  # saved before any autocast conversion (Custom_Kernel.py:16)
+        dt = _autocast_target(Q, half_entry=(Q.dtype == torch.float16))
+        return ops.causal_dot_product(Q.to(dt), K.to(dt), V.to(dt), False)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        Q, K, V = ctx.saved_tensors
+        if Q.dtype not in _SUPPORTED:
+            raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
+        # One fused call in the saved tensors' dtype replaces the three launches of
+        # Custom_Kernel.py:106-108 (same operand permutations inside the library).
+        g = grad_output.contiguous().to(Q.dtype)
+        return ops.causal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g)
+
+
+class NonCausalAttention(torch.autograd.Function):
+    """O = Q (K^T V): the BERT form (BERT_Trainer/BertCosAttention.py:249) as one fused operator."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V):
+        if Q.dtype not in _SUPPORTED:
+            raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
+        Q, K, V = Q.contiguous(), K.contiguous(), V.contiguous()
+        ctx.save_for_backward(Q, K, V)
+        dt = _autocast_target(Q)
+        return ops.noncausal_dot_product(Q.to(dt), K.to(dt), V.to(dt))
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        Q, K, V = ctx.saved_tensors
+        g = grad_output.contiguous().to(Q.dtype)
+        return ops.noncausal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g)

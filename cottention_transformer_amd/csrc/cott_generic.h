@@ -1,0 +1,194 @@
+// Plain-FMA kernels for every storage type (fp32, fp64, and 16-bit types whose head dims fall
+// outside the MFMA kernels' range), plus the bandwidth-bound decode step.
+#pragma once
+#include "cott_common.h"
+
+namespace cott {
+
+struct StF32 {
+    typedef float elem;
+    typedef float acc;
+    __device__ static __forceinline__ acc load(const elem *p) { return *p; }
+    __device__ static __forceinline__ void store(elem *p, acc v) { *p = v; }
+};
+struct StF64 {
+    typedef double elem;
+    typedef double acc;
+    __device__ static __forceinline__ acc load(const elem *p) { return *p; }
+    __device__ static __forceinline__ void store(elem *p, acc v) { *p = v; }
+};
+struct StBf16 {
+    typedef u16 elem;
+    typedef float acc;
+    __device__ static __forceinline__ acc load(const elem *p) { return Bf16::to_float(*p); }
+    __device__ static __forceinline__ void store(elem *p, acc v) { *p = Bf16::from_float(v); }
+};
+struct StFp16 {
+    typedef u16 elem;
+    typedef float acc;
+    __device__ static __forceinline__ acc load(const elem *p) { return Fp16::to_float(*p); }
+    __device__ static __forceinline__ void store(elem *p, acc v) { *p = Fp16::from_float(v); }
+};
+
+// Chunked scan with a [di][DJT] slice of the state in LDS; one workgroup per (j-slice, head)
+// walks the whole sequence.  CH (chunk length) and DJT (slice width) are chosen by the host so
+// that the dynamic LDS footprint fits.  CAUSAL=false: out = A (B^T C) in two passes.
+template <class ST, bool CAUSAL>
+__global__ __launch_bounds__(256) void generic_scan_kernel(const typename ST::elem *__restrict__ A,
+                                                           const typename ST::elem *__restrict__ B,
+                                                           const typename ST::elem *__restrict__ C,
+                                                           typename ST::elem *__restrict__ O, int N, int di, int dj,
+                                                           int CH, int DJT, int nslices, int reversed) {
+    typedef typename ST::acc acc_t;
+    extern __shared__ __attribute__((aligned(32))) unsigned char smem_raw[];
+    acc_t *sA = reinterpret_cast<acc_t *>(smem_raw);  // [CH][di+1]
+    acc_t *sB = sA + CH * (di + 1);                   // [CH][di+1]
+    acc_t *sC = sB + CH * (di + 1);                   // [CH][DJT]
+    acc_t *sP = sC + CH * DJT;                        // [CH][CH+1]
+    acc_t *sS = sP + CH * (CH + 1);                   // [di][DJT]
+    const int tid = threadIdx.x;
+    const int j0 = (blockIdx.x % nslices) * DJT, bh = blockIdx.x / nslices;
+    A += (size_t)bh * N * di;
+    B += (size_t)bh * N * di;
+    C += (size_t)bh * N * dj;
+    O += (size_t)bh * N * dj;
+    const int nchunks = (N + CH - 1) / CH;
+    const int lda = di + 1;
+
+    for (int x = tid; x < di * DJT; x += 256) sS[x] = (acc_t)0;
+
+    auto load_bc = [&](int row0) {
+        for (int x = tid; x < CH * di; x += 256) {
+            const int r = x / di, i = x % di;
+            sB[r * lda + i] = (row0 + r < N) ? ST::load(B + (size_t)(row0 + r) * di + i) : (acc_t)0;
+        }
+        for (int x = tid; x < CH * DJT; x += 256) {
+            const int r = x / DJT, jj = x % DJT;
+            sC[x] = (row0 + r < N && j0 + jj < dj) ? ST::load(C + (size_t)(row0 + r) * dj + j0 + jj) : (acc_t)0;
+        }
+    };
+    auto update_state = [&]() {
+        for (int x = tid; x < di * DJT; x += 256) {
+            const int i = x / DJT, jj = x % DJT;
+            acc_t s = sS[x];
+            for (int t = 0; t < CH; ++t) s += sB[t * lda + i] * sC[t * DJT + jj];
+            sS[x] = s;
+        }
+    };
+
+    if (!CAUSAL) {
+        for (int c = 0; c < nchunks; ++c) {
+            __syncthreads();
+            load_bc(c * CH);
+            __syncthreads();
+            update_state();
+        }
+    }
+
+    for (int p = 0; p < nchunks; ++p) {
+        const int row0 = (reversed ? nchunks - 1 - p : p) * CH;
+        __syncthreads();
+        for (int x = tid; x < CH * di; x += 256) {
+            const int r = x / di, i = x % di;
+            sA[r * lda + i] = (row0 + r < N) ? ST::load(A + (size_t)(row0 + r) * di + i) : (acc_t)0;
+        }
+        if (CAUSAL) load_bc(row0);
+        __syncthreads();
+        if (CAUSAL) {
+            for (int x = tid; x < CH * CH; x += 256) {
+                const int r = x / CH, t = x % CH;
+                acc_t s = (acc_t)0;
+                if (reversed ? (t >= r) : (t <= r))
+                    for (int i = 0; i < di; ++i) s += sA[r * lda + i] * sB[t * lda + i];
+                sP[r * (CH + 1) + t] = s;
+            }
+            __syncthreads();
+        }
+        for (int x = tid; x < CH * DJT; x += 256) {
+            const int r = x / DJT, jj = x % DJT;
+            acc_t s = (acc_t)0;
+            if (CAUSAL)
+                for (int t = 0; t < CH; ++t) s += sP[r * (CH + 1) + t] * sC[t * DJT + jj];
+            for (int i = 0; i < di; ++i) s += sA[r * lda + i] * sS[i * DJT + jj];
+            if (row0 + r < N && j0 + jj < dj) ST::store(O + (size_t)(row0 + r) * dj + j0 + jj, s);
+        }
+        if (CAUSAL) {
+            __syncthreads();
+            update_state();
+        }
+    }
+}
+
+// Decode step: one workgroup per (batch, head) streams its [dk][dv] state once.
+//   S[i][j] += k[i] v[j] ;  o[j] = sum_i q[i] S[i][j]
+// Thread t owns a 4-wide column strip (t % nvb) and every rg-th row starting at t / nvb; rows
+// are processed 8 at a time with all loads issued before the first store.
+template <class ST, class SF /* state scalar: float or double */>
+__global__ __launch_bounds__(256) void decode_kernel(SF *__restrict__ S, const typename ST::elem *__restrict__ q,
+                                                     const typename ST::elem *__restrict__ k,
+                                                     const typename ST::elem *__restrict__ v,
+                                                     typename ST::elem *__restrict__ o, int dk, int dv) {
+    typedef SF __attribute__((ext_vector_type(4))) sf4;
+    extern __shared__ __attribute__((aligned(32))) unsigned char smem_raw[];
+    SF *sq = reinterpret_cast<SF *>(smem_raw);  // [dk]
+    SF *sk = sq + dk;                           // [dk]
+    sf4 *sred = reinterpret_cast<sf4 *>(sk + dk);  // [256]
+    const int tid = threadIdx.x, bh = blockIdx.x;
+    S += (size_t)bh * dk * dv;
+    q += (size_t)bh * dk;
+    k += (size_t)bh * dk;
+    v += (size_t)bh * dv;
+    o += (size_t)bh * dv;
+    for (int i = tid; i < dk; i += 256) {
+        sq[i] = (SF)ST::load(q + i);
+        sk[i] = (SF)ST::load(k + i);
+    }
+    __syncthreads();
+    const int nv = dv / 4;
+    const int nvb = nv < 256 ? nv : 256;
+    const int rg = 256 / nvb;
+    const int mc = tid % nvb, mr = tid / nvb;
+    for (int c0 = 0; c0 < nv; c0 += nvb) {
+        const int c4 = c0 + mc;
+        const bool live = (mr < rg) && (c4 < nv);
+        sf4 acc = {0, 0, 0, 0};
+        if (live) {
+            sf4 vv;
+            vv.x = (SF)ST::load(v + 4 * c4);
+            vv.y = (SF)ST::load(v + 4 * c4 + 1);
+            vv.z = (SF)ST::load(v + 4 * c4 + 2);
+            vv.w = (SF)ST::load(v + 4 * c4 + 3);
+            sf4 *col = reinterpret_cast<sf4 *>(S) + c4;
+            for (int r0 = mr; r0 < dk; r0 += 8 * rg) {
+                sf4 s[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int r = r0 + u * rg;
+                    if (r < dk) s[u] = __builtin_nontemporal_load(col + (size_t)r * nv);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int r = r0 + u * rg;
+                    if (r < dk) {
+                        s[u] += sk[r] * vv;
+                        __builtin_nontemporal_store(s[u], col + (size_t)r * nv);
+                        acc += sq[r] * s[u];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        sred[tid] = acc;
+        __syncthreads();
+        if (mr == 0 && c4 < nv) {
+            sf4 t = sred[mc];
+            for (int r = 1; r < rg; ++r) t += sred[r * nvb + mc];
+            ST::store(o + 4 * c4, (typename ST::acc)t.x);
+            ST::store(o + 4 * c4 + 1, (typename ST::acc)t.y);
+            ST::store(o + 4 * c4 + 2, (typename ST::acc)t.z);
+            ST::store(o + 4 * c4 + 3, (typename ST::acc)t.w);
+        }
+    }
+}
+
+}  // namespace cott

@@ -1,0 +1,91 @@
+// Plain-FMA fallback launches (all dtypes) and the decode step.
+#include "cott_generic.h"
+#include "cott_launch.h"
+#include "../../include/cottention.h"
+
+namespace cott {
+namespace {
+
+constexpr size_t kLdsBudget = 150 * 1024;
+
+struct GenericTiling {
+    int CH, DJT;
+    size_t bytes;
+};
+
+size_t generic_lds_bytes(int di, int CH, int DJT, size_t acc_size) {
+    return ((size_t)2 * CH * (di + 1) + (size_t)CH * DJT + (size_t)CH * (CH + 1) + (size_t)di * DJT) * acc_size;
+}
+
+bool pick_tiling(int di, size_t acc_size, GenericTiling *out) {
+    static const int cands[][2] = {{32, 32}, {32, 16}, {16, 16}, {8, 16}, {8, 8}, {4, 8}};
+    for (const auto &c : cands) {
+        const size_t b = generic_lds_bytes(di, c[0], c[1], acc_size);
+        if (b <= kLdsBudget) {
+            *out = GenericTiling{c[0], c[1], b};
+            return true;
+        }
+    }
+    return false;
+}
+
+size_t acc_size_of(int dtype) { return dtype == COTT_F64 ? sizeof(double) : sizeof(float); }
+
+template <class ST, bool CAUSAL>
+hipError_t run_generic(const ScanArgs &a) {
+    GenericTiling t;
+    if (!pick_tiling(a.di, sizeof(typename ST::acc), &t)) return hipErrorInvalidValue;
+    auto kern = generic_scan_kernel<ST, CAUSAL>;
+    if (t.bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)t.bytes);
+        if (e != hipSuccess) return e;
+    }
+    const int nslices = (a.dj + t.DJT - 1) / t.DJT;
+    typedef typename ST::elem E;
+    kern<<<dim3((unsigned)(a.BH * nslices)), dim3(256), t.bytes, a.stream>>>(
+        static_cast<const E *>(a.A), static_cast<const E *>(a.B), static_cast<const E *>(a.C), static_cast<E *>(a.O),
+        a.N, a.di, a.dj, t.CH, t.DJT, nslices, a.reversed);
+    return hipGetLastError();
+}
+
+template <class ST, class SF>
+hipError_t run_decode(void *state, const void *q, const void *k, const void *v, void *o, int BH, int dk, int dv,
+                      hipStream_t stream) {
+    typedef typename ST::elem E;
+    const size_t lds = (size_t)2 * dk * sizeof(SF) + 256 * 4 * sizeof(SF);
+    decode_kernel<ST, SF><<<dim3((unsigned)BH), dim3(256), lds, stream>>>(
+        static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
+        static_cast<E *>(o), dk, dv);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool generic_fits(int dtype, int di) {
+    GenericTiling t;
+    return pick_tiling(di, acc_size_of(dtype), &t);
+}
+
+hipError_t launch_generic(int dtype, bool causal, const ScanArgs &a) {
+    switch (dtype) {
+        case COTT_F32: return causal ? run_generic<StF32, true>(a) : run_generic<StF32, false>(a);
+        case COTT_F64: return causal ? run_generic<StF64, true>(a) : run_generic<StF64, false>(a);
+        case COTT_F16: return causal ? run_generic<StFp16, true>(a) : run_generic<StFp16, false>(a);
+        case COTT_BF16: return causal ? run_generic<StBf16, true>(a) : run_generic<StBf16, false>(a);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_decode(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH,
+                         int dk, int dv, hipStream_t stream) {
+    switch (dtype) {
+        case COTT_F32: return run_decode<StF32, float>(state, q, k, v, o, BH, dk, dv, stream);
+        case COTT_F64: return run_decode<StF64, double>(state, q, k, v, o, BH, dk, dv, stream);
+        case COTT_F16: return run_decode<StFp16, float>(state, q, k, v, o, BH, dk, dv, stream);
+        case COTT_BF16: return run_decode<StBf16, float>(state, q, k, v, o, BH, dk, dv, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace cott

@@ -1,0 +1,164 @@
+"""Host-side operators over torch tensors: thin wrappers that validate, allocate outputs and
+workspace with torch, and enqueue the HIP kernels on torch's current stream through the C ABI.
+
+Tensor contract is the reference's: (B, H, N, D) for q/k/v/o (Cuda_Kernel/combined_kernel_general.cu
+:360-369), state (B, H, Dk, Dv) for decode.  Nothing here computes on the CPU.
+"""
+import torch
+
+from . import _loader
+
+_DTYPES = {torch.float32: _loader.F32, torch.float64: _loader.F64, torch.float16: _loader.F16,
+           torch.bfloat16: _loader.BF16}
+
+
+def _check(rc, what):
+    if rc == _loader.OK:
+        return
+    msg = _loader.last_error() or f"{what} failed with status {rc}"
+    raise RuntimeError(msg)
+
+
+def _dtype_code(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise ValueError("Only float32, float64, float16, and bfloat16 are supported") from None
+
+
+def _require_gpu(**tensors):
+    for name, t in tensors.items():
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be a CUDA tensor")  # wording of combined_kernel_general.cu:355-357
+    devs = {t.device for t in tensors.values()}
+    if len(devs) != 1:
+        raise RuntimeError(f"all tensors must be on the same device, got {sorted(map(str, devs))}")
+
+
+def _shapes(q, k, v):
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise RuntimeError("Q, K and V must have shape (N, H, S, D)")
+    if q.size(3) != k.size(3):
+        raise RuntimeError("Q and K must have the same dimension")  # combined_kernel_general.cu:365
+    if q.shape[:3] != k.shape[:3] or q.shape[:3] != v.shape[:3]:
+        raise RuntimeError(f"Q, K and V must agree in (N, H, S): {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")
+    b, h, n, dk = q.shape
+    return b, h, n, dk, v.size(3)
+
+
+def _workspace(nbytes, device):
+    if nbytes == 0:
+        return None, 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return ws, ws.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def causal_dot_product(q, k, v, reversed=False):
+    """o[s,j] = sum_i q[s,i] sum_{s'<=s (>=s if reversed)} k[s',i] v[s',j]; all of one dtype."""
+    _require_gpu(Q=q, K=k, V=v)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("Q, K and V must have the same dtype")
+    code = _dtype_code(q)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        ws, ws_ptr = _workspace(L.cott_causal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+        rc = L.cott_causal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,
+                               int(bool(reversed)), ws_ptr, ws.numel() if ws is not None else 0, _stream())
+    _check(rc, "cott_causal_fwd")
+    return o
+
+
+def causal_backward(q, k, v, grad_out):
+    """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out."""
+    _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if grad_out.shape != v.shape:
+        raise RuntimeError(f"prev_grad must have V's shape {tuple(v.shape)}, got {tuple(grad_out.shape)}")
+    if not (q.dtype == k.dtype == v.dtype == grad_out.dtype):
+        raise RuntimeError("Q, K, V and prev_grad must have the same dtype")
+    code = _dtype_code(q)
+    q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), grad_out.contiguous()
+    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        ws, ws_ptr = _workspace(L.cott_causal_bwd_workspace_bytes(b, h, n, dk, dv, code), q.device)
+        rc = L.cott_causal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(), dk_.data_ptr(),
+                               dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0,
+                               _stream())
+    _check(rc, "cott_causal_bwd")
+    return dq, dk_, dv_
+
+
+def noncausal_dot_product(q, k, v):
+    """o = q (k^T v) per (batch, head): BERT_Trainer/BertCosAttention.py:249."""
+    _require_gpu(Q=q, K=k, V=v)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("Q, K and V must have the same dtype")
+    code = _dtype_code(q)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        ws, ws_ptr = _workspace(L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+        rc = L.cott_noncausal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,
+                                  ws_ptr, ws.numel() if ws is not None else 0, _stream())
+    _check(rc, "cott_noncausal_fwd")
+    return o
+
+
+def noncausal_backward(q, k, v, grad_out):
+    """(dQ, dK, dV) of noncausal_dot_product."""
+    _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if grad_out.shape != v.shape:
+        raise RuntimeError(f"prev_grad must have V's shape {tuple(v.shape)}, got {tuple(grad_out.shape)}")
+    if not (q.dtype == k.dtype == v.dtype == grad_out.dtype):
+        raise RuntimeError("Q, K, V and prev_grad must have the same dtype")
+    code = _dtype_code(q)
+    q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), grad_out.contiguous()
+    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        ws, ws_ptr = _workspace(L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+        rc = L.cott_noncausal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(),
+                                  dk_.data_ptr(), dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr,
+                                  ws.numel() if ws is not None else 0, _stream())
+    _check(rc, "cott_noncausal_bwd")
+    return dq, dk_, dv_
+
+
+def decode_step(state, q, k, v, out=None):
+    """One recurrent step, in place on `state` (B,H,Dk,Dv; fp32, or fp64 for fp64 inputs):
+    state += k v^T ; returns o = q state  (GPT_Trainer/GPTCosAttention.py:264,267).
+    q,k: (B,H,Dk); v: (B,H,Dv).  The reference's `past_KV` is `state.transpose(-1,-2)`."""
+    _require_gpu(state=state, q=q, k=k, v=v)
+    if state.dim() != 4 or q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise RuntimeError("decode_step: state (B,H,Dk,Dv), q/k (B,H,Dk), v (B,H,Dv)")
+    b, h, dk, dv = state.shape
+    if q.shape != (b, h, dk) or k.shape != (b, h, dk) or v.shape != (b, h, dv):
+        raise RuntimeError("decode_step: q/k/v do not match the state shape")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("q, k and v must have the same dtype")
+    code = _dtype_code(q)
+    want = torch.float64 if q.dtype == torch.float64 else torch.float32
+    if state.dtype != want or not state.is_contiguous():
+        raise RuntimeError(f"decode_step: state must be a contiguous {want} tensor (it is updated in place)")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    if out is None:
+        out = torch.empty((b, h, dv), dtype=q.dtype, device=q.device)
+    elif out.shape != (b, h, dv) or out.dtype != q.dtype or not out.is_contiguous() or out.device != q.device:
+        raise RuntimeError("decode_step: bad `out` tensor")
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        rc = L.cott_decode_step(state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b, h, dk,
+                                dv, code, _stream())
+    _check(rc, "cott_decode_step")
+    return out

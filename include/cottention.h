@@ -1,0 +1,98 @@
+/*
+ * cottention.h -- C ABI of libcottention_hip.so: cosine linear attention for AMD MI355X (gfx950).
+ *
+ * This is the boundary a host binds instead of the reference's pybind/ATen extension.  All entry
+ * points take raw device pointers, plain sizes and a HIP stream (passed as void*; NULL = the
+ * default stream).  The library never allocates, frees or synchronises: outputs and workspaces
+ * are caller-owned device memory, kernels are enqueued on the given stream and the call returns.
+ *
+ * Tensors are contiguous row-major (B, H, N, D) exactly as the reference kernels index them
+ * (Cuda_Kernel/combined_kernel_general.cu:136 `((n*H+h)*S+s)*D+d`).  Pointers must be 16-byte
+ * aligned.  `dtype` selects the storage type of q/k/v/o; accumulation is fp32 (fp64 for
+ * COTT_F64), unlike the reference, which accumulates in the storage type (:121,:133).
+ *
+ * Every function returns COTT_OK or an error code; cott_last_error() gives the text for the most
+ * recent failure on the calling thread.  Shape rules follow combined_kernel_general.cu:365-374:
+ * q and k share their last dimension, every head dimension is a multiple of 16 and at least 32.
+ */
+#ifndef COTTENTION_H
+#define COTTENTION_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define COTT_API __attribute__((visibility("default")))
+
+#define COTT_OK 0
+#define COTT_ERR_INVALID 1     /* bad pointer, shape or flag                        */
+#define COTT_ERR_UNSUPPORTED 2 /* legal request this build has no kernel for       */
+#define COTT_ERR_WORKSPACE 3   /* workspace missing or smaller than required       */
+#define COTT_ERR_HIP 4         /* the HIP runtime reported a launch error          */
+
+typedef enum cott_dtype {
+    COTT_F32 = 0,  /* kernel.float32  : combined_kernel_general.cu:445 */
+    COTT_F64 = 1,  /* kernel.float64  : :446                           */
+    COTT_F16 = 2,  /* kernel.float16  : :447                           */
+    COTT_BF16 = 3  /* kernel.bfloat16 : :449                           */
+} cott_dtype;
+
+/* Library version, major*10000 + minor*100 + patch. */
+COTT_API int cott_version(void);
+
+/* Text of the last error raised on this thread ("" if none).  Replaces the c10::Error that
+ * TORCH_CHECK throws in combined_kernel_general.cu:355-374. */
+COTT_API const char *cott_last_error(void);
+
+/* ---- generic causal op ---------------------------------------------------------------------
+ *   o[s,j] = sum_i q[s,i] * sum_{s' <= s (>= s if reversed)} k[s',i] * v[s',j]
+ * Replaces kernel_call<T> / forward_<T>, Cuda_Kernel/combined_kernel_general.cu:257-289,352-429
+ * (Python: FastAttention2.kernel.<dtype>(Q,K,V,block_size,inplace,reversed), :444-454).
+ * q,k: (B,H,N,Dk); v,o: (B,H,N,Dv).  The diagonal s'=s is included.  `reversed` is the flag of
+ * :126-130.  Workspace: cott_causal_workspace_bytes() bytes of device memory (may be 0). */
+COTT_API size_t cott_causal_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype);
+COTT_API int cott_causal_fwd(const void *q, const void *k, const void *v, void *o,
+                    int B, int H, int N, int Dk, int Dv, int dtype, int reversed,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- causal backward ------------------------------------------------------------------------
+ * (dq, dk, dv) of o = cott_causal_fwd(q,k,v) contracted with d_o.  Replaces the three launches
+ * of CustomAttention.backward, Cuda_Kernel/Custom_Kernel.py:106-108 (closed forms :63,:68,:72)
+ * and the older fused entry point backward_<T>, Cuda_Kernel/backwardv2_comb.cu:172-224
+ * (Python: FastAttention.backward.<dtype>(Q,K,V,prev_grad,block_size) -> [dQ,dK,dV]).
+ * d_o, dv: (B,H,N,Dv); dq, dk: (B,H,N,Dk). */
+COTT_API size_t cott_causal_bwd_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype);
+COTT_API int cott_causal_bwd(const void *q, const void *k, const void *v, const void *d_o,
+                    void *dq, void *dk, void *dv,
+                    int B, int H, int N, int Dk, int Dv, int dtype,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- non-causal form ------------------------------------------------------------------------
+ *   o = q (k^T v)   per (batch, head)
+ * Replaces the two einsums of BERT_Trainer/BertCosAttention.py:249 (the (QK^T)V branch at :222
+ * is the same value).  Backward: dq = d_o (v^T k), dk = v (d_o^T q)
+ * (GPT_Trainer/GPTCosAttention.py:34-35), dv = k (q^T d_o). */
+COTT_API size_t cott_noncausal_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype);
+COTT_API int cott_noncausal_fwd(const void *q, const void *k, const void *v, void *o,
+                       int B, int H, int N, int Dk, int Dv, int dtype,
+                       void *workspace, size_t workspace_bytes, void *stream);
+COTT_API int cott_noncausal_bwd(const void *q, const void *k, const void *v, const void *d_o,
+                       void *dq, void *dk, void *dv,
+                       int B, int H, int N, int Dk, int Dv, int dtype,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- recurrent decode step ------------------------------------------------------------------
+ *   S[b,h,dk,dv] += k[b,h,dk] * v[b,h,dv] ;  o[b,h,dv] = sum_dk q[b,h,dk] * S[b,h,dk,dv]
+ * Replaces the per-token body of GPT_Trainer/GPTCosAttention.py:262-269 (:264 update, :267 read;
+ * the output uses the UPDATED state).  `state` is caller-owned, (B,H,Dk,Dv), fp32 (fp64 for
+ * COTT_F64) and updated in place; the reference keeps the transposed orientation (B,H,Dv,Dk) in
+ * fp64 (:80).  q,k: (B,H,Dk); v,o: (B,H,Dv) in `dtype`.  Needs no workspace. */
+COTT_API int cott_decode_step(void *state, const void *q, const void *k, const void *v, void *o,
+                     int B, int H, int Dk, int Dv, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COTTENTION_H */
