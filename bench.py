@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Benchmark of the cosine-linear-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A step is one causal forward + backward (dQ, dK, dV) over one synthetic batch at the headline
+shape B=8 H=16 N=2048 D=64 bf16, called through the C ABI on torch's current stream with every
+input already resident in HBM.  Prints ONE JSON line: whole-job tokens/s, the roofline object of
+the dominant kernel (HIP events recorded by the library around each of its launches), and the CPU
+baseline (the reference's PyTorch cumsum formulation timed on the host cores of this box).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary configs (non-causal, decode, long)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+def make_inputs(torch, b, h, n, dk, dv, dtype, device, seed=0, grad=True):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.nn.functional.normalize(torch.randn(b, h, n, dk, generator=g), p=2, dim=-1)
+    k = torch.nn.functional.normalize(torch.randn(b, h, n, dk, generator=g), p=2, dim=-1)
+    v = torch.randn(b, h, n, dv, generator=g)
+    out = [q, k, v]
+    if grad:
+        out.append(torch.randn(b, h, n, dv, generator=g))
+    return [t.to(dtype).to(device) for t in out]
+
+
+def time_region(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def cpu_baseline(torch):
+    """Reference CPU path: cumsum form forward (GPT_Trainer/GPTCosAttention.py:319) + autograd
+    backward, fp32, on a bounded sample: one batch element of the headline shape."""
+    from oracle import torch_forms as tf
+    b, h, n, d = 1, 16, 2048, 64
+    q, k, v, g = tf.synthetic_inputs((b, h, n, d), seed=0, dtype=torch.float32)
+    times = []
+    for it in range(4):
+        qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+        t0 = time.perf_counter()
+        tf.causal_cumsum(qa, ka, va).backward(g)
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times[1:])
+    return {"value": b * n / t, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"(B,H,N,D)=({b},{h},{n},{d}) fp32: 1 of the 8 batch elements of the headline shape, torch cumsum "
+                      f"form fwd + autograd bwd, median of 3 after 1 warm-up; {t:.2f} s per pass"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+    import cottention_transformer_amd as ct
+    from cottention_transformer_amd import _loader
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, N, D = 8, 16, 2048, 64
+    q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
+
+    def step():
+        o = ct.causal_dot_product(q, k, v)
+        grads = ct.causal_backward(q, k, v, do)
+        return o, grads
+
+    sec = time_region(torch, step, args.steps, args.warmup)
+    tokens_per_s = B * N / sec
+
+    # forward-only / backward-only split (same buffers)
+    sec_f = time_region(torch, lambda: ct.causal_dot_product(q, k, v), args.steps, 5)
+    sec_b = time_region(torch, lambda: ct.causal_backward(q, k, v, do), args.steps, 5)
+
+    # Per-kernel durations: the library brackets each launch with HIP events on the launch stream.
+    _loader.profile_enable(True)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    _loader.profile_enable(False)
+    kern = {}
+    for name in _loader.KERNEL_IDS:
+        ms, n = _loader.profile_read(name)
+        if n:
+            kern[name] = {"launches_per_step": n / args.steps, "avg_us": 1e3 * ms / n, "us_per_step": 1e3 * ms / args.steps}
+    dominant = max(kern, key=lambda kname: kern[kname]["us_per_step"])
+    esz = 2
+    tensor_bytes = B * H * N * D * esz
+    # algorithmic bytes of ONE launch of each kernel family at this shape (tensor passes x 32 MiB)
+    passes = {"scan": 4, "bwd_dkdv": 6, "group_state": 2}
+    alg_bytes = passes.get(dominant, 4) * tensor_bytes
+    achieved = alg_bytes / (kern[dominant]["avg_us"] * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                "kernel": dominant, "avg_us": kern[dominant]["avg_us"],
+                "algorithmic_bytes_per_launch": alg_bytes,
+                "whole_step": {"algorithmic_bytes": 11 * tensor_bytes,
+                               "achieved_GBps": 11 * tensor_bytes / sec / 1e9,
+                               "frac_hbm": 11 * tensor_bytes / sec / 1e9 / HBM_PEAK_GBS,
+                               "algorithmic_tflops": 14.0 * B * H * N * D * D / sec / 1e12,
+                               "frac_mfma_bf16": 14.0 * B * H * N * D * D / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS}}
+
+    extras = {"fwd_us": sec_f * 1e6, "bwd_us": sec_b * 1e6, "kernels": kern}
+    if not args.no_extras:
+        extras.update(run_extras(torch, ct, dev))
+
+    out = {
+        "metric": "causal cos-attn fwd+bwd tokens/s, B8 H16 N2048 D64 bf16; % MFMA/HBM peak",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[2]: GPT-300M-shape causal cosine attention fwd+bwd (dQ,dK,dV), "
+                               "B=8 H=16 N=2048 D=64 bf16, fp32 state carry", "B": B, "H": H, "N": N, "D": D},
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(torch),
+        "extras": extras,
+    }
+    print(json.dumps(out))
+
+
+def run_extras(torch, ct, dev):
+    """Secondary configurations of the same path (not the headline value)."""
+    ex = {}
+    # non-causal forward, B=32 H=12 N=512 D=64 bf16
+    b, h, n, d = 32, 12, 512, 64
+    q, k, v = make_inputs(torch, b, h, n, d, d, torch.bfloat16, dev, grad=False)
+    s = time_region(torch, lambda: ct.noncausal_dot_product(q, k, v), 100, 10)
+    byts = 4 * b * h * n * d * 2
+    ex["noncausal_fwd_B32_H12_N512_D64"] = {"us": s * 1e6, "tokens_per_s": b * n / s, "GBps": byts / s / 1e9,
+                                            "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS}
+    del q, k, v
+    # recurrent decode, state (256,16,128,128) fp32, 512 consecutive steps with fresh q,k,v per step
+    b, h, d, steps = 256, 16, 128, 512
+    g = torch.Generator(device=dev).manual_seed(0)
+    S = (0.01 * torch.randn(b, h, d, d, generator=g, device=dev, dtype=torch.float32)).contiguous()
+    qs = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g, device=dev), dim=-1).to(torch.bfloat16)
+    ks = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g, device=dev), dim=-1).to(torch.bfloat16)
+    vs = torch.randn(steps, b, h, d, generator=g, device=dev).to(torch.bfloat16)
+    out = torch.empty(b, h, d, dtype=torch.bfloat16, device=dev)
+    for t in range(8):
+        ct.decode_step(S, qs[t], ks[t], vs[t], out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(steps):
+        ct.decode_step(S, qs[t], ks[t], vs[t], out=out)
+    torch.cuda.synchronize()
+    s = time.perf_counter() - t0
+    byts = steps * (2 * b * h * d * d * 4 + 4 * b * h * d * 2)
+    ex["decode_B256_H16_D128_512steps"] = {"ms_total": s * 1e3, "us_per_step": s / steps * 1e6,
+                                           "tokens_per_s": b * steps / s, "GBps": byts / s / 1e9,
+                                           "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS,
+                                           "note": "state is 256 MiB = the size of the last-level cache; "
+                                                   "GB/s is algorithmic bytes / time"}
+    del S, qs, ks, vs
+    # long context fwd+bwd, B=1 H=16 D=128 bf16, N sweep
+    sweep = {}
+    for n in (4096, 16384, 65536):
+        q, k, v, do = make_inputs(torch, 1, 16, n, 128, 128, torch.bfloat16, dev)
+
+        def step():
+            ct.causal_dot_product(q, k, v)
+            ct.causal_backward(q, k, v, do)
+        s = time_region(torch, step, 20, 3)
+        byts = 11 * 16 * n * 128 * 2
+        sweep[str(n)] = {"us": s * 1e6, "tokens_per_s": n / s, "GBps": byts / s / 1e9,
+                         "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS}
+        del q, k, v, do
+    ex["long_context_fwd_bwd_B1_H16_D128"] = sweep
+    return ex
+
+
+if __name__ == "__main__":
+    main()

@@ -24,7 +24,25 @@ SIGNATURES = {
     "cott_noncausal_fwd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_decode_step": (_i, [_vp] * 5 + [_i] * 5 + [_vp]),
+    "cott_profile_enable": (_i, [_i]),
+    "cott_profile_read": (_i, [_i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_long)]),
+    "cott_kernel_name": (ctypes.c_char_p, [_i]),
 }
+
+KERNEL_IDS = {"group_state": 0, "state_prefix": 1, "scan": 2, "apply": 3, "bwd_dkdv": 4, "generic": 5, "decode": 6}
+
+
+def profile_enable(on):
+    lib().cott_profile_enable(int(bool(on)))
+
+
+def profile_read(kernel):
+    """(total_ms, launches) of one kernel family since the last read; waits for those launches."""
+    ms, n = ctypes.c_double(0.0), ctypes.c_long(0)
+    rc = lib().cott_profile_read(KERNEL_IDS[kernel], ctypes.byref(ms), ctypes.byref(n))
+    if rc != OK:
+        raise RuntimeError(last_error())
+    return ms.value, n.value
 
 
 def lib_path():

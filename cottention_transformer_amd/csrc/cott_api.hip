@@ -6,9 +6,41 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
+#include <vector>
 
 #include "../../include/cottention.h"
 #include "cott_launch.h"
+
+namespace cott {
+namespace {
+struct ProfRecord {
+    int id;
+    hipEvent_t start, stop;
+};
+std::mutex g_prof_mu;
+std::vector<ProfRecord> g_prof_records;
+bool g_prof_on = false;
+}  // namespace
+
+ProfScope::ProfScope(int kernel_id, hipStream_t stream) : id_(kernel_id), stream_(stream), start_(nullptr), active_(false) {
+    if (!g_prof_on) return;
+    if (hipEventCreate(&start_) != hipSuccess) return;
+    active_ = hipEventRecord(start_, stream_) == hipSuccess;
+    if (!active_) (void)hipEventDestroy(start_);
+}
+
+ProfScope::~ProfScope() {
+    if (!active_) return;
+    hipEvent_t stop;
+    if (hipEventCreate(&stop) != hipSuccess || hipEventRecord(stop, stream_) != hipSuccess) {
+        (void)hipEventDestroy(start_);
+        return;
+    }
+    std::lock_guard<std::mutex> lock(g_prof_mu);
+    g_prof_records.push_back(ProfRecord{id_, start_, stop});
+}
+}  // namespace cott
 
 namespace {
 
@@ -130,6 +162,45 @@ size_t noncausal_ws_bytes(long BH, int N, int di, int dj, int dtype) {
 extern "C" {
 
 int cott_version(void) { return 100; }
+
+int cott_profile_enable(int on) {
+    std::lock_guard<std::mutex> lock(cott::g_prof_mu);
+    cott::g_prof_on = on != 0;
+    return COTT_OK;
+}
+
+int cott_profile_read(int kernel_id, double *total_ms, long *launches) {
+    if (kernel_id < 0 || kernel_id >= cott::K_COUNT || !total_ms || !launches)
+        return fail(COTT_ERR_INVALID, "cott_profile_read: bad argument");
+    std::lock_guard<std::mutex> lock(cott::g_prof_mu);
+    double sum = 0.0;
+    long n = 0;
+    std::vector<cott::ProfRecord> keep;
+    for (const cott::ProfRecord &r : cott::g_prof_records) {
+        if (r.id != kernel_id) {
+            keep.push_back(r);
+            continue;
+        }
+        float ms = 0.f;
+        if (hipEventSynchronize(r.stop) == hipSuccess && hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+            sum += ms;
+            ++n;
+        }
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    cott::g_prof_records.swap(keep);
+    *total_ms = sum;
+    *launches = n;
+    return COTT_OK;
+}
+
+const char *cott_kernel_name(int kernel_id) {
+    static const char *names[cott::K_COUNT] = {"group_state_kernel", "state_prefix_kernel", "scan_kernel<causal>",
+                                               "scan_kernel<apply>", "bwd_dkdv_kernel",     "generic_scan_kernel",
+                                               "decode_kernel"};
+    return (kernel_id >= 0 && kernel_id < cott::K_COUNT) ? names[kernel_id] : "";
+}
 
 const char *cott_last_error(void) { return g_err; }
 

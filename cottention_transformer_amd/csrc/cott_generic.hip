@@ -43,6 +43,7 @@ hipError_t run_generic(const ScanArgs &a) {
     }
     const int nslices = (a.dj + t.DJT - 1) / t.DJT;
     typedef typename ST::elem E;
+    ProfScope ps(K_GENERIC, a.stream);
     kern<<<dim3((unsigned)(a.BH * nslices)), dim3(256), t.bytes, a.stream>>>(
         static_cast<const E *>(a.A), static_cast<const E *>(a.B), static_cast<const E *>(a.C), static_cast<E *>(a.O),
         a.N, a.di, a.dj, t.CH, t.DJT, nslices, a.reversed);
@@ -54,6 +55,7 @@ hipError_t run_decode(void *state, const void *q, const void *k, const void *v, 
                       hipStream_t stream) {
     typedef typename ST::elem E;
     const size_t lds = (size_t)2 * dk * sizeof(SF) + 256 * 4 * sizeof(SF);
+    ProfScope ps(K_DECODE, stream);
     decode_kernel<ST, SF><<<dim3((unsigned)BH), dim3(256), lds, stream>>>(
         static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
         static_cast<E *>(o), dk, dv);

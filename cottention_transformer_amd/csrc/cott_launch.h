@@ -16,6 +16,25 @@ struct ScanArgs {
     hipStream_t stream;
 };
 
+// Kernel families, as reported by cott_profile_read().
+enum KernelId { K_GROUP_STATE = 0, K_STATE_PREFIX, K_SCAN, K_APPLY, K_BWD_DKDV, K_GENERIC, K_DECODE, K_COUNT };
+
+// While profiling is enabled (cott_profile_enable), brackets the launches made in its lifetime
+// with a pair of HIP events on the launch stream; otherwise does nothing.
+class ProfScope {
+  public:
+    ProfScope(int kernel_id, hipStream_t stream);
+    ~ProfScope();
+    ProfScope(const ProfScope &) = delete;
+    ProfScope &operator=(const ProfScope &) = delete;
+
+  private:
+    int id_;
+    hipStream_t stream_;
+    hipEvent_t start_;
+    bool active_;
+};
+
 // Padded state size of the MFMA path (head dims padded to 32, 64 or 128).
 inline int mfma_pad(int d) { return d <= 32 ? 32 : (d <= 64 ? 64 : 128); }
 inline size_t mfma_state_floats(int di, int dj) { return (size_t)mfma_pad(di) * mfma_pad(dj); }

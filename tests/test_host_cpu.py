@@ -1,0 +1,127 @@
+"""CPU-side checks: the oracle reproduces the committed golden fixtures, the C-ABI library loads and
+exports every symbol the header declares, and the host layer rejects what the reference rejects.
+No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from util import load_golden, rel_l2
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- oracle vs golden fixtures -------------------------------------------------------------------
+
+@pytest.mark.parametrize("name", ["causal_cfg1_1x2x128x64.npz", "causal_odd_1x2x63x32_dv48.npz"])
+def test_oracle_reproduces_causal_golden(oracle, name):
+    g = load_golden(name)
+    assert rel_l2(oracle.causal(g["q"], g["k"], g["v"]), g["o"]) < 1e-14
+    assert rel_l2(oracle.causal(g["q"], g["k"], g["v"], True), g["o_rev"]) < 1e-14
+    for got, key in zip(oracle.causal_bwd(g["q"], g["k"], g["v"], g["g"]), ("dq", "dk", "dv")):
+        assert rel_l2(got, g[key]) < 1e-14
+    # the golden outputs are themselves consistent with the O(N^2) form
+    assert rel_l2(oracle.causal_masked(g["q"], g["k"], g["v"]), g["o"]) < 1e-12
+
+
+def test_oracle_reproduces_noncausal_and_decode_golden(oracle):
+    g = load_golden("noncausal_2x2x50x32.npz")
+    assert rel_l2(oracle.noncausal(g["q"], g["k"], g["v"]), g["o"]) < 1e-14
+    for got, key in zip(oracle.noncausal_bwd(g["q"], g["k"], g["v"], g["g"]), ("dq", "dk", "dv")):
+        assert rel_l2(got, g[key]) < 1e-14
+    d = load_golden("decode_2x2x32x48_4steps.npz")
+    state = d["s0"].astype(np.float64).copy()
+    for t in range(d["q"].shape[0]):
+        assert rel_l2(oracle.decode_step(state, d["q"][t], d["k"][t], d["v"][t]), d["o"][t]) < 1e-14
+    assert rel_l2(state, d["s_final"]) < 1e-14
+
+
+# ---- the C ABI -------------------------------------------------------------------------------------
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "cottention.h")).read()
+    return sorted(set(re.findall(r"COTT_API[^;(]*?\b(cott_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from cottention_transformer_amd import _loader
+    names = _declared_symbols()
+    assert {"cott_causal_fwd", "cott_causal_bwd", "cott_noncausal_fwd", "cott_noncausal_bwd", "cott_decode_step",
+            "cott_last_error", "cott_version"} <= set(names)
+    lib = _loader.lib()                     # builds with hipcc if no shared object is present
+    raw = ctypes.CDLL(_loader.lib_path())
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in include/cottention.h but not exported"
+    assert set(names) == set(_loader.SIGNATURES), "ctypes signatures out of step with the header"
+    assert lib.cott_version() >= 100
+
+
+def test_workspace_queries_are_pure_host_functions():
+    from cottention_transformer_amd import _loader
+    L = _loader.lib()
+    # headline shape, bf16: a few groups per head, 64x64 fp32 state per group
+    ws = L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.BF16)
+    assert ws > 0 and ws % (128 * 64 * 64 * 4) == 0
+    # one chunk -> one group -> no workspace; fp32 takes the generic path -> none either
+    assert L.cott_causal_workspace_bytes(64, 16, 64, 64, 64, _loader.BF16) == 0
+    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 0
+    assert L.cott_causal_bwd_workspace_bytes(8, 16, 2048, 64, 64, _loader.BF16) >= ws
+    assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.BF16) > 0
+
+
+def test_c_abi_argument_errors_without_a_gpu():
+    from cottention_transformer_amd import _loader
+    L = _loader.lib()
+    # D_attn % 16 and D_attn >= 32: combined_kernel_general.cu:372-374
+    assert L.cott_causal_fwd(16, 16, 16, 16, 1, 1, 8, 24, 32, _loader.F32, 0, None, 0, None) == _loader.ERR_INVALID
+    assert "divisible by 16" in _loader.last_error()
+    assert L.cott_causal_fwd(16, 16, 16, 16, 1, 1, 8, 16, 32, _loader.F32, 0, None, 0, None) == _loader.ERR_INVALID
+    assert "16*2" in _loader.last_error()
+    assert L.cott_causal_fwd(16, 16, 16, 16, 1, 1, 8, 64, 64, 9, 0, None, 0, None) == _loader.ERR_INVALID
+    assert L.cott_causal_fwd(None, 16, 16, 16, 1, 1, 8, 64, 64, _loader.F32, 0, None, 0, None) == _loader.ERR_INVALID
+    assert L.cott_causal_fwd(8, 16, 16, 16, 1, 1, 8, 64, 64, _loader.F32, 0, None, 0, None) == _loader.ERR_INVALID
+    assert "aligned" in _loader.last_error()
+    # missing workspace on the grouped MFMA path
+    assert L.cott_causal_fwd(16, 16, 16, 16, 1, 1, 4096, 64, 64, _loader.BF16, 0, None, 0, None) == _loader.ERR_WORKSPACE
+    # empty problems are a no-op
+    assert L.cott_causal_fwd(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, 0, None, 0, None) == _loader.OK
+    assert L.cott_decode_step(16, 16, 16, 16, 16, 1, 1, 32, 30, _loader.F32, None) == _loader.ERR_UNSUPPORTED
+
+
+# ---- host layer mirrors the reference's checks ----------------------------------------------------
+
+def test_host_rejects_cpu_tensors_like_the_reference():
+    import cottention_transformer_amd as ct
+    q = torch.randn(1, 2, 8, 32)
+    with pytest.raises(RuntimeError, match="Q must be a CUDA tensor"):   # combined_kernel_general.cu:355
+        ct.causal_dot_product(q, q, q)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        ct.decode_step(torch.zeros(1, 2, 32, 32), q[:, :, 0], q[:, :, 0], q[:, :, 0])
+
+
+def test_dropin_module_names_resolve():
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "cottention_transformer_amd", "Cuda_Kernel"))
+    try:
+        import Custom_Kernel
+        import FastAttention
+        import FastAttention2
+        from FastAttention2 import kernel
+    finally:
+        sys.path.pop(0)
+    for name in ("float32", "float64", "float16", "bfloat16"):
+        assert callable(getattr(kernel, name))
+        assert callable(getattr(FastAttention.forward, name)) and callable(getattr(FastAttention.backward, name))
+    for name in ("forward_float32", "forward_float16", "forward_bfloat16", "backward_float32", "backward_float16",
+                 "backward_bfloat16"):                                            # Cuda_Kernel/pybind.cpp:10-27
+        assert callable(getattr(FastAttention, name))
+    assert issubclass(Custom_Kernel.CustomAttention, torch.autograd.Function)
+    assert FastAttention2.kernel is kernel
+    q = torch.randn(1, 2, 8, 32)
+    with pytest.raises(RuntimeError, match="Q must be a CUDA tensor"):
+        kernel.float32(q, q, q, 1, False, False)
+    with pytest.raises(ValueError):                                               # Custom_Kernel.py:31-32
+        Custom_Kernel.CustomAttention.apply(q.to(torch.int32), q, q)
