@@ -27,6 +27,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary configs (non-causal, decode, long)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
 
 
@@ -87,6 +90,13 @@ def main():
     B, H, N, D = 8, 16, 2048, 64
     q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
 
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     def step():
         o = ct.causal_dot_product(q, k, v)
         grads = ct.causal_backward(q, k, v, do)
@@ -114,7 +124,8 @@ def main():
     esz = 2
     tensor_bytes = B * H * N * D * esz
     # algorithmic bytes of ONE launch of each kernel family at this shape (tensor passes x 32 MiB)
-    passes = {"scan": 4, "bwd_dkdv": 6, "group_state": 2}
+    # scan (forward launch): read Q,K,V + write O; scan_grad (one launch for dQ,dK,dV): read Q,K,V,dO + write 3
+    passes = {"scan": 4, "scan_grad": 7, "group_state": 2}
     alg_bytes = passes.get(dominant, 4) * tensor_bytes
     achieved = alg_bytes / (kern[dominant]["avg_us"] * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -29,7 +29,7 @@ SIGNATURES = {
     "cott_kernel_name": (ctypes.c_char_p, [_i]),
 }
 
-KERNEL_IDS = {"group_state": 0, "state_prefix": 1, "scan": 2, "apply": 3, "bwd_dkdv": 4, "generic": 5, "decode": 6}
+KERNEL_IDS = {"group_state": 0, "state_prefix": 1, "scan": 2, "apply": 3, "scan_grad": 4, "generic": 5, "decode": 6}
 
 
 def profile_enable(on):
@@ -46,6 +46,10 @@ def profile_read(kernel):
 
 
 def lib_path():
+    """In-tree shared object; COTT_LIBRARY points at another build of the same ABI."""
+    override = os.environ.get("COTT_LIBRARY")
+    if override:
+        return override
     from . import build as _build
     return _build.LIB_PATH
 

@@ -66,34 +66,76 @@ size_t elem_size(int dtype) {
     return 0;
 }
 
-// Workgroups the chunked scan aims for: a few per CU of a 256-CU part.  COTT_TARGET_WGS overrides.
-int target_workgroups() {
-    static const int v = [] {
-        const char *s = getenv("COTT_TARGET_WGS");
-        const int x = s ? atoi(s) : 0;
-        return x > 0 ? x : 768;
-    }();
-    return v;
+int env_int(const char *name, int dflt) {
+    const char *s = getenv(name);
+    if (!s || !*s) return dflt;
+    return atoi(s);
 }
 
-struct Plan {
-    int nchunks, cpg, G;
-};
-
-Plan make_plan(long BH, int N) {
-    Plan p;
-    p.nchunks = (N + 63) / 64;
-    long want = (target_workgroups() + BH - 1) / BH;
-    if (want < 1) want = 1;
-    if (want > p.nchunks) want = p.nchunks;
-    p.cpg = (int)((p.nchunks + want - 1) / want);
-    p.G = (p.nchunks + p.cpg - 1) / p.cpg;
-    return p;
+// Workgroups a launch aims for: one per CU of a 256-CU part.  COTT_TARGET_WGS overrides.
+int target_workgroups() {
+    static const int v = [] { const int x = env_int("COTT_TARGET_WGS", 0); return x > 0 ? x : 256; }();
+    return v;
+}
+// COTT_SPLIT: -1 auto (default), 0 never, 1 always split the output columns of each op in two.
+int split_policy() {
+    static const int v = env_int("COTT_SPLIT", -1);
+    return v;
 }
 
 bool use_mfma(int dtype, int di, int dj) {
     return (dtype == COTT_F16 || dtype == COTT_BF16) && di % 16 == 0 && dj % 16 == 0 && di >= 32 && dj >= 32 &&
            di <= 128 && dj <= 128;
+}
+
+// One full-tensor generic op out = G(A,B,C).
+struct Op {
+    const void *A, *B, *C;
+    void *O;
+    int di, dj, reversed;
+};
+
+// How a set of `nops` ops with the same padded head dims is laid on the chip.
+struct SetPlan {
+    int halves;           // 1, or 2 = every op split into two column halves (two problems)
+    int nchunks, cpg, G;  // sequence cut: chunks of 64, chunks per group, groups per head
+    size_t ws_bytes;      // group-state slots
+};
+
+SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal) {
+    SetPlan p;
+    const long tgt = target_workgroups();
+    const bool can_split = dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
+    const int pol = split_policy();
+    p.halves = (can_split && (pol == 1 || (pol < 0 && BH * nops < tgt))) ? 2 : 1;
+    p.nchunks = (N + 63) / 64;
+    long want = (tgt + BH * nops * p.halves - 1) / (BH * nops * p.halves);
+    if (want < 1) want = 1;
+    if (want > p.nchunks) want = p.nchunks;
+    p.cpg = (int)((p.nchunks + want - 1) / want);
+    p.G = (p.nchunks + p.cpg - 1) / p.cpg;
+    const size_t state = cott::mfma_state_floats(di, dj / p.halves) * sizeof(float);
+    p.ws_bytes = (p.G > 1 || !causal) ? (size_t)nops * p.halves * BH * p.G * state : 0;
+    return p;
+}
+
+int pad_key(const Op &o) { return cott::mfma_pad(o.di) * 1000 + cott::mfma_pad(o.dj); }
+
+// Workspace needed by run_ops for the same arguments.
+size_t ops_workspace(const Op *ops, int n, long BH, int N, int dtype, bool causal) {
+    if (BH <= 0 || N <= 0) return 0;
+    for (int i = 0; i < n; ++i)
+        if (!use_mfma(dtype, ops[i].di, ops[i].dj)) return 0;
+    size_t total = 0;
+    bool done[8] = {false};
+    for (int i = 0; i < n; ++i) {
+        if (done[i]) continue;
+        int cnt = 0;
+        for (int j = i; j < n; ++j)
+            if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; ++cnt; }
+        total += plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal).ws_bytes;
+    }
+    return total;
 }
 
 // Shape rules shared by every (B,H,N,D) entry point.  `di` is the contracted head dim of the
@@ -106,55 +148,79 @@ int check_common(const char *fn, int B, int H, int N, int di, int dj, int dtype)
     if (dj < 1) return fail(COTT_ERR_INVALID, "%s: D_value must be positive (got %d)", fn, dj);
     if ((long)B * H > (1L << 22)) return fail(COTT_ERR_UNSUPPORTED, "%s: B*H = %ld exceeds 2^22", fn, (long)B * H);
     const long dmax = di > dj ? di : dj;
-    if ((long)N * dmax >= (1L << 31)) return fail(COTT_ERR_UNSUPPORTED, "%s: N*D = %ld exceeds 2^31", fn, (long)N * dmax);
+    if ((long)N * dmax > (1L << 30)) return fail(COTT_ERR_UNSUPPORTED, "%s: N*D = %ld exceeds 2^30", fn, (long)N * dmax);
     return COTT_OK;
 }
 
-size_t ws_bytes_for(long BH, int N, int di, int dj, int dtype) {
-    if (BH <= 0 || N <= 0 || !use_mfma(dtype, di, dj)) return 0;
-    const Plan p = make_plan(BH, N);
-    if (p.G <= 1) return 0;
-    return (size_t)BH * p.G * cott::mfma_state_floats(di, dj) * sizeof(float);
-}
-
-// out = G(A, B, C) on the best available kernel family.
-int run_op(const char *fn, bool causal, const void *A, const void *B, const void *C, void *O, long BH, int N, int di,
-           int dj, int dtype, int reversed, void *ws, size_t ws_bytes, hipStream_t stream) {
-    cott::ScanArgs a;
-    a.A = A; a.B = B; a.C = C; a.O = O;
-    a.BH = (int)BH; a.N = N; a.di = di; a.dj = dj;
-    a.reversed = reversed ? 1 : 0;
-    a.stream = stream;
-    a.ws = nullptr;
-    a.nchunks = a.cpg = a.G = 1;
-    hipError_t e;
-    if (use_mfma(dtype, di, dj)) {
-        const Plan p = make_plan(BH, N);
-        a.nchunks = p.nchunks; a.cpg = p.cpg; a.G = p.G;
-        const size_t need = (size_t)BH * p.G * cott::mfma_state_floats(di, dj) * sizeof(float);
-        if (p.G > 1 || !causal) {
-            if (ws == nullptr || ws_bytes < need || !aligned16(ws))
-                return fail(COTT_ERR_WORKSPACE, "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", fn, need,
-                            ws ? ws_bytes : (size_t)0);
-            a.ws = static_cast<float *>(ws);
+// Runs n generic ops (n <= 3) over the same (BH, N) on the best available kernel family.
+int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, int dtype, void *ws, size_t ws_bytes,
+            hipStream_t stream) {
+    bool mfma = true;
+    for (int i = 0; i < n; ++i) mfma = mfma && use_mfma(dtype, ops[i].di, ops[i].dj);
+    const size_t esz = elem_size(dtype);
+    if (!mfma) {
+        for (int i = 0; i < n; ++i) {
+            if (!cott::generic_fits(dtype, ops[i].di))
+                return fail(COTT_ERR_UNSUPPORTED, "%s: head dim %d too large for dtype %d on this build", fn, ops[i].di,
+                            dtype);
+            cott::OpDesc d{ops[i].A, ops[i].B, ops[i].C, ops[i].O, ops[i].di, ops[i].dj, ops[i].dj, ops[i].reversed};
+            hipError_t e = cott::launch_generic(dtype, causal, d, (int)BH, N, stream);
+            if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
         }
+        return COTT_OK;
+    }
+    const size_t need = ops_workspace(ops, n, BH, N, dtype, causal);
+    if (need > 0 && (ws == nullptr || ws_bytes < need || !aligned16(ws)))
+        return fail(COTT_ERR_WORKSPACE, "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", fn, need,
+                    ws ? ws_bytes : (size_t)0);
+    char *ws_cursor = static_cast<char *>(ws);
+    bool done[8] = {false};
+    for (int i = 0; i < n; ++i) {
+        if (done[i]) continue;
+        cott::SetArgs a;
+        a.count = 0;
+        int members[8], cnt = 0;
+        for (int j = i; j < n; ++j)
+            if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; members[cnt++] = j; }
+        const SetPlan p = plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal);
+        for (int c = 0; c < cnt; ++c) {
+            const Op &o = ops[members[c]];
+            const int djh = o.dj / p.halves;
+            for (int h = 0; h < p.halves; ++h) {
+                cott::OpDesc &d = a.op[a.count++];
+                d.A = o.A;
+                d.B = o.B;
+                d.C = static_cast<const char *>(o.C) + (size_t)h * djh * esz;
+                d.O = static_cast<char *>(o.O) + (size_t)h * djh * esz;
+                d.di = o.di;
+                d.dj = djh;
+                d.ldc = o.dj;
+                d.reversed = o.reversed;
+            }
+        }
+        a.ws = p.ws_bytes ? reinterpret_cast<float *>(ws_cursor) : nullptr;
+        ws_cursor += p.ws_bytes;
+        a.BH = (int)BH; a.N = N;
+        a.nchunks = p.nchunks; a.cpg = p.cpg; a.G = p.G;
+        a.scan_prof_id = n > 1 ? cott::K_SCAN_GRAD : cott::K_SCAN;
+        a.stream = stream;
+        hipError_t e;
         if (dtype == COTT_BF16)
             e = causal ? cott::launch_causal_mfma_bf16(a) : cott::launch_noncausal_mfma_bf16(a);
         else
             e = causal ? cott::launch_causal_mfma_fp16(a) : cott::launch_noncausal_mfma_fp16(a);
-    } else {
-        if (!cott::generic_fits(dtype, di))
-            return fail(COTT_ERR_UNSUPPORTED, "%s: head dim %d too large for dtype %d on this build", fn, di, dtype);
-        e = cott::launch_generic(dtype, causal, a);
+        if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
     }
-    if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
     return COTT_OK;
 }
 
-size_t noncausal_ws_bytes(long BH, int N, int di, int dj, int dtype) {
-    if (BH <= 0 || N <= 0 || !use_mfma(dtype, di, dj)) return 0;
-    const Plan p = make_plan(BH, N);
-    return (size_t)BH * p.G * cott::mfma_state_floats(di, dj) * sizeof(float);
+// The three gradients as generic ops with permuted operands (Cuda_Kernel/Custom_Kernel.py:106-108;
+// for the non-causal form dq = d_o (v^T k), dk = v (d_o^T q), dv = k (q^T d_o), nothing reversed).
+void grad_ops(Op *ops, const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv, int Dk,
+              int Dv, bool causal) {
+    ops[0] = Op{d_o, v, k, dq, Dv, Dk, 0};
+    ops[1] = Op{v, d_o, q, dk, Dv, Dk, causal ? 1 : 0};
+    ops[2] = Op{k, q, d_o, dv, Dk, Dv, causal ? 1 : 0};
 }
 
 }  // namespace
@@ -197,7 +263,7 @@ int cott_profile_read(int kernel_id, double *total_ms, long *launches) {
 
 const char *cott_kernel_name(int kernel_id) {
     static const char *names[cott::K_COUNT] = {"group_state_kernel", "state_prefix_kernel", "scan_kernel<causal>",
-                                               "scan_kernel<apply>", "bwd_dkdv_kernel",     "generic_scan_kernel",
+                                               "scan_kernel<apply>", "scan_kernel<causal> (dQ,dK,dV set)", "generic_scan_kernel",
                                                "decode_kernel"};
     return (kernel_id >= 0 && kernel_id < cott::K_COUNT) ? names[kernel_id] : "";
 }
@@ -205,7 +271,8 @@ const char *cott_kernel_name(int kernel_id) {
 const char *cott_last_error(void) { return g_err; }
 
 size_t cott_causal_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype) {
-    return ws_bytes_for((long)B * H, N, Dk, Dv, dtype);
+    const Op op{nullptr, nullptr, nullptr, nullptr, Dk, Dv, 0};
+    return ops_workspace(&op, 1, (long)B * H, N, dtype, true);
 }
 
 int cott_causal_fwd(const void *q, const void *k, const void *v, void *o, int B, int H, int N, int Dk, int Dv,
@@ -216,14 +283,14 @@ int cott_causal_fwd(const void *q, const void *k, const void *v, void *o, int B,
     if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
-    return run_op(fn, true, q, k, v, o, (long)B * H, N, Dk, Dv, dtype, reversed, workspace, workspace_bytes,
-                  static_cast<hipStream_t>(stream));
+    const Op op{q, k, v, o, Dk, Dv, reversed ? 1 : 0};
+    return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 size_t cott_causal_bwd_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype) {
-    const size_t a = ws_bytes_for((long)B * H, N, Dv, Dk, dtype);  // dQ, dK: contract over Dv
-    const size_t b = ws_bytes_for((long)B * H, N, Dk, Dv, dtype);  // dV: contract over Dk
-    return a > b ? a : b;
+    Op ops[3];
+    grad_ops(ops, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, Dk, Dv, true);
+    return ops_workspace(ops, 3, (long)B * H, N, dtype, true);
 }
 
 int cott_causal_bwd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
@@ -237,18 +304,18 @@ int cott_causal_bwd(const void *q, const void *k, const void *v, const void *d_o
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
         !aligned16(dv))
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const long BH = (long)B * H;
-    // Operand permutations of Cuda_Kernel/Custom_Kernel.py:106-108.
-    if (int rc = run_op(fn, true, d_o, v, k, dq, BH, N, Dv, Dk, dtype, 0, workspace, workspace_bytes, s)) return rc;
-    if (int rc = run_op(fn, true, v, d_o, q, dk, BH, N, Dv, Dk, dtype, 1, workspace, workspace_bytes, s)) return rc;
-    return run_op(fn, true, k, q, d_o, dv, BH, N, Dk, Dv, dtype, 1, workspace, workspace_bytes, s);
+    Op ops[3];
+    grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
+    return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 size_t cott_noncausal_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype) {
-    const size_t a = noncausal_ws_bytes((long)B * H, N, Dv, Dk, dtype);
-    const size_t b = noncausal_ws_bytes((long)B * H, N, Dk, Dv, dtype);
-    return a > b ? a : b;
+    Op ops[3];
+    grad_ops(ops, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, Dk, Dv, false);
+    const size_t bwd = ops_workspace(ops, 3, (long)B * H, N, dtype, false);
+    const Op op{nullptr, nullptr, nullptr, nullptr, Dk, Dv, 0};
+    const size_t fwd = ops_workspace(&op, 1, (long)B * H, N, dtype, false);
+    return fwd > bwd ? fwd : bwd;
 }
 
 int cott_noncausal_fwd(const void *q, const void *k, const void *v, void *o, int B, int H, int N, int Dk, int Dv,
@@ -259,8 +326,8 @@ int cott_noncausal_fwd(const void *q, const void *k, const void *v, void *o, int
     if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
-    return run_op(fn, false, q, k, v, o, (long)B * H, N, Dk, Dv, dtype, 0, workspace, workspace_bytes,
-                  static_cast<hipStream_t>(stream));
+    const Op op{q, k, v, o, Dk, Dv, 0};
+    return run_ops(fn, false, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int cott_noncausal_bwd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
@@ -274,12 +341,9 @@ int cott_noncausal_bwd(const void *q, const void *k, const void *v, const void *
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
         !aligned16(dv))
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const long BH = (long)B * H;
-    // dq = d_o (v^T k) ; dk = v (d_o^T q) ; dv = k (q^T d_o)
-    if (int rc = run_op(fn, false, d_o, v, k, dq, BH, N, Dv, Dk, dtype, 0, workspace, workspace_bytes, s)) return rc;
-    if (int rc = run_op(fn, false, v, d_o, q, dk, BH, N, Dv, Dk, dtype, 0, workspace, workspace_bytes, s)) return rc;
-    return run_op(fn, false, k, q, d_o, dv, BH, N, Dk, Dv, dtype, 0, workspace, workspace_bytes, s);
+    Op ops[3];
+    grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, false);
+    return run_ops(fn, false, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int cott_decode_step(void *state, const void *q, const void *k, const void *v, void *o, int B, int H, int Dk, int Dv,

@@ -75,4 +75,19 @@ __device__ __forceinline__ u32x4 ld_global16(const u16 *p, bool ok) {
     return ok ? *reinterpret_cast<const u32x4 *>(p) : z;
 }
 
+// Raw buffer descriptor over `bytes` bytes at p.  Buffer loads past the end return zero and buffer
+// stores past the end are dropped by the hardware range check, so tile loads and stores need no
+// branches (which keeps the compiler's outstanding-load counting exact in pipelined loops).
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(rsrc_t r, uint32_t byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_store8(rsrc_t r, uint32_t byte_off, u32x2 v) {
+    __builtin_amdgcn_raw_buffer_store_b64(v, r, (int)byte_off, 0, 0);
+}
+constexpr uint32_t kOobOffset = 0x80000000u;  // beyond any descriptor this library builds
+
 }  // namespace cott

@@ -32,7 +32,7 @@ bool pick_tiling(int di, size_t acc_size, GenericTiling *out) {
 size_t acc_size_of(int dtype) { return dtype == COTT_F64 ? sizeof(double) : sizeof(float); }
 
 template <class ST, bool CAUSAL>
-hipError_t run_generic(const ScanArgs &a) {
+hipError_t run_generic(const OpDesc &a, int BH, int N, hipStream_t stream) {
     GenericTiling t;
     if (!pick_tiling(a.di, sizeof(typename ST::acc), &t)) return hipErrorInvalidValue;
     auto kern = generic_scan_kernel<ST, CAUSAL>;
@@ -43,10 +43,10 @@ hipError_t run_generic(const ScanArgs &a) {
     }
     const int nslices = (a.dj + t.DJT - 1) / t.DJT;
     typedef typename ST::elem E;
-    ProfScope ps(K_GENERIC, a.stream);
-    kern<<<dim3((unsigned)(a.BH * nslices)), dim3(256), t.bytes, a.stream>>>(
+    ProfScope ps(K_GENERIC, stream);
+    kern<<<dim3((unsigned)(BH * nslices)), dim3(256), t.bytes, stream>>>(
         static_cast<const E *>(a.A), static_cast<const E *>(a.B), static_cast<const E *>(a.C), static_cast<E *>(a.O),
-        a.N, a.di, a.dj, t.CH, t.DJT, nslices, a.reversed);
+        N, a.di, a.dj, t.CH, t.DJT, nslices, a.reversed);
     return hipGetLastError();
 }
 
@@ -69,12 +69,12 @@ bool generic_fits(int dtype, int di) {
     return pick_tiling(di, acc_size_of(dtype), &t);
 }
 
-hipError_t launch_generic(int dtype, bool causal, const ScanArgs &a) {
+hipError_t launch_generic(int dtype, bool causal, const OpDesc &a, int BH, int N, hipStream_t stream) {
     switch (dtype) {
-        case COTT_F32: return causal ? run_generic<StF32, true>(a) : run_generic<StF32, false>(a);
-        case COTT_F64: return causal ? run_generic<StF64, true>(a) : run_generic<StF64, false>(a);
-        case COTT_F16: return causal ? run_generic<StFp16, true>(a) : run_generic<StFp16, false>(a);
-        case COTT_BF16: return causal ? run_generic<StBf16, true>(a) : run_generic<StBf16, false>(a);
+        case COTT_F32: return causal ? run_generic<StF32, true>(a, BH, N, stream) : run_generic<StF32, false>(a, BH, N, stream);
+        case COTT_F64: return causal ? run_generic<StF64, true>(a, BH, N, stream) : run_generic<StF64, false>(a, BH, N, stream);
+        case COTT_F16: return causal ? run_generic<StFp16, true>(a, BH, N, stream) : run_generic<StFp16, false>(a, BH, N, stream);
+        case COTT_BF16: return causal ? run_generic<StBf16, true>(a, BH, N, stream) : run_generic<StBf16, false>(a, BH, N, stream);
     }
     return hipErrorInvalidValue;
 }

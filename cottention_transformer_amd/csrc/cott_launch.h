@@ -5,19 +5,27 @@
 
 namespace cott {
 
-// One generic op  out = G(A, B, C)  over BH independent heads.
-struct ScanArgs {
-    const void *A, *B, *C;  // A,B: (BH,N,di)  C: (BH,N,dj)
-    void *O;                // (BH,N,dj)
-    float *ws;              // per-group state slots, BH*G*state_floats(di,dj) floats (MFMA path, G>1)
-    int BH, N, di, dj;
-    int reversed;
-    int nchunks, cpg, G;    // MFMA path: chunks of 64, chunks per group, groups per head
+// One generic op  out = G(A, B, C)  over BH independent heads; C and O may be a column slice
+// (dj columns out of rows of ldc elements, pointers already offset to the first column).
+struct OpDesc {
+    const void *A, *B, *C;  // A,B: (BH,N,di)  C: (BH,N,ldc)
+    void *O;                // (BH,N,ldc)
+    int di, dj, ldc, reversed;
+};
+
+// A set of ops launched together over the same (BH, N); MFMA path: all share padded head dims.
+struct SetArgs {
+    OpDesc op[6];
+    int count;
+    float *ws;            // count * BH * G * state_floats floats when G > 1 or non-causal, else unused
+    int BH, N;
+    int nchunks, cpg, G;  // chunks of 64, chunks per group, groups per head
+    int scan_prof_id;     // K_SCAN for a forward launch, K_SCAN_GRAD for the three-gradient launch
     hipStream_t stream;
 };
 
 // Kernel families, as reported by cott_profile_read().
-enum KernelId { K_GROUP_STATE = 0, K_STATE_PREFIX, K_SCAN, K_APPLY, K_BWD_DKDV, K_GENERIC, K_DECODE, K_COUNT };
+enum KernelId { K_GROUP_STATE = 0, K_STATE_PREFIX, K_SCAN, K_APPLY, K_SCAN_GRAD, K_GENERIC, K_DECODE, K_COUNT };
 
 // While profiling is enabled (cott_profile_enable), brackets the launches made in its lifetime
 // with a pair of HIP events on the launch stream; otherwise does nothing.
@@ -39,14 +47,15 @@ class ProfScope {
 inline int mfma_pad(int d) { return d <= 32 ? 32 : (d <= 64 ? 64 : 128); }
 inline size_t mfma_state_floats(int di, int dj) { return (size_t)mfma_pad(di) * mfma_pad(dj); }
 
-// dtype is COTT_F16 or COTT_BF16; 32 <= di,dj <= 128, multiples of 16.
-hipError_t launch_causal_mfma_bf16(const ScanArgs &a);
-hipError_t launch_causal_mfma_fp16(const ScanArgs &a);
-hipError_t launch_noncausal_mfma_bf16(const ScanArgs &a);
-hipError_t launch_noncausal_mfma_fp16(const ScanArgs &a);
+// 16-bit storage; every op: 32 <= di,dj <= 128, multiples of 16, same padded dims across the set.
+hipError_t launch_causal_mfma_bf16(const SetArgs &a);
+hipError_t launch_causal_mfma_fp16(const SetArgs &a);
+hipError_t launch_noncausal_mfma_bf16(const SetArgs &a);
+hipError_t launch_noncausal_mfma_fp16(const SetArgs &a);
 
-// Plain-FMA fallback for any dtype / head dim.  Returns hipErrorInvalidValue if no tiling fits LDS.
-hipError_t launch_generic(int dtype, bool causal, const ScanArgs &a);
+// Plain-FMA fallback for any dtype / head dim, one op (full tensors: ldc == dj).
+// Returns hipErrorInvalidValue if no tiling fits LDS.
+hipError_t launch_generic(int dtype, bool causal, const OpDesc &op, int BH, int N, hipStream_t stream);
 bool generic_fits(int dtype, int di);
 
 hipError_t launch_decode(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH,

@@ -3,11 +3,16 @@
 // Generic op (per batch*head):  out[s,j] = sum_i A[s,i] * sum_{s' <= s (>= s if reversed)} B[s',i] C[s',j]
 // restructured over chunks of 64 positions (scan order p, state S[i][j] carried in fp32):
 //     out_c = ((A_c B_c^T) o mask) C_c + A_c S_c ;   S_{c+1} = S_c + B_c^T C_c
-// The sequence of one head is cut into G groups of consecutive chunks so that B*H*G workgroups
-// fill the chip: group_state_kernel sums B^T C over each group, state_prefix_kernel turns the
-// per-group sums into exclusive prefixes, scan_kernel runs the chunk recurrence seeded with its
-// group's prefix.  The same three kernels serve the forward pass and, with permuted operands,
-// every gradient (dQ = G(dO,V,K), dK = G(V,dO,Q,rev), dV = G(K,Q,dO,rev)).
+//
+// One launch runs a SET of such problems over the same (BH, N) grid -- the two column halves of a
+// forward pass, or the three gradients dQ = G(dO,V,K), dK = G(V,dO,Q,rev), dV = G(K,Q,dO,rev).  The
+// workgroups that work on the same head are placed on the same XCD and start together, so an
+// operand shared between problems (Q and K of the two halves; Q, K, V, dO of the gradients) comes
+// from HBM once and from that XCD's L2 afterwards.
+//
+// When B*H alone cannot fill the chip the sequence of one head is also cut into G groups of
+// consecutive chunks: group_state_kernel sums B^T C over each group, state_prefix_kernel turns the
+// per-group sums into exclusive prefixes, scan_kernel runs the recurrence seeded with its prefix.
 #pragma once
 #include "cott_common.h"
 
@@ -15,6 +20,23 @@ namespace cott {
 
 constexpr int kChunk = 64;     // positions per chunk
 constexpr int kThreads = 256;  // 4 wavefronts per workgroup
+constexpr int kMaxProblems = 6;
+constexpr int kXcds = 8;       // workgroup i is dispatched to XCD i % 8
+
+// One generic op.  A, B: rows of `di` elements, contiguous.  C, O: `dj` columns taken from rows of
+// `ldc` elements (the pointers already include the first column), so a problem can own a column
+// slice of a wider tensor.  gstate: G slots of DI*DJ floats per head (G > 1 or non-causal).
+struct Problem {
+    const u16 *A, *B, *C;
+    u16 *O;
+    float *gstate;
+    int di, dj, ldc, reversed;
+};
+
+struct ProblemSet {
+    Problem p[kMaxProblems];
+    int count;
+};
 
 template <int DI, int DJ>
 struct Tiling {
@@ -29,104 +51,160 @@ struct Tiling {
     static constexpr int STATE_FLOATS = DI * DJ;
 };
 
-// [64][D] tile, global -> registers.  Thread t owns 16-byte vectors t, t+256, ...; rows past N
-// and columns past the runtime width d read as zero, so padded positions add nothing to a state.
+// Workgroup -> (head, problem, group).  Linear id i runs on XCD i % 8; per XCD the ids are ordered
+// (head block, group, problem), so the workgroups of one head and group are neighbours in the
+// dispatch order of ONE XCD.
+struct WorkItem {
+    int bh, prob, grp;
+};
+__device__ __forceinline__ WorkItem decode_workgroup(int nprob, int G) {
+    const int i = blockIdx.x;
+    const int xcd = i % kXcds;
+    int slot = i / kXcds;
+    WorkItem wi;
+    wi.prob = slot % nprob;
+    slot /= nprob;
+    wi.grp = slot % G;
+    wi.bh = (slot / G) * kXcds + xcd;
+    return wi;
+}
+inline unsigned grid_for(int BH, int nprob, int G) {
+    return (unsigned)(((BH + kXcds - 1) / kXcds) * kXcds * nprob * G);
+}
+
+// [64][D] tile, global -> registers, through a buffer descriptor of the head.  Thread t owns 16-byte
+// vectors t, t+256, ...; rows past N read as zero (hardware range check).  Pure loads, no use of the
+// result here, so nothing waits on them until the tile is staged.
 template <int D>
-__device__ __forceinline__ void load_tile(u32x4 (&r)[D / 32], const u16 *head, int row0, int N, int d, int tid) {
+__device__ __forceinline__ void load_tile(u32x4 *r, rsrc_t rs, int row0, int ld, int tid) {
 #pragma unroll
     for (int u = 0; u < D / 32; ++u) {
         const int v = tid + kThreads * u;
         const int row = row0 + v / (D / 8);
         const int col = (v % (D / 8)) * 8;
-        r[u] = ld_global16(head + (size_t)row * d + col, row < N && col < d);
+        r[u] = buf_load16(rs, (uint32_t)(row * ld + col) * 2u);
     }
 }
 
+// registers -> LDS tile [64][D+8]; columns past the runtime width d are zeroed here, so padded
+// positions add nothing to a product or a state.
 template <int D>
-__device__ __forceinline__ void store_tile(u16 *tile, const u32x4 (&r)[D / 32], int tid) {
+__device__ __forceinline__ void store_tile(u16 *tile, const u32x4 *r, int d, int tid) {
 #pragma unroll
     for (int u = 0; u < D / 32; ++u) {
         const int v = tid + kThreads * u;
-        *reinterpret_cast<u32x4 *>(tile + (v / (D / 8)) * (D + 8) + (v % (D / 8)) * 8) = r[u];
+        const int col = (v % (D / 8)) * 8;
+        *reinterpret_cast<u32x4 *>(tile + (v / (D / 8)) * (D + 8) + col) = (col < d) ? r[u] : u32x4{0u, 0u, 0u, 0u};
     }
 }
 
 // S[i][j] += sum_{tok<64} B[tok][i] * C[tok][j] for the tiles this wavefront owns
 // (tile index t = w*TPW + u -> (t / NJT, t % NJT)).  Both operands are column fragments of the
-// row-major LDS tiles, fetched with transposing reads.
+// row-major LDS tiles, fetched with transposing reads; all fragments of a 32-token step are read
+// before its MFMAs so the LDS latency is paid once per step, not once per tile.
 template <class TR, int DI, int DJ>
-__device__ __forceinline__ void state_update(f32x4 *S, const u16 *sB, const u16 *sC,
-                                             int w, int g, int m) {
+__device__ __forceinline__ void state_update(f32x4 *S, const u16 *sB, const u16 *sC, int w, int g, int m) {
     using TL = Tiling<DI, DJ>;
+    constexpr int ROWS = (TL::TPW + TL::NJT - 1) / TL::NJT;       // tile rows (values of `it`) per wavefront
+    constexpr int COLS = TL::TPW < TL::NJT ? TL::TPW : TL::NJT;   // distinct `jt` per wavefront
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
         const int k0 = 32 * kb + 8 * g;
-        u32x4 a;
+        u32x4 a[ROWS], b[COLS];
 #pragma unroll
-        for (int u = 0; u < TL::TPW; ++u) {
-            const int t = w * TL::TPW + u;
-            const int it = t / TL::NJT, jt = t % TL::NJT;
-            if (u % TL::NJT == 0) a = cat(lds_col4(sB, TL::BS, k0, 16 * it, m), lds_col4(sB, TL::BS, k0 + 4, 16 * it, m));
-            const u32x4 b = cat(lds_col4(sC, TL::CS, k0, 16 * jt, m), lds_col4(sC, TL::CS, k0 + 4, 16 * jt, m));
-            S[u] = TR::mfma(a, b, S[u]);
+        for (int r = 0; r < ROWS; ++r) {
+            const int it = (w * TL::TPW + r * TL::NJT) / TL::NJT;
+            a[r] = cat(lds_col4(sB, TL::BS, k0, 16 * it, m), lds_col4(sB, TL::BS, k0 + 4, 16 * it, m));
         }
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            const int jt = (w * TL::TPW + c) % TL::NJT;
+            b[c] = cat(lds_col4(sC, TL::CS, k0, 16 * jt, m), lds_col4(sC, TL::CS, k0 + 4, 16 * jt, m));
+        }
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) S[u] = TR::mfma(a[u / TL::NJT], b[u % COLS], S[u]);
     }
 }
 
+// Pipeline shared by both kernels: global loads run PF chunks ahead in PF register stages (static
+// indices: the chunk loop is unrolled by PF), the LDS tiles are double-buffered so that chunk p+1
+// is staged while chunk p is consumed, and ONE barrier separates consecutive chunks.  Every load
+// and store in the loop is unconditional (prefetch past the end of the group re-reads its last
+// chunk), which lets the compiler wait on exactly the stage it needs.
+
 // Sum of B^T C over each group of chunks, written in register-native order:
-// float4 index (w*TPW + u)*64 + lane of slot (bh*G + grp).
-template <class TR, int DI, int DJ>
-__global__ __launch_bounds__(kThreads) void group_state_kernel(const u16 *__restrict__ B, const u16 *__restrict__ C,
-                                                               float *__restrict__ gstate, int N, int di, int dj,
-                                                               int nchunks, int cpg, int G, int ngroups,
-                                                               int reversed) {
+// float4 index (w*TPW + u)*64 + lane of slot (bh*G + grp).  `ngroups` of the G groups are launched
+// (the causal scan never needs the last group's sum).
+template <class TR, int DI, int DJ, int PF>
+__global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg,
+                                                               int G, int ngroups) {
     using TL = Tiling<DI, DJ>;
-    __shared__ __attribute__((aligned(16))) u16 sB[kChunk * TL::BS];
-    __shared__ __attribute__((aligned(16))) u16 sC[kChunk * TL::CS];
-    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, m = l & 15;
-    const int grp = blockIdx.x % ngroups, bh = blockIdx.x / ngroups;  // G slots per head, `ngroups` launched
-    B += (size_t)bh * N * di;
-    C += (size_t)bh * N * dj;
-    const int p0 = grp * cpg;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS;
+    __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
+    __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
+    const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const WorkItem wi = decode_workgroup(set.count, ngroups);
+    if (wi.bh >= BH) return;
+    const Problem &pr = set.p[wi.prob];
+    const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
+    const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
+    const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const int p0 = wi.grp * cpg;
     const int p1 = min(p0 + cpg, nchunks);
 
     f32x4 S[TL::TPW];
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    u32x4 rb[DI / 32], rc[DJ / 32];
-    {
-        const int c = reversed ? nchunks - 1 - p0 : p0;
-        load_tile<DI>(rb, B, c * kChunk, N, di, tid);
-        load_tile<DJ>(rc, C, c * kChunk, N, dj, tid);
-    }
-    for (int p = p0; p < p1; ++p) {
-        __syncthreads();
-        store_tile<DI>(sB, rb, tid);
-        store_tile<DJ>(sC, rc, tid);
-        __syncthreads();
-        if (p + 1 < p1) {
-            const int c = reversed ? nchunks - 2 - p : p + 1;
-            load_tile<DI>(rb, B, c * kChunk, N, di, tid);
-            load_tile<DJ>(rc, C, c * kChunk, N, dj, tid);
-        }
-        state_update<TR, DI, DJ>(S, sB, sC, w, g, m);
-    }
-    f32x4 *out = reinterpret_cast<f32x4 *>(gstate + ((size_t)bh * G + grp) * TL::STATE_FLOATS);
+    u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
+    auto load_chunk = [&](int s, int p) {
+        const int pc = min(p, p1 - 1);
+        const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
+        load_tile<DI>(rb[s], rB, row0, di, tid);
+        load_tile<DJ>(rc[s], rC, row0, ldc, tid);
+    };
+    auto finish = [&]() {
+        f32x4 *out = reinterpret_cast<f32x4 *>(pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS);
 #pragma unroll
-    for (int u = 0; u < TL::TPW; ++u) out[(w * TL::TPW + u) * 64 + l] = S[u];
+        for (int u = 0; u < TL::TPW; ++u) out[(w * TL::TPW + u) * 64 + l] = S[u];
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
+    store_tile<DI>(sB, rb[0], di, tid);
+    store_tile<DJ>(sC, rc[0], dj, tid);
+    load_chunk(0, p0 + PF);
+    __syncthreads();
+    for (int pb = p0;; pb += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int p = pb + s;
+            if (p >= p1) {
+                finish();
+                return;
+            }
+            const int s1 = (s + 1) % PF;
+            const int buf = (p - p0) & 1;
+            store_tile<DI>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+            store_tile<DJ>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+            load_chunk(s1, p + 1 + PF);
+            state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+            __syncthreads();
+        }
+    }
 }
 
 // Over the G slots of one head, element-wise: mode 0 -> exclusive prefix in place (slot g gets the
 // sum of slots < g; only the first `ncomputed` slots hold data), mode 1 -> total into slot 0.
-static __global__ __launch_bounds__(kThreads) void state_prefix_kernel(float *__restrict__ gstate, int G, int ncomputed,
-                                                                int state_floats, int mode) {
+static __global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSet set, int BH, int G, int ncomputed,
+                                                                       int state_floats, int mode) {
     const int sf4 = state_floats / 4;
-    const int blocks_per_head = (sf4 + kThreads - 1) / kThreads;
-    const int bh = blockIdx.x / blocks_per_head;
-    const int e = (blockIdx.x % blocks_per_head) * kThreads + threadIdx.x;
-    if (e >= sf4) return;
-    f32x4 *p = reinterpret_cast<f32x4 *>(gstate + (size_t)bh * G * state_floats) + e;
+    const int blocks_per_state = (sf4 + kThreads - 1) / kThreads;
+    const int e = (blockIdx.x % blocks_per_state) * kThreads + threadIdx.x;
+    const int rest = blockIdx.x / blocks_per_state;
+    const int prob = rest % set.count, bh = rest / set.count;
+    if (e >= sf4 || bh >= BH) return;
+    f32x4 *p = reinterpret_cast<f32x4 *>(set.p[prob].gstate + (size_t)bh * G * state_floats) + e;
     f32x4 run = {0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < G; ++s) {
         f32x4 t = {0.f, 0.f, 0.f, 0.f};
@@ -137,132 +215,167 @@ static __global__ __launch_bounds__(kThreads) void state_prefix_kernel(float *__
     if (mode == 1) p[0] = run;
 }
 
-// The chunk recurrence for one group of one head.  CAUSAL=false is the non-causal apply pass:
-// out = A * S_total with the state taken from slot 0 and never updated.
+// The chunk recurrence for one group of one head of one problem.  CAUSAL=false is the non-causal
+// apply pass: out = A * S_total with the state taken from slot 0 and never updated.
 //
 // Work split (4 wavefronts, chunk of 64): wavefront w owns output positions 16w..16w+15 of the
 // chunk.  It forms P^T = B_c A_w^T tile by tile (so the accumulator layout IS the operand layout
 // of the next product -- the masked scores never leave registers), then
-// out_w^T = C_c^T P^T + S^T A_w^T, stored as 8-byte row segments.
-template <class TR, int DI, int DJ, bool CAUSAL>
-__global__ __launch_bounds__(kThreads) void scan_kernel(const u16 *__restrict__ A, const u16 *__restrict__ B,
-                                                        const u16 *__restrict__ C, u16 *__restrict__ O,
-                                                        const float *__restrict__ gstate, int N, int di, int dj,
-                                                        int nchunks, int cpg, int G, int reversed) {
+// out_w^T = C_c^T P^T + S^T A_w^T, stored as 8-byte row segments.  The body is straight-line code:
+// score tiles above the diagonal are computed and zeroed rather than skipped.
+template <class TR, int DI, int DJ, bool CAUSAL, int PF>
+__global__ __launch_bounds__(kThreads) void scan_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G) {
     using TL = Tiling<DI, DJ>;
-    __shared__ __attribute__((aligned(16))) u16 sB[CAUSAL ? kChunk * TL::BS : 8];
-    __shared__ __attribute__((aligned(16))) u16 sC[CAUSAL ? kChunk * TL::CS : 8];
-    __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
-    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, m = l & 15;
-    const int grp = blockIdx.x % G, bh = blockIdx.x / G;
-    A += (size_t)bh * N * di;
-    B += (size_t)bh * N * di;
-    C += (size_t)bh * N * dj;
-    O += (size_t)bh * N * dj;
-    const int p0 = grp * cpg;
+    constexpr int SB = CAUSAL ? kChunk * TL::BS : 8, SC = CAUSAL ? kChunk * TL::CS : 8, SSZ = DJ * TL::SS;
+    __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
+    __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
+    __shared__ __attribute__((aligned(16))) u16 sS[(CAUSAL ? 2 : 1) * SSZ];
+    const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const WorkItem wi = decode_workgroup(set.count, G);
+    if (wi.bh >= BH) return;
+    const Problem &pr = set.p[wi.prob];
+    const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
+    const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
+    const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
+    const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const int p0 = wi.grp * cpg;
     const int p1 = min(p0 + cpg, nchunks);
 
     f32x4 S[TL::TPW];
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (gstate != nullptr) {
-        const f32x4 *gs =
-            reinterpret_cast<const f32x4 *>(gstate + ((size_t)bh * G + (CAUSAL ? grp : 0)) * TL::STATE_FLOATS);
+    if (pr.gstate != nullptr) {
+        const f32x4 *gs = reinterpret_cast<const f32x4 *>(pr.gstate + ((size_t)wi.bh * G + (CAUSAL ? wi.grp : 0)) *
+                                                                         TL::STATE_FLOATS);
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
     }
 
-    u32x4 rb[DI / 32], rc[DJ / 32], qn[TL::KS], qc[TL::KS];
-    auto load_chunk = [&](int p) {
-        const int row0 = (reversed ? nchunks - 1 - p : p) * kChunk;
+    u32x4 rb[PF][CAUSAL ? DI / 32 : 1], rc[PF][CAUSAL ? DJ / 32 : 1], qn[PF][TL::KS], qc[TL::KS], qx[TL::KS];
+    auto load_chunk = [&](int s, int p) {
+        const int pc = min(p, p1 - 1);
+        const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
         if (CAUSAL) {
-            load_tile<DI>(rb, B, row0, N, di, tid);
-            load_tile<DJ>(rc, C, row0, N, dj, tid);
+            load_tile<DI>(rb[s], rB, row0, di, tid);
+            load_tile<DJ>(rc[s], rC, row0, ldc, tid);
         }
         const int row = row0 + 16 * w + m;
 #pragma unroll
         for (int ks = 0; ks < TL::KS; ++ks) {
             const int col = 32 * ks + 8 * g;
-            qn[ks] = ld_global16(A + (size_t)row * di + col, row < N && col < di);
+            qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + col) * 2u);
         }
     };
-    load_chunk(p0);
-
-    for (int p = p0; p < p1; ++p) {
-        const int row0 = (reversed ? nchunks - 1 - p : p) * kChunk;
-        __syncthreads();  // every wavefront is done reading the previous chunk's tiles
-        if (CAUSAL) {
-            store_tile<DI>(sB, rb, tid);
-            store_tile<DJ>(sC, rc, tid);
-        }
-        if (CAUSAL || p == p0) {
-            // 16-bit copy of the state BEFORE this chunk, transposed to [j][i] for the A_w S product
+    // 16-bit copy of the state, transposed to [j][i] for the A_w S product
+    auto put_state = [&](u16 *dst) {
 #pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) {
-                const int t = w * TL::TPW + u;
-                const int it = t / TL::NJT, jt = t % TL::NJT;
-                u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
-                *reinterpret_cast<u32x2 *>(sS + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
+        for (int u = 0; u < TL::TPW; ++u) {
+            const int t = w * TL::TPW + u;
+            const int it = t / TL::NJT, jt = t % TL::NJT;
+            u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
+            *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
+        }
+    };
+
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
+    if (CAUSAL) {
+        store_tile<DI>(sB, rb[0], di, tid);
+        store_tile<DJ>(sC, rc[0], dj, tid);
+    }
+    put_state(sS);
+#pragma unroll
+    for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[0][ks] : u32x4{0u, 0u, 0u, 0u};
+    load_chunk(0, p0 + PF);
+    __syncthreads();
+
+    for (int pb = p0;; pb += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int p = pb + s;
+            if (p >= p1) return;  // uniform over the workgroup; nothing follows the loop
+            const int s1 = (s + 1) % PF;
+            const int buf = CAUSAL ? ((p - p0) & 1) : 0;
+            const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
+            const int row0 = (reversed ? nchunks - 1 - p : p) * kChunk;
+
+            // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
+            if (CAUSAL) {
+                store_tile<DI>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+                store_tile<DJ>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
             }
-        }
 #pragma unroll
-        for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = qn[ks];
-        __syncthreads();
-        if (p + 1 < p1) load_chunk(p + 1);  // prefetch: lands while this chunk is computed
+            for (int ks = 0; ks < TL::KS; ++ks) qx[ks] = (32 * ks + 8 * g < di) ? qn[s1][ks] : u32x4{0u, 0u, 0u, 0u};
+            load_chunk(s1, p + 1 + PF);
 
-        // masked scores, transposed: pk[jt] = P^T[16jt+4g .. +3][16w+m]
-        u32x2 pk[4];
-        if (CAUSAL) {
+            const int orow = row0 + 16 * w + m;
+            // masked scores, transposed: pk[jt] = P^T[16jt+4g .. +3][16w+m].  Fragment reads first,
+            // MFMAs after, so LDS latency overlaps with the matrix pipe instead of alternating with it.
+            u32x2 pk[4];
+            if (CAUSAL) {
+                u32x4 kf[4][TL::KS];
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
-                pk[jt] = u32x2{0u, 0u};
-                const bool active = reversed ? (jt >= w) : (jt <= w);
-                if (active) {
+                for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        kf[jt][ks] = *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
                     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int ks = 0; ks < TL::KS; ++ks) {
-                        const u32x4 a = *reinterpret_cast<const u32x4 *>(sB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
-                        acc = TR::mfma(a, qc[ks], acc);
-                    }
-                    if (jt == w) {
+                    for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ks], acc);
+                    const int d0 = 16 * (jt - w) + 4 * g - m;  // key position minus query position, r = 0
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const bool keep = reversed ? (4 * g + r >= m) : (4 * g + r <= m);
-                            acc[r] = keep ? acc[r] : 0.f;
-                        }
+                    for (int r = 0; r < 4; ++r) {
+                        const bool keep = reversed ? (d0 + r >= 0) : (d0 + r <= 0);
+                        acc[r] = keep ? acc[r] : 0.f;
                     }
                     pk[jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
                 }
             }
-        }
 
-        const int orow = row0 + 16 * w + m;
+            constexpr int JB = (8 / TL::KS < TL::NJT) ? (8 / TL::KS) : TL::NJT;  // output tiles per read batch
 #pragma unroll
-        for (int jt = 0; jt < TL::NJT; ++jt) {
-            f32x4 o = {0.f, 0.f, 0.f, 0.f};
-            if (CAUSAL) {
+            for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
+                u32x4 vf[JB][2], sf[JB][TL::KS];
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    const bool active = reversed ? (2 * kb + 1 >= w) : (2 * kb <= w);
-                    if (active) {
-                        const u32x4 a = cat(lds_col4(sC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
-                                            lds_col4(sC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
-                        o = TR::mfma(a, cat(pk[2 * kb], pk[2 * kb + 1]), o);
+                for (int jj = 0; jj < JB; ++jj) {
+                    const int jt = j0 + jj;
+                    if (CAUSAL) {
+#pragma unroll
+                        for (int kb = 0; kb < 2; ++kb)
+                            vf[jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
+                                             lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
                     }
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        sf[jj][ks] = *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
+                }
+#pragma unroll
+                for (int jj = 0; jj < JB; ++jj) {
+                    const int jt = j0 + jj;
+                    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+                    if (CAUSAL) {
+#pragma unroll
+                        for (int kb = 0; kb < 2; ++kb) o = TR::mfma(vf[jj][kb], cat(pk[2 * kb], pk[2 * kb + 1]), o);
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ks], o);
+                    const int col = 16 * jt + 4 * g;
+                    const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
+                    buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
                 }
             }
+            if (CAUSAL) {
+                state_update<TR, DI, DJ>(S, cB, cC, w, g, m);
+                put_state(sS + (buf ^ 1) * SSZ);
+            }
 #pragma unroll
-            for (int ks = 0; ks < TL::KS; ++ks) {
-                const u32x4 a = *reinterpret_cast<const u32x4 *>(sS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
-                o = TR::mfma(a, qc[ks], o);
-            }
-            const int col = 16 * jt + 4 * g;
-            if (orow < N && col < dj) {
-                u32x2 v = {TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
-                *reinterpret_cast<u32x2 *>(O + (size_t)orow * dj + col) = v;
-            }
+            for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = qx[ks];
+            if (CAUSAL) __syncthreads();
         }
-        if (CAUSAL) state_update<TR, DI, DJ>(S, sB, sC, w, g, m);
     }
 }
 

@@ -1,6 +1,6 @@
 // bf16 instantiations of the MFMA chunked-scan kernels.
 #include "cott_mfma_launch.inc"
 namespace cott {
-hipError_t launch_causal_mfma_bf16(const ScanArgs &a) { return dispatch<Bf16, true>(a); }
-hipError_t launch_noncausal_mfma_bf16(const ScanArgs &a) { return dispatch<Bf16, false>(a); }
+hipError_t launch_causal_mfma_bf16(const SetArgs &a) { return dispatch<Bf16, true>(a); }
+hipError_t launch_noncausal_mfma_bf16(const SetArgs &a) { return dispatch<Bf16, false>(a); }
 }  // namespace cott

@@ -96,8 +96,9 @@ COTT_API int cott_decode_step(void *state, const void *q, const void *k, const v
  * While enabled, every kernel launch made by the entry points above is bracketed by a pair of HIP
  * events on the launch stream (this is the one place the library creates HIP objects).
  * cott_profile_read() waits for the recorded launches of one kernel family, returns their summed
- * duration and count, and forgets them.  Kernel ids: 0 group_state, 1 state_prefix, 2 causal scan,
- * 3 non-causal apply, 4 fused dK/dV, 5 generic scan, 6 decode.  Stands where the reference wraps
+ * duration and count, and forgets them.  Kernel ids: 0 group_state, 1 state_prefix, 2 causal scan
+ * (forward launch), 3 non-causal apply, 4 causal scan (the launch that computes dQ, dK and dV together),
+ * 5 generic scan, 6 decode.  Stands where the reference wraps
  * its kernel call in torch.autograd.profiler (Cuda_Kernel/Custom_Kernel.py:165-179). */
 COTT_API int cott_profile_enable(int on);
 COTT_API int cott_profile_read(int kernel_id, double *total_ms, long *launches);

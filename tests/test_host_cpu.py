@@ -62,13 +62,15 @@ def test_library_exports_every_declared_symbol():
 def test_workspace_queries_are_pure_host_functions():
     from cottention_transformer_amd import _loader
     L = _loader.lib()
-    # headline shape, bf16: a few groups per head, 64x64 fp32 state per group
-    ws = L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.BF16)
-    assert ws > 0 and ws % (128 * 64 * 64 * 4) == 0
-    # one chunk -> one group -> no workspace; fp32 takes the generic path -> none either
-    assert L.cott_causal_workspace_bytes(64, 16, 64, 64, 64, _loader.BF16) == 0
-    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 0
-    assert L.cott_causal_bwd_workspace_bytes(8, 16, 2048, 64, 64, _loader.BF16) >= ws
+    # few heads, long sequence: the sequence is cut into groups, each with an fp32 state slot per problem
+    ws = L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.BF16)
+    assert ws > 0 and ws % (64 * 32 * 4) == 0
+    # headline shape: B*H (x2 column halves) already fills the chip -> one group -> no workspace
+    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.BF16) == 0
+    # fp32 takes the generic path -> none either
+    assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F32) == 0
+    assert L.cott_causal_bwd_workspace_bytes(1, 2, 8192, 64, 64, _loader.BF16) >= ws
+    # the non-causal form always stages K^T V through the workspace
     assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.BF16) > 0
 
 
