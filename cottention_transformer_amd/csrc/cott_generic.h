@@ -121,14 +121,16 @@ __global__ __launch_bounds__(256) void generic_scan_kernel(const typename ST::el
 
 // Decode step: one workgroup per (batch, head) streams its [dk][dv] state once.
 //   S[i][j] += k[i] v[j] ;  o[j] = sum_i q[i] S[i][j]
-// Thread t owns a 4-wide column strip (t % nvb) and every rg-th row starting at t / nvb; rows
-// are processed 8 at a time with all loads issued before the first store.
+// Thread t owns a 4-wide column strip (t % nvb) and every rg-th row starting at t / nvb.  Rows are
+// processed 16 at a time; the state loads of a pass are issued before anything else (q and k are
+// staged through LDS while they are in flight) and every load precedes the first store.
 template <class ST, class SF /* state scalar: float or double */>
 __global__ __launch_bounds__(256) void decode_kernel(SF *__restrict__ S, const typename ST::elem *__restrict__ q,
                                                      const typename ST::elem *__restrict__ k,
                                                      const typename ST::elem *__restrict__ v,
                                                      typename ST::elem *__restrict__ o, int dk, int dv) {
     typedef SF __attribute__((ext_vector_type(4))) sf4;
+    constexpr int U = 16;
     extern __shared__ __attribute__((aligned(32))) unsigned char smem_raw[];
     SF *sq = reinterpret_cast<SF *>(smem_raw);  // [dk]
     SF *sk = sq + dk;                           // [dk]
@@ -139,41 +141,45 @@ __global__ __launch_bounds__(256) void decode_kernel(SF *__restrict__ S, const t
     k += (size_t)bh * dk;
     v += (size_t)bh * dv;
     o += (size_t)bh * dv;
-    for (int i = tid; i < dk; i += 256) {
-        sq[i] = (SF)ST::load(q + i);
-        sk[i] = (SF)ST::load(k + i);
-    }
-    __syncthreads();
     const int nv = dv / 4;
     const int nvb = nv < 256 ? nv : 256;
     const int rg = 256 / nvb;
     const int mc = tid % nvb, mr = tid / nvb;
+    bool staged = false;
     for (int c0 = 0; c0 < nv; c0 += nvb) {
         const int c4 = c0 + mc;
         const bool live = (mr < rg) && (c4 < nv);
         sf4 acc = {0, 0, 0, 0};
-        if (live) {
-            sf4 vv;
-            vv.x = (SF)ST::load(v + 4 * c4);
-            vv.y = (SF)ST::load(v + 4 * c4 + 1);
-            vv.z = (SF)ST::load(v + 4 * c4 + 2);
-            vv.w = (SF)ST::load(v + 4 * c4 + 3);
-            sf4 *col = reinterpret_cast<sf4 *>(S) + c4;
-            for (int r0 = mr; r0 < dk; r0 += 8 * rg) {
-                sf4 s[8];
+        sf4 vv = {0, 0, 0, 0};
+        sf4 *col = reinterpret_cast<sf4 *>(S) + (live ? c4 : 0);
+        for (int r0 = mr; r0 < dk || !staged; r0 += U * rg) {
+            sf4 s[U];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int r = r0 + u * rg;
-                    if (r < dk) s[u] = __builtin_nontemporal_load(col + (size_t)r * nv);
+            for (int u = 0; u < U; ++u) {
+                const int r = r0 + u * rg;
+                if (live && r < dk) s[u] = col[(size_t)r * nv];
+            }
+            if (!staged) {  // first pass of the workgroup: q, k -> LDS while the state is in flight
+                for (int i = tid; i < dk; i += 256) {
+                    sq[i] = (SF)ST::load(q + i);
+                    sk[i] = (SF)ST::load(k + i);
                 }
+                __syncthreads();
+                staged = true;
+            }
+            if (live && r0 == mr) {
+                vv.x = (SF)ST::load(v + 4 * c4);
+                vv.y = (SF)ST::load(v + 4 * c4 + 1);
+                vv.z = (SF)ST::load(v + 4 * c4 + 2);
+                vv.w = (SF)ST::load(v + 4 * c4 + 3);
+            }
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int r = r0 + u * rg;
-                    if (r < dk) {
-                        s[u] += sk[r] * vv;
-                        __builtin_nontemporal_store(s[u], col + (size_t)r * nv);
-                        acc += sq[r] * s[u];
-                    }
+            for (int u = 0; u < U; ++u) {
+                const int r = r0 + u * rg;
+                if (live && r < dk) {
+                    s[u] += sk[r] * vv;
+                    col[(size_t)r * nv] = s[u];
+                    acc += sq[r] * s[u];
                 }
             }
         }
@@ -188,6 +194,83 @@ __global__ __launch_bounds__(256) void decode_kernel(SF *__restrict__ S, const t
             ST::store(o + 4 * c4 + 2, (typename ST::acc)t.z);
             ST::store(o + 4 * c4 + 3, (typename ST::acc)t.w);
         }
+    }
+}
+
+// Decode step, one WAVEFRONT per (batch, head): no workgroup barrier anywhere, so the four heads of
+// a workgroup stream independently.  For dv/4 = nv in {8,16,32,64} columns of float4: lane l owns
+// column l % nv and every (64/nv)-th row starting at l / nv; q and k are staged in a per-wavefront
+// LDS slice while the first batch of state loads is in flight; the row groups are combined with
+// lane-xor shuffles.  Plain (cacheable) loads and stores: a state that fits the last-level cache is
+// then served from it on the next step.
+template <class ST, class SF>
+__global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, const typename ST::elem *__restrict__ q,
+                                                          const typename ST::elem *__restrict__ k,
+                                                          const typename ST::elem *__restrict__ v,
+                                                          typename ST::elem *__restrict__ o, int BH, int dk, int dv) {
+    typedef SF __attribute__((ext_vector_type(4))) sf4;
+    constexpr int U = 16;
+    extern __shared__ __attribute__((aligned(32))) unsigned char smem_raw[];
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int bh = blockIdx.x * 4 + wv;
+    if (bh >= BH) return;
+    SF *sq = reinterpret_cast<SF *>(smem_raw) + (size_t)wv * 2 * dk;  // this wavefront's [q | k]
+    SF *sk = sq + dk;
+    S += (size_t)bh * dk * dv;
+    q += (size_t)bh * dk;
+    k += (size_t)bh * dk;
+    v += (size_t)bh * dv;
+    o += (size_t)bh * dv;
+    const int nv = dv / 4;       // 8, 16, 32 or 64
+    const int rpw = 64 / nv;     // rows covered by one wavefront-wide load
+    const int mc = lane % nv, mr = lane / nv;
+    sf4 *col = reinterpret_cast<sf4 *>(S) + mc;
+    sf4 acc = {0, 0, 0, 0};
+    sf4 vv = {0, 0, 0, 0};
+    bool staged = false;
+    for (int r0 = mr; r0 < dk; r0 += U * rpw) {
+        sf4 s[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int r = r0 + u * rpw;
+            if (r < dk) s[u] = col[(size_t)r * nv];
+        }
+        if (!staged) {
+            for (int i = lane; i < dk; i += 64) {
+                sq[i] = (SF)ST::load(q + i);
+                sk[i] = (SF)ST::load(k + i);
+            }
+            vv.x = (SF)ST::load(v + 4 * mc);
+            vv.y = (SF)ST::load(v + 4 * mc + 1);
+            vv.z = (SF)ST::load(v + 4 * mc + 2);
+            vv.w = (SF)ST::load(v + 4 * mc + 3);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            staged = true;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int r = r0 + u * rpw;
+            if (r < dk) {
+                s[u] += sk[r] * vv;
+                col[(size_t)r * nv] = s[u];
+                acc += sq[r] * s[u];
+            }
+        }
+    }
+    for (int off = nv; off < 64; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off);
+        acc.y += __shfl_xor(acc.y, off);
+        acc.z += __shfl_xor(acc.z, off);
+        acc.w += __shfl_xor(acc.w, off);
+    }
+    if (mr == 0) {
+        ST::store(o + 4 * mc, (typename ST::acc)acc.x);
+        ST::store(o + 4 * mc + 1, (typename ST::acc)acc.y);
+        ST::store(o + 4 * mc + 2, (typename ST::acc)acc.z);
+        ST::store(o + 4 * mc + 3, (typename ST::acc)acc.w);
     }
 }
 

@@ -54,8 +54,17 @@ template <class ST, class SF>
 hipError_t run_decode(void *state, const void *q, const void *k, const void *v, void *o, int BH, int dk, int dv,
                       hipStream_t stream) {
     typedef typename ST::elem E;
-    const size_t lds = (size_t)2 * dk * sizeof(SF) + 256 * 4 * sizeof(SF);
     ProfScope ps(K_DECODE, stream);
+    const int nv = dv / 4;
+    if ((nv == 8 || nv == 16 || nv == 32 || nv == 64) && dk <= 1024) {
+        // one wavefront per head, four heads per workgroup
+        const size_t lds_w = (size_t)4 * 2 * dk * sizeof(SF);
+        decode_wave_kernel<ST, SF><<<dim3((unsigned)((BH + 3) / 4)), dim3(256), lds_w, stream>>>(
+            static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
+            static_cast<E *>(o), BH, dk, dv);
+        return hipGetLastError();
+    }
+    const size_t lds = (size_t)2 * dk * sizeof(SF) + 256 * 4 * sizeof(SF);
     decode_kernel<ST, SF><<<dim3((unsigned)BH), dim3(256), lds, stream>>>(
         static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
         static_cast<E *>(o), dk, dv);
