@@ -19,6 +19,12 @@ import time
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
+# HBM-side bytes per launch at the headline shape, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
+# `bench.py --calibration-copy` (counters scaled by their reading for the 256 MiB copy in the same run).
+# A counter run cannot be made from inside this script; the figures and commands are in
+# profiles/scan_kernel_headline_hbm_traffic_pmc.txt.
+MEASURED_TRAFFIC_BYTES = {"scan": 128.10 * 2**20, "scan_grad": 312.78 * 2**20}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -129,7 +135,7 @@ def main():
     alg_bytes = passes.get(dominant, 4) * tensor_bytes
     achieved = alg_bytes / (kern[dominant]["avg_us"] * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
                 "kernel": dominant, "avg_us": kern[dominant]["avg_us"],
                 "algorithmic_bytes_per_launch": alg_bytes,
                 "whole_step": {"algorithmic_bytes": 11 * tensor_bytes,
