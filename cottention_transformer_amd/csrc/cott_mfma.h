@@ -41,8 +41,12 @@ struct ProblemSet {
 template <int DI, int DJ>
 struct Tiling {
     static_assert(DI % 32 == 0 && DJ % 32 == 0, "padded head dims are multiples of 32");
-    static constexpr int BS = DI + 8;            // LDS row stride (elements) of a [64][DI] tile
-    static constexpr int CS = DJ + 8;            // ... of a [64][DJ] tile
+    // LDS row strides (elements).  The paddings were chosen by measuring SQ_LDS_BANK_CONFLICT: 16/16/8 had
+    // the fewest conflict cycles of the combinations tried.
+    static constexpr int BS = DI + 16;           // [64][DI] tile: b128 row reads and transposing reads
+    // ... of a [64][DJ] tile.  This tile is only read with transposing reads, which touch 4 consecutive
+    // rows x 8 dwords per quarter-wave: a row stride of 8 (mod 32) dwords keeps them on distinct banks.
+    static constexpr int CS = DJ + 16;
     static constexpr int SS = DI + 8;            // ... of the transposed 16-bit state [DJ][DI]
     static constexpr int NIT = DI / 16;          // 16-wide tiles along i
     static constexpr int NJT = DJ / 16;          // 16-wide tiles along j
@@ -88,13 +92,13 @@ __device__ __forceinline__ void load_tile(u32x4 *r, rsrc_t rs, int row0, int ld,
 
 // registers -> LDS tile [64][D+8]; columns past the runtime width d are zeroed here, so padded
 // positions add nothing to a product or a state.
-template <int D>
+template <int D, int STRIDE>
 __device__ __forceinline__ void store_tile(u16 *tile, const u32x4 *r, int d, int tid) {
 #pragma unroll
     for (int u = 0; u < D / 32; ++u) {
         const int v = tid + kThreads * u;
         const int col = (v % (D / 8)) * 8;
-        *reinterpret_cast<u32x4 *>(tile + (v / (D / 8)) * (D + 8) + col) = (col < d) ? r[u] : u32x4{0u, 0u, 0u, 0u};
+        *reinterpret_cast<u32x4 *>(tile + (v / (D / 8)) * STRIDE + col) = (col < d) ? r[u] : u32x4{0u, 0u, 0u, 0u};
     }
 }
 
@@ -171,8 +175,8 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
-    store_tile<DI>(sB, rb[0], di, tid);
-    store_tile<DJ>(sC, rc[0], dj, tid);
+    store_tile<DI, TL::BS>(sB, rb[0], di, tid);
+    store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
     load_chunk(0, p0 + PF);
     __syncthreads();
     for (int pb = p0;; pb += PF) {
@@ -185,8 +189,8 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
             }
             const int s1 = (s + 1) % PF;
             const int buf = (p - p0) & 1;
-            store_tile<DI>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-            store_tile<DJ>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+            store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+            store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
             load_chunk(s1, p + 1 + PF);
             state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
             __syncthreads();
@@ -215,166 +219,239 @@ static __global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSe
     if (mode == 1) p[0] = run;
 }
 
-// The chunk recurrence for one group of one head of one problem.  CAUSAL=false is the non-causal
-// apply pass: out = A * S_total with the state taken from slot 0 and never updated.
+// The chunk recurrence for one group of one head of one problem.
 //
-// Work split (4 wavefronts, chunk of 64): wavefront w owns output positions 16w..16w+15 of the
-// chunk.  It forms P^T = B_c A_w^T tile by tile (so the accumulator layout IS the operand layout
-// of the next product -- the masked scores never leave registers), then
-// out_w^T = C_c^T P^T + S^T A_w^T, stored as 8-byte row segments.  The body is straight-line code:
-// score tiles above the diagonal are computed and zeroed rather than skipped.
-template <class TR, int DI, int DJ, bool CAUSAL, int PF>
-__global__ __launch_bounds__(kThreads) void scan_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G) {
+// Eight wavefronts in two roles, two per SIMD, so that one role's LDS / VALU / memory latencies are
+// covered by the other role's matrix work:
+//   * "output" wavefronts 0-3: wavefront w owns output positions 16w..16w+15 of the chunk.  It forms
+//     P^T = B_c A_w^T tile by tile (so the accumulator layout IS the operand layout of the next
+//     product -- the masked scores never leave registers), then out_w^T = C_c^T P^T + S^T A_w^T,
+//     stored as 8-byte row segments.  Score tiles above the diagonal are computed and zeroed.
+//   * "state" wavefronts 4-7: move the B and C tiles global -> registers -> LDS (PF chunks ahead),
+//     carry the fp32 state S += B_c^T C_c in their accumulators and publish its 16-bit copy for the
+//     next chunk.
+// One barrier per chunk joins the roles; LDS tiles and the 16-bit state are double-buffered.
+template <class TR, int DI, int DJ, int PF>
+__global__ __launch_bounds__(2 * kThreads) void scan_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg,
+                                                            int G) {
     using TL = Tiling<DI, DJ>;
-    constexpr int SB = CAUSAL ? kChunk * TL::BS : 8, SC = CAUSAL ? kChunk * TL::CS : 8, SSZ = DJ * TL::SS;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
-    __shared__ __attribute__((aligned(16))) u16 sS[(CAUSAL ? 2 : 1) * SSZ];
+    __shared__ __attribute__((aligned(16))) u16 sS[2 * SSZ];
+    const int l = threadIdx.x & 63, g = l >> 4, m = l & 15;
+    const int w8 = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const bool state_role = w8 >= 4;
+    const int w = w8 & 3;              // index within the role
+    const int tid = threadIdx.x & 255; // thread index within the role
+    const WorkItem wi = decode_workgroup(set.count, G);
+    if (wi.bh >= BH) return;
+    const Problem &pr = set.p[wi.prob];
+    const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
+    const int p0 = wi.grp * cpg;
+    const int p1 = min(p0 + cpg, nchunks);
+
+    if (state_role) {
+        const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
+        const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+        f32x4 S[TL::TPW];
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (pr.gstate != nullptr) {
+            const f32x4 *gs =
+                reinterpret_cast<const f32x4 *>(pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS);
+#pragma unroll
+            for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
+        }
+        u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
+        auto load_chunk = [&](int s, int p) {
+            const int pc = min(p, p1 - 1);
+            const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
+            load_tile<DI>(rb[s], rB, row0, di, tid);
+            load_tile<DJ>(rc[s], rC, row0, ldc, tid);
+        };
+        // 16-bit copy of the state, transposed to [j][i] for the A_w S product
+        auto put_state = [&](u16 *dst) {
+#pragma unroll
+            for (int u = 0; u < TL::TPW; ++u) {
+                const int t = w * TL::TPW + u;
+                const int it = t / TL::NJT, jt = t % TL::NJT;
+                u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
+                *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
+            }
+        };
+#pragma unroll
+        for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
+        store_tile<DI, TL::BS>(sB, rb[0], di, tid);
+        store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
+        put_state(sS);
+        load_chunk(0, p0 + PF);
+        __syncthreads();
+        for (int pb = p0;; pb += PF) {
+#pragma unroll
+            for (int s = 0; s < PF; ++s) {
+                const int p = pb + s;
+                if (p >= p1) return;  // uniform over the workgroup; nothing follows the loop
+                const int s1 = (s + 1) % PF;
+                const int buf = (p - p0) & 1;
+                // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
+                store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+                store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+                load_chunk(s1, p + 1 + PF);
+                state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+                put_state(sS + (buf ^ 1) * SSZ);
+                __syncthreads();
+            }
+        }
+    } else {
+        const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
+        const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+        u32x4 qn[PF][TL::KS], qc[TL::KS];
+        auto load_q = [&](int s, int p) {
+            const int pc = min(p, p1 - 1);
+            const int row = (reversed ? nchunks - 1 - pc : pc) * kChunk + 16 * w + m;
+#pragma unroll
+            for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + 32 * ks + 8 * g) * 2u);
+        };
+#pragma unroll
+        for (int s = 0; s < PF; ++s) load_q(s, p0 + s);
+        __syncthreads();
+        for (int pb = p0;; pb += PF) {
+#pragma unroll
+            for (int s = 0; s < PF; ++s) {
+                const int p = pb + s;
+                if (p >= p1) return;
+                const int buf = (p - p0) & 1;
+                const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
+                const int row0 = (reversed ? nchunks - 1 - p : p) * kChunk;
+#pragma unroll
+                for (int ks = 0; ks < TL::KS; ++ks)
+                    qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
+                load_q(s, p + PF);
+
+                // masked scores, transposed: pk[jt] = P^T[16jt+4g .. +3][16w+m]; fragment reads first,
+                // MFMAs after, so the LDS latency is paid once per batch
+                u32x2 pk[4];
+                {
+                    u32x4 kf[4][TL::KS];
+#pragma unroll
+                    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                        for (int ks = 0; ks < TL::KS; ++ks)
+                            kf[jt][ks] =
+                                *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
+#pragma unroll
+                    for (int jt = 0; jt < 4; ++jt) {
+                        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ks], acc);
+                        const int d0 = 16 * (jt - w) + 4 * g - m;  // key position minus query position, r = 0
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const bool keep = reversed ? (d0 + r >= 0) : (d0 + r <= 0);
+                            acc[r] = keep ? acc[r] : 0.f;
+                        }
+                        pk[jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
+                    }
+                }
+
+                const int orow = row0 + 16 * w + m;
+                constexpr int JB = (8 / TL::KS < TL::NJT) ? (8 / TL::KS) : TL::NJT;  // output tiles per read batch
+#pragma unroll
+                for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
+                    u32x4 vf[JB][2], sf[JB][TL::KS];
+#pragma unroll
+                    for (int jj = 0; jj < JB; ++jj) {
+                        const int jt = j0 + jj;
+#pragma unroll
+                        for (int kb = 0; kb < 2; ++kb)
+                            vf[jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
+                                             lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
+#pragma unroll
+                        for (int ks = 0; ks < TL::KS; ++ks)
+                            sf[jj][ks] =
+                                *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
+                    }
+#pragma unroll
+                    for (int jj = 0; jj < JB; ++jj) {
+                        const int jt = j0 + jj;
+                        f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int kb = 0; kb < 2; ++kb) o = TR::mfma(vf[jj][kb], cat(pk[2 * kb], pk[2 * kb + 1]), o);
+#pragma unroll
+                        for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ks], o);
+                        const int col = 16 * jt + 4 * g;
+                        const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
+                        buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+}
+
+// Non-causal apply pass: out = A * S_total for one group of chunks, the state taken from slot 0 of
+// the head and held as 16-bit A-operand tiles in LDS.  Wavefront w owns rows 16w..16w+15 of a chunk.
+template <class TR, int DI, int DJ, int PF>
+__global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G) {
+    using TL = Tiling<DI, DJ>;
+    __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const WorkItem wi = decode_workgroup(set.count, G);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
-    const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
+    const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
     const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-    const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-    const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
     const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
     const int p0 = wi.grp * cpg;
     const int p1 = min(p0 + cpg, nchunks);
-
-    f32x4 S[TL::TPW];
-#pragma unroll
-    for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (pr.gstate != nullptr) {
-        const f32x4 *gs = reinterpret_cast<const f32x4 *>(pr.gstate + ((size_t)wi.bh * G + (CAUSAL ? wi.grp : 0)) *
-                                                                         TL::STATE_FLOATS);
-#pragma unroll
-        for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
-    }
-
-    u32x4 rb[PF][CAUSAL ? DI / 32 : 1], rc[PF][CAUSAL ? DJ / 32 : 1], qn[PF][TL::KS], qc[TL::KS], qx[TL::KS];
-    auto load_chunk = [&](int s, int p) {
-        const int pc = min(p, p1 - 1);
-        const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
-        if (CAUSAL) {
-            load_tile<DI>(rb[s], rB, row0, di, tid);
-            load_tile<DJ>(rc[s], rC, row0, ldc, tid);
-        }
-        const int row = row0 + 16 * w + m;
-#pragma unroll
-        for (int ks = 0; ks < TL::KS; ++ks) {
-            const int col = 32 * ks + 8 * g;
-            qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + col) * 2u);
-        }
-    };
-    // 16-bit copy of the state, transposed to [j][i] for the A_w S product
-    auto put_state = [&](u16 *dst) {
+    {
+        const f32x4 *gs = reinterpret_cast<const f32x4 *>(pr.gstate + (size_t)wi.bh * G * TL::STATE_FLOATS);
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) {
+            const f32x4 sv = gs[(w * TL::TPW + u) * 64 + l];
             const int t = w * TL::TPW + u;
             const int it = t / TL::NJT, jt = t % TL::NJT;
-            u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
-            *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
+            u32x2 pk = {TR::pack2(sv[0], sv[1]), TR::pack2(sv[2], sv[3])};
+            *reinterpret_cast<u32x2 *>(sS + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
         }
-    };
-
-#pragma unroll
-    for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
-    if (CAUSAL) {
-        store_tile<DI>(sB, rb[0], di, tid);
-        store_tile<DJ>(sC, rc[0], dj, tid);
     }
-    put_state(sS);
+    u32x4 qn[PF][TL::KS];
+    auto load_q = [&](int s, int p) {
+        const int row = min(p, p1 - 1) * kChunk + 16 * w + m;
 #pragma unroll
-    for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[0][ks] : u32x4{0u, 0u, 0u, 0u};
-    load_chunk(0, p0 + PF);
+        for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + 32 * ks + 8 * g) * 2u);
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_q(s, p0 + s);
     __syncthreads();
-
+    u32x4 sf[TL::NJT][TL::KS];  // this wavefront reads the whole state once
+#pragma unroll
+    for (int jt = 0; jt < TL::NJT; ++jt)
+#pragma unroll
+        for (int ks = 0; ks < TL::KS; ++ks)
+            sf[jt][ks] = *reinterpret_cast<const u32x4 *>(sS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
     for (int pb = p0;; pb += PF) {
 #pragma unroll
         for (int s = 0; s < PF; ++s) {
             const int p = pb + s;
-            if (p >= p1) return;  // uniform over the workgroup; nothing follows the loop
-            const int s1 = (s + 1) % PF;
-            const int buf = CAUSAL ? ((p - p0) & 1) : 0;
-            const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
-            const int row0 = (reversed ? nchunks - 1 - p : p) * kChunk;
-
-            // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
-            if (CAUSAL) {
-                store_tile<DI>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-                store_tile<DJ>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+            if (p >= p1) return;
+            u32x4 qc[TL::KS];
+#pragma unroll
+            for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
+            load_q(s, p + PF);
+            const int orow = p * kChunk + 16 * w + m;
+#pragma unroll
+            for (int jt = 0; jt < TL::NJT; ++jt) {
+                f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jt][ks], qc[ks], o);
+                const int col = 16 * jt + 4 * g;
+                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
+                buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
             }
-#pragma unroll
-            for (int ks = 0; ks < TL::KS; ++ks) qx[ks] = (32 * ks + 8 * g < di) ? qn[s1][ks] : u32x4{0u, 0u, 0u, 0u};
-            load_chunk(s1, p + 1 + PF);
-
-            const int orow = row0 + 16 * w + m;
-            // masked scores, transposed: pk[jt] = P^T[16jt+4g .. +3][16w+m].  Fragment reads first,
-            // MFMAs after, so LDS latency overlaps with the matrix pipe instead of alternating with it.
-            u32x2 pk[4];
-            if (CAUSAL) {
-                u32x4 kf[4][TL::KS];
-#pragma unroll
-                for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-                    for (int ks = 0; ks < TL::KS; ++ks)
-                        kf[jt][ks] = *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
-#pragma unroll
-                for (int jt = 0; jt < 4; ++jt) {
-                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ks], acc);
-                    const int d0 = 16 * (jt - w) + 4 * g - m;  // key position minus query position, r = 0
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const bool keep = reversed ? (d0 + r >= 0) : (d0 + r <= 0);
-                        acc[r] = keep ? acc[r] : 0.f;
-                    }
-                    pk[jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
-                }
-            }
-
-            constexpr int JB = (8 / TL::KS < TL::NJT) ? (8 / TL::KS) : TL::NJT;  // output tiles per read batch
-#pragma unroll
-            for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
-                u32x4 vf[JB][2], sf[JB][TL::KS];
-#pragma unroll
-                for (int jj = 0; jj < JB; ++jj) {
-                    const int jt = j0 + jj;
-                    if (CAUSAL) {
-#pragma unroll
-                        for (int kb = 0; kb < 2; ++kb)
-                            vf[jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
-                                             lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
-                    }
-#pragma unroll
-                    for (int ks = 0; ks < TL::KS; ++ks)
-                        sf[jj][ks] = *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
-                }
-#pragma unroll
-                for (int jj = 0; jj < JB; ++jj) {
-                    const int jt = j0 + jj;
-                    f32x4 o = {0.f, 0.f, 0.f, 0.f};
-                    if (CAUSAL) {
-#pragma unroll
-                        for (int kb = 0; kb < 2; ++kb) o = TR::mfma(vf[jj][kb], cat(pk[2 * kb], pk[2 * kb + 1]), o);
-                    }
-#pragma unroll
-                    for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ks], o);
-                    const int col = 16 * jt + 4 * g;
-                    const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
-                    buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
-                }
-            }
-            if (CAUSAL) {
-                state_update<TR, DI, DJ>(S, cB, cC, w, g, m);
-                put_state(sS + (buf ^ 1) * SSZ);
-            }
-#pragma unroll
-            for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = qx[ks];
-            if (CAUSAL) __syncthreads();
         }
     }
 }
