@@ -72,7 +72,9 @@ int env_int(const char *name, int dflt) {
     return atoi(s);
 }
 
-// Workgroups a launch aims for: one per CU of a 256-CU part.  COTT_TARGET_WGS overrides.
+// Workgroups a launch aims for: one per CU of a 256-CU part (a second workgroup on a CU adds only ~20 %
+// throughput to these LDS-heavy kernels, so grids just above the CU count run almost twice as long).
+// COTT_TARGET_WGS overrides.
 int target_workgroups() {
     static const int v = [] { const int x = env_int("COTT_TARGET_WGS", 0); return x > 0 ? x : 256; }();
     return v;
@@ -107,12 +109,33 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal) {
     const long tgt = target_workgroups();
     const bool can_split = dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
     const int pol = split_policy();
-    p.halves = (can_split && (pol == 1 || (pol < 0 && BH * nops < tgt))) ? 2 : 1;
     p.nchunks = (N + 63) / 64;
-    long want = (tgt + BH * nops * p.halves - 1) / (BH * nops * p.halves);
-    if (want < 1) want = 1;
-    if (want > p.nchunks) want = p.nchunks;
-    p.cpg = (int)((p.nchunks + want - 1) / want);
+    // Choose (column halves, sequence groups) to fill the target without exceeding it: halves cost
+    // repeated score tiles but no memory traffic, groups cost one extra read of two operands.
+    long best_total = -1;
+    int best_h = 1, best_g = 1;
+    for (int h = 1; h <= 2; ++h) {
+        if (h == 2 && (!can_split || pol == 0)) continue;
+        if (h == 1 && can_split && pol == 1) continue;
+        const long base = BH * nops * h;
+        long g = base >= tgt ? 1 : tgt / base;
+        if (g > p.nchunks) g = p.nchunks;
+        const int cpg = (int)((p.nchunks + g - 1) / g);
+        g = (p.nchunks + cpg - 1) / cpg;
+        const long total = base * g;
+        // prefer the fuller grid; on a tie prefer fewer groups (less re-reading)
+        const bool better = best_total < 0 || (total <= tgt && best_total > tgt) ||
+                            ((total <= tgt) == (best_total <= tgt) &&
+                             ((total <= tgt) ? (total > best_total || (total == best_total && g < best_g))
+                                             : (total < best_total)));
+        if (better) {
+            best_total = total;
+            best_h = h;
+            best_g = (int)g;
+        }
+    }
+    p.halves = best_h;
+    p.cpg = (p.nchunks + best_g - 1) / best_g;
     p.G = (p.nchunks + p.cpg - 1) / p.cpg;
     const size_t state = cott::mfma_state_floats(di, dj / p.halves) * sizeof(float);
     p.ws_bytes = (p.G > 1 || !causal) ? (size_t)nops * p.halves * BH * p.G * state : 0;
