@@ -47,7 +47,7 @@ struct Tiling {
     // ... of a [64][DJ] tile.  This tile is only read with transposing reads, which touch 4 consecutive
     // rows x 8 dwords per quarter-wave: a row stride of 8 (mod 32) dwords keeps them on distinct banks.
     static constexpr int CS = DJ + 16;
-    static constexpr int SS = DI + 8;            // ... of the transposed 16-bit state [DJ][DI]
+    static constexpr int SS = DI + 16;           // ... of the transposed 16-bit state [DJ][DI] (b128 row reads)
     static constexpr int NIT = DI / 16;          // 16-wide tiles along i
     static constexpr int NJT = DJ / 16;          // 16-wide tiles along j
     static constexpr int TPW = NIT * NJT / 4;    // fp32 state tiles owned by one wavefront
@@ -76,14 +76,14 @@ inline unsigned grid_for(int BH, int nprob, int G) {
     return (unsigned)(((BH + kXcds - 1) / kXcds) * kXcds * nprob * G);
 }
 
-// [64][D] tile, global -> registers, through a buffer descriptor of the head.  Thread t owns 16-byte
-// vectors t, t+256, ...; rows past N read as zero (hardware range check).  Pure loads, no use of the
+// [64][D] tile, global -> registers, through a buffer descriptor of the head.  Thread t of NT owns 16-byte
+// vectors t, t+NT, ...; rows past N read as zero (hardware range check).  Pure loads, no use of the
 // result here, so nothing waits on them until the tile is staged.
-template <int D>
+template <int D, int NT = kThreads>
 __device__ __forceinline__ void load_tile(u32x4 *r, rsrc_t rs, int row0, int ld, int tid) {
 #pragma unroll
-    for (int u = 0; u < D / 32; ++u) {
-        const int v = tid + kThreads * u;
+    for (int u = 0; u < 8 * D / NT; ++u) {
+        const int v = tid + NT * u;
         const int row = row0 + v / (D / 8);
         const int col = (v % (D / 8)) * 8;
         r[u] = buf_load16(rs, (uint32_t)(row * ld + col) * 2u);
@@ -92,11 +92,11 @@ __device__ __forceinline__ void load_tile(u32x4 *r, rsrc_t rs, int row0, int ld,
 
 // registers -> LDS tile [64][D+8]; columns past the runtime width d are zeroed here, so padded
 // positions add nothing to a product or a state.
-template <int D, int STRIDE>
+template <int D, int STRIDE, int NT = kThreads>
 __device__ __forceinline__ void store_tile(u16 *tile, const u32x4 *r, int d, int tid) {
 #pragma unroll
-    for (int u = 0; u < D / 32; ++u) {
-        const int v = tid + kThreads * u;
+    for (int u = 0; u < 8 * D / NT; ++u) {
+        const int v = tid + NT * u;
         const int col = (v % (D / 8)) * 8;
         *reinterpret_cast<u32x4 *>(tile + (v / (D / 8)) * STRIDE + col) = (col < d) ? r[u] : u32x4{0u, 0u, 0u, 0u};
     }
@@ -221,29 +221,32 @@ static __global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSe
 
 // The chunk recurrence for one group of one head of one problem.
 //
-// Eight wavefronts in two roles, two per SIMD, so that one role's LDS / VALU / memory latencies are
-// covered by the other role's matrix work:
-//   * "output" wavefronts 0-3: wavefront w owns output positions 16w..16w+15 of the chunk.  It forms
-//     P^T = B_c A_w^T tile by tile (so the accumulator layout IS the operand layout of the next
-//     product -- the masked scores never leave registers), then out_w^T = C_c^T P^T + S^T A_w^T,
-//     stored as 8-byte row segments.  Score tiles above the diagonal are computed and zeroed.
-//   * "state" wavefronts 4-7: move the B and C tiles global -> registers -> LDS (PF chunks ahead),
-//     carry the fp32 state S += B_c^T C_c in their accumulators and publish its 16-bit copy for the
-//     next chunk.
+// Wavefronts in three roles that share the SIMDs, so that each role's LDS / VALU / memory latencies
+// are covered by the other roles' work and no role's per-chunk dependency chain carries the others':
+//   * OW "output" wavefronts (first in the workgroup), each owning 64/OW output positions of the
+//     chunk as IB = 4/OW blocks of 16.  A block's scores are formed transposed, P^T = B_c A_blk^T,
+//     tile by tile, so the accumulator layout IS the operand layout of the next product and the
+//     masked scores never leave registers; then out_blk^T = C_c^T P^T + S^T A_blk^T, stored as 8-byte
+//     row segments.  Score tiles above the diagonal are computed and zeroed.
+//   * four "state" wavefronts carry the fp32 state S += B_c^T C_c in their accumulators and publish
+//     its 16-bit copy for the next chunk.
+//   * LW "loader" wavefronts move the B and C tiles global -> registers -> LDS, PF chunks ahead.
 // One barrier per chunk joins the roles; LDS tiles and the 16-bit state are double-buffered.
-template <class TR, int DI, int DJ, int PF>
-__global__ __launch_bounds__(2 * kThreads) void scan_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg,
-                                                            int G) {
+template <class TR, int DI, int DJ, int PF, int OW, int LW>
+__global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set, int BH, int N, int nchunks,
+                                                                  int cpg, int G) {
     using TL = Tiling<DI, DJ>;
+    static_assert(OW == 2 || OW == 4, "two or four output wavefronts");
+    static_assert(LW == 2 || LW == 4, "two or four loader wavefronts");
+    constexpr int IB = 4 / OW;
+    constexpr int LT = 64 * LW;  // loader threads
+    static_assert((8 * DI) % LT == 0 && (8 * DJ) % LT == 0, "tile vectors divide over the loader threads");
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
     __shared__ __attribute__((aligned(16))) u16 sS[2 * SSZ];
     const int l = threadIdx.x & 63, g = l >> 4, m = l & 15;
-    const int w8 = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const bool state_role = w8 >= 4;
-    const int w = w8 & 3;              // index within the role
-    const int tid = threadIdx.x & 255; // thread index within the role
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const WorkItem wi = decode_workgroup(set.count, G);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
@@ -251,40 +254,22 @@ __global__ __launch_bounds__(2 * kThreads) void scan_kernel(ProblemSet set, int 
     const int p0 = wi.grp * cpg;
     const int p1 = min(p0 + cpg, nchunks);
 
-    if (state_role) {
+    if (wv >= OW + 4) {
+        // ---------------------------------------------------------------- loader wavefronts
+        const int tid = (int)threadIdx.x - 64 * (OW + 4);  // 0..LT-1
         const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
         const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
-        f32x4 S[TL::TPW];
-#pragma unroll
-        for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (pr.gstate != nullptr) {
-            const f32x4 *gs =
-                reinterpret_cast<const f32x4 *>(pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS);
-#pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
-        }
-        u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
+        u32x4 rb[PF][8 * DI / LT], rc[PF][8 * DJ / LT];
         auto load_chunk = [&](int s, int p) {
             const int pc = min(p, p1 - 1);
             const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
-            load_tile<DI>(rb[s], rB, row0, di, tid);
-            load_tile<DJ>(rc[s], rC, row0, ldc, tid);
-        };
-        // 16-bit copy of the state, transposed to [j][i] for the A_w S product
-        auto put_state = [&](u16 *dst) {
-#pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) {
-                const int t = w * TL::TPW + u;
-                const int it = t / TL::NJT, jt = t % TL::NJT;
-                u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
-                *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
-            }
+            load_tile<DI, LT>(rb[s], rB, row0, di, tid);
+            load_tile<DJ, LT>(rc[s], rC, row0, ldc, tid);
         };
 #pragma unroll
         for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
-        store_tile<DI, TL::BS>(sB, rb[0], di, tid);
-        store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
-        put_state(sS);
+        store_tile<DI, TL::BS, LT>(sB, rb[0], di, tid);
+        store_tile<DJ, TL::CS, LT>(sC, rc[0], dj, tid);
         load_chunk(0, p0 + PF);
         __syncthreads();
         for (int pb = p0;; pb += PF) {
@@ -295,23 +280,56 @@ __global__ __launch_bounds__(2 * kThreads) void scan_kernel(ProblemSet set, int 
                 const int s1 = (s + 1) % PF;
                 const int buf = (p - p0) & 1;
                 // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
-                store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-                store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+                store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+                store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
                 load_chunk(s1, p + 1 + PF);
-                state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
-                put_state(sS + (buf ^ 1) * SSZ);
                 __syncthreads();
             }
         }
+    } else if (wv >= OW) {
+        // ---------------------------------------------------------------- state wavefronts
+        const int w = wv - OW;  // 0..3
+        f32x4 S[TL::TPW];
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (pr.gstate != nullptr) {
+            const f32x4 *gs =
+                reinterpret_cast<const f32x4 *>(pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS);
+#pragma unroll
+            for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
+        }
+        // 16-bit copy of the state, transposed to [j][i] for the A_blk S product
+        auto put_state = [&](u16 *dst) {
+#pragma unroll
+            for (int u = 0; u < TL::TPW; ++u) {
+                const int t = w * TL::TPW + u;
+                const int it = t / TL::NJT, jt = t % TL::NJT;
+                u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
+                *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
+            }
+        };
+        put_state(sS);
+        __syncthreads();
+        for (int p = p0; p < p1; ++p) {
+            const int buf = (p - p0) & 1;
+            state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+            put_state(sS + (buf ^ 1) * SSZ);
+            __syncthreads();
+        }
     } else {
+        // ---------------------------------------------------------------- output wavefronts
+        const int w = wv;  // 0..OW-1
         const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
         const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
-        u32x4 qn[PF][TL::KS], qc[TL::KS];
+        u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
         auto load_q = [&](int s, int p) {
             const int pc = min(p, p1 - 1);
-            const int row = (reversed ? nchunks - 1 - pc : pc) * kChunk + 16 * w + m;
+            const int row = (reversed ? nchunks - 1 - pc : pc) * kChunk + 16 * IB * w + m;
 #pragma unroll
-            for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + 32 * ks + 8 * g) * 2u);
+            for (int ib = 0; ib < IB; ++ib)
+#pragma unroll
+                for (int ks = 0; ks < TL::KS; ++ks)
+                    qn[s][ib][ks] = buf_load16(rA, (uint32_t)((row + 16 * ib) * di + 32 * ks + 8 * g) * 2u);
         };
 #pragma unroll
         for (int s = 0; s < PF; ++s) load_q(s, p0 + s);
@@ -325,13 +343,15 @@ __global__ __launch_bounds__(2 * kThreads) void scan_kernel(ProblemSet set, int 
                 const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
                 const int row0 = (reversed ? nchunks - 1 - p : p) * kChunk;
 #pragma unroll
-                for (int ks = 0; ks < TL::KS; ++ks)
-                    qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
+                for (int ib = 0; ib < IB; ++ib)
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        qc[ib][ks] = (32 * ks + 8 * g < di) ? qn[s][ib][ks] : u32x4{0u, 0u, 0u, 0u};
                 load_q(s, p + PF);
 
-                // masked scores, transposed: pk[jt] = P^T[16jt+4g .. +3][16w+m]; fragment reads first,
-                // MFMAs after, so the LDS latency is paid once per batch
-                u32x2 pk[4];
+                // masked scores, transposed: pk[ib][jt] = P^T[16jt+4g .. +3][16(IB*w+ib)+m]; fragment
+                // reads first, MFMAs after, so the LDS latency is paid once per batch
+                u32x2 pk[IB][4];
                 {
                     u32x4 kf[4][TL::KS];
 #pragma unroll
@@ -341,22 +361,25 @@ __global__ __launch_bounds__(2 * kThreads) void scan_kernel(ProblemSet set, int 
                             kf[jt][ks] =
                                 *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
 #pragma unroll
-                    for (int jt = 0; jt < 4; ++jt) {
-                        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                    for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
-                        for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ks], acc);
-                        const int d0 = 16 * (jt - w) + 4 * g - m;  // key position minus query position, r = 0
+                        for (int jt = 0; jt < 4; ++jt) {
+                            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const bool keep = reversed ? (d0 + r >= 0) : (d0 + r <= 0);
-                            acc[r] = keep ? acc[r] : 0.f;
+                            for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ib][ks], acc);
+                            const int d0 = 16 * (jt - (IB * w + ib)) + 4 * g - m;  // key pos - query pos at r = 0
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                const bool keep = reversed ? (d0 + r >= 0) : (d0 + r <= 0);
+                                acc[r] = keep ? acc[r] : 0.f;
+                            }
+                            pk[ib][jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
                         }
-                        pk[jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
-                    }
                 }
 
-                const int orow = row0 + 16 * w + m;
-                constexpr int JB = (8 / TL::KS < TL::NJT) ? (8 / TL::KS) : TL::NJT;  // output tiles per read batch
+                const int orow = row0 + 16 * IB * w + m;
+                constexpr int JBmax = (IB == 1) ? 8 : 4;
+                constexpr int JB = (JBmax / TL::KS < 1) ? 1 : ((JBmax / TL::KS < TL::NJT) ? (JBmax / TL::KS) : TL::NJT);
 #pragma unroll
                 for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
                     u32x4 vf[JB][2], sf[JB][TL::KS];
@@ -373,17 +396,21 @@ __global__ __launch_bounds__(2 * kThreads) void scan_kernel(ProblemSet set, int 
                                 *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
                     }
 #pragma unroll
-                    for (int jj = 0; jj < JB; ++jj) {
-                        const int jt = j0 + jj;
-                        f32x4 o = {0.f, 0.f, 0.f, 0.f};
+                    for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
-                        for (int kb = 0; kb < 2; ++kb) o = TR::mfma(vf[jj][kb], cat(pk[2 * kb], pk[2 * kb + 1]), o);
+                        for (int jj = 0; jj < JB; ++jj) {
+                            const int jt = j0 + jj;
+                            f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ks], o);
-                        const int col = 16 * jt + 4 * g;
-                        const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
-                        buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
-                    }
+                            for (int kb = 0; kb < 2; ++kb)
+                                o = TR::mfma(vf[jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
+#pragma unroll
+                            for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ib][ks], o);
+                            const int col = 16 * jt + 4 * g;
+                            const uint32_t off =
+                                (col < dj) ? (uint32_t)((orow + 16 * ib) * ldc + col) * 2u : kOobOffset;
+                            buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
+                        }
                 }
                 __syncthreads();
             }
