@@ -483,4 +483,111 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
     }
 }
 
+// Non-causal form for a head that one workgroup handles alone (no sequence groups): pass 1 sums
+// S = B^T C over the whole sequence in fp32 accumulators (the group_state loop), pass 2 applies
+// out = A S chunk by chunk with the 16-bit state held in registers.  No workspace, one launch.
+template <class TR, int DI, int DJ, int PF>
+__global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int BH, int N, int nchunks) {
+    using TL = Tiling<DI, DJ>;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS;
+    __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
+    __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
+    __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
+    const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const WorkItem wi = decode_workgroup(set.count, 1);
+    if (wi.bh >= BH) return;
+    const Problem &pr = set.p[wi.prob];
+    const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
+    const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
+    const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
+    const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+
+    u32x4 qn[PF][TL::KS];
+    auto load_q = [&](int s, int p) {
+        const int row = min(p, nchunks - 1) * kChunk + 16 * w + m;
+#pragma unroll
+        for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + 32 * ks + 8 * g) * 2u);
+    };
+
+    // ---- pass 1: S = sum over all chunks of B_c^T C_c
+    f32x4 S[TL::TPW];
+#pragma unroll
+    for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    {
+        u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
+        auto load_chunk = [&](int s, int p) {
+            const int row0 = min(p, nchunks - 1) * kChunk;
+            load_tile<DI>(rb[s], rB, row0, di, tid);
+            load_tile<DJ>(rc[s], rC, row0, ldc, tid);
+        };
+#pragma unroll
+        for (int s = 0; s < PF; ++s) load_chunk(s, s);
+        store_tile<DI, TL::BS>(sB, rb[0], di, tid);
+        store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
+        load_chunk(0, PF);
+        __syncthreads();
+        bool more = true;
+        for (int pb = 0; more; pb += PF) {
+#pragma unroll
+            for (int s = 0; s < PF; ++s) {
+                const int p = pb + s;
+                if (p >= nchunks) {
+                    more = false;
+                } else {
+                    const int s1 = (s + 1) % PF;
+                    const int buf = p & 1;
+                    store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+                    store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+                    load_chunk(s1, p + 1 + PF);
+                    state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+                    __syncthreads();
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_q(s, s);  // in flight while the state is converted
+
+    // ---- hand-over: 16-bit state, transposed to [j][i], through LDS into every wavefront's registers
+#pragma unroll
+    for (int u = 0; u < TL::TPW; ++u) {
+        const int t = w * TL::TPW + u;
+        const int it = t / TL::NJT, jt = t % TL::NJT;
+        u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
+        *reinterpret_cast<u32x2 *>(sS + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
+    }
+    __syncthreads();
+    u32x4 sf[TL::NJT][TL::KS];
+#pragma unroll
+    for (int jt = 0; jt < TL::NJT; ++jt)
+#pragma unroll
+        for (int ks = 0; ks < TL::KS; ++ks)
+            sf[jt][ks] = *reinterpret_cast<const u32x4 *>(sS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
+
+    // ---- pass 2: out_c = A_c S
+    for (int pb = 0;; pb += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int p = pb + s;
+            if (p >= nchunks) return;
+            u32x4 qc[TL::KS];
+#pragma unroll
+            for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
+            load_q(s, p + PF);
+            const int orow = p * kChunk + 16 * w + m;
+#pragma unroll
+            for (int jt = 0; jt < TL::NJT; ++jt) {
+                f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jt][ks], qc[ks], o);
+                const int col = 16 * jt + 4 * g;
+                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
+                buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
+            }
+        }
+    }
+}
+
 }  // namespace cott

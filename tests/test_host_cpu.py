@@ -70,8 +70,9 @@ def test_workspace_queries_are_pure_host_functions():
     # fp32 takes the generic path -> none either
     assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F32) == 0
     assert L.cott_causal_bwd_workspace_bytes(1, 2, 8192, 64, 64, _loader.BF16) > 0
-    # the non-causal form always stages K^T V through the workspace
-    assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.BF16) > 0
+    # non-causal: many heads -> one fused launch per head, no workspace; few heads -> group slots
+    assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.BF16) == 0
+    assert L.cott_noncausal_workspace_bytes(1, 2, 8192, 64, 64, _loader.BF16) > 0
 
 
 def test_c_abi_argument_errors_without_a_gpu():
