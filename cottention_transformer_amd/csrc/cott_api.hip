@@ -85,9 +85,12 @@ int split_policy() {
     return v;
 }
 
-bool use_mfma(int dtype, int di, int dj) {
-    return (dtype == COTT_F16 || dtype == COTT_BF16) && di % 16 == 0 && dj % 16 == 0 && di >= 32 && dj >= 32 &&
-           di <= 128 && dj <= 128;
+bool use_mfma(int dtype, int di, int dj, int N) {
+    const bool dims = di % 16 == 0 && dj % 16 == 0 && di >= 32 && dj >= 32 && di <= 128 && dj <= 128;
+    if (dtype == COTT_F16 || dtype == COTT_BF16) return dims;
+    // fp32: byte offsets within a head must stay below 2^32
+    if (dtype == COTT_F32) return dims && (long)N * (di > dj ? di : dj) <= (1L << 29);
+    return false;
 }
 
 // One full-tensor generic op out = G(A,B,C).
@@ -104,10 +107,10 @@ struct SetPlan {
     size_t ws_bytes;      // group-state slots
 };
 
-SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal) {
+SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtype) {
     SetPlan p;
     const long tgt = target_workgroups();
-    const bool can_split = dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
+    const bool can_split = dtype != COTT_F32 && dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
     const int pol = split_policy();
     p.nchunks = (N + 63) / 64;
     // Choose (column halves, sequence groups) to fill the target without exceeding it: halves cost
@@ -138,8 +141,9 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal) {
     p.cpg = (p.nchunks + best_g - 1) / best_g;
     p.G = (p.nchunks + p.cpg - 1) / p.cpg;
     const size_t state = cott::mfma_state_floats(di, dj / p.halves) * sizeof(float);
-    (void)causal;
-    p.ws_bytes = p.G > 1 ? (size_t)nops * p.halves * BH * p.G * state : 0;
+    // the fp32 kernels stage the non-causal state through the workspace even for one group
+    const bool slots = p.G > 1 || (!causal && dtype == COTT_F32);
+    p.ws_bytes = slots ? (size_t)nops * p.halves * BH * p.G * state : 0;
     return p;
 }
 
@@ -149,7 +153,7 @@ int pad_key(const Op &o) { return cott::mfma_pad(o.di) * 1000 + cott::mfma_pad(o
 size_t ops_workspace(const Op *ops, int n, long BH, int N, int dtype, bool causal) {
     if (BH <= 0 || N <= 0) return 0;
     for (int i = 0; i < n; ++i)
-        if (!use_mfma(dtype, ops[i].di, ops[i].dj)) return 0;
+        if (!use_mfma(dtype, ops[i].di, ops[i].dj, N)) return 0;
     size_t total = 0;
     bool done[8] = {false};
     for (int i = 0; i < n; ++i) {
@@ -157,7 +161,7 @@ size_t ops_workspace(const Op *ops, int n, long BH, int N, int dtype, bool causa
         int cnt = 0;
         for (int j = i; j < n; ++j)
             if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; ++cnt; }
-        total += plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal).ws_bytes;
+        total += plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal, dtype).ws_bytes;
     }
     return total;
 }
@@ -180,7 +184,7 @@ int check_common(const char *fn, int B, int H, int N, int di, int dj, int dtype)
 int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, int dtype, void *ws, size_t ws_bytes,
             hipStream_t stream) {
     bool mfma = true;
-    for (int i = 0; i < n; ++i) mfma = mfma && use_mfma(dtype, ops[i].di, ops[i].dj);
+    for (int i = 0; i < n; ++i) mfma = mfma && use_mfma(dtype, ops[i].di, ops[i].dj, N);
     const size_t esz = elem_size(dtype);
     if (!mfma) {
         for (int i = 0; i < n; ++i) {
@@ -206,7 +210,7 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         int members[8], cnt = 0;
         for (int j = i; j < n; ++j)
             if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; members[cnt++] = j; }
-        const SetPlan p = plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal);
+        const SetPlan p = plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal, dtype);
         for (int c = 0; c < cnt; ++c) {
             const Op &o = ops[members[c]];
             const int djh = o.dj / p.halves;
@@ -229,7 +233,9 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         a.scan_prof_id = n > 1 ? cott::K_SCAN_GRAD : cott::K_SCAN;
         a.stream = stream;
         hipError_t e;
-        if (dtype == COTT_BF16)
+        if (dtype == COTT_F32)
+            e = causal ? cott::launch_causal_mfma_f32(a) : cott::launch_noncausal_mfma_f32(a);
+        else if (dtype == COTT_BF16)
             e = causal ? cott::launch_causal_mfma_bf16(a) : cott::launch_noncausal_mfma_bf16(a);
         else
             e = causal ? cott::launch_causal_mfma_fp16(a) : cott::launch_noncausal_mfma_fp16(a);

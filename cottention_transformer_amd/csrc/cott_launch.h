@@ -17,7 +17,7 @@ struct OpDesc {
 struct SetArgs {
     OpDesc op[6];
     int count;
-    float *ws;            // count * BH * G * state_floats floats when G > 1 or non-causal, else unused
+    float *ws;            // count * BH * G * state_floats floats of group-state slots, or null when unused
     int BH, N;
     int nchunks, cpg, G;  // chunks of 64, chunks per group, groups per head
     int scan_prof_id;     // K_SCAN for a forward launch, K_SCAN_GRAD for the three-gradient launch
@@ -52,6 +52,9 @@ hipError_t launch_causal_mfma_bf16(const SetArgs &a);
 hipError_t launch_causal_mfma_fp16(const SetArgs &a);
 hipError_t launch_noncausal_mfma_bf16(const SetArgs &a);
 hipError_t launch_noncausal_mfma_fp16(const SetArgs &a);
+// fp32 storage on the fp32 MFMA; same limits, no column-half problems, workspace also for the non-causal form.
+hipError_t launch_causal_mfma_f32(const SetArgs &a);
+hipError_t launch_noncausal_mfma_f32(const SetArgs &a);
 
 // Plain-FMA fallback for any dtype / head dim, one op (full tensors: ldc == dj).
 // Returns hipErrorInvalidValue if no tiling fits LDS.

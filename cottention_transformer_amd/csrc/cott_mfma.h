@@ -26,17 +26,21 @@ constexpr int kXcds = 8;       // workgroup i is dispatched to XCD i % 8
 // One generic op.  A, B: rows of `di` elements, contiguous.  C, O: `dj` columns taken from rows of
 // `ldc` elements (the pointers already include the first column), so a problem can own a column
 // slice of a wider tensor.  gstate: G slots of DI*DJ floats per head (G > 1 or non-causal).
-struct Problem {
-    const u16 *A, *B, *C;
-    u16 *O;
+template <class E>
+struct ProblemT {
+    const E *A, *B, *C;
+    E *O;
     float *gstate;
     int di, dj, ldc, reversed;
 };
 
-struct ProblemSet {
-    Problem p[kMaxProblems];
+template <class E>
+struct ProblemSetT {
+    ProblemT<E> p[kMaxProblems];
     int count;
 };
+typedef ProblemT<u16> Problem;  // 16-bit storage (bf16 / fp16)
+typedef ProblemSetT<u16> ProblemSet;
 
 template <int DI, int DJ>
 struct Tiling {
@@ -200,8 +204,9 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
 
 // Over the G slots of one head, element-wise: mode 0 -> exclusive prefix in place (slot g gets the
 // sum of slots < g; only the first `ncomputed` slots hold data), mode 1 -> total into slot 0.
-static __global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSet set, int BH, int G, int ncomputed,
-                                                                       int state_floats, int mode) {
+template <class E>
+__global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSetT<E> set, int BH, int G, int ncomputed,
+                                                                int state_floats, int mode) {
     const int sf4 = state_floats / 4;
     const int blocks_per_state = (sf4 + kThreads - 1) / kThreads;
     const int e = (blockIdx.x % blocks_per_state) * kThreads + threadIdx.x;

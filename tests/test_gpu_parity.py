@@ -47,6 +47,12 @@ CAUSAL_CASES = [
     (1, 1, 70, 256, 48, F32),     # D beyond the MFMA range -> generic path
     (1, 2, 77, 256, 256, BF),     # 16-bit storage on the generic path
     (1, 1, 64, 64, 24, F32),      # D_value not a multiple of 16 (only D_attn is checked, :372-374)
+    (1, 2, 1023, 64, 64, F32),    # fp32 MFMA kernels: ragged tail, one chunk per group
+    (2, 2, 257, 48, 80, F32),     # ... head dims padded to 64 / 128, steps of 32 positions
+    (1, 1, 130, 128, 128, F32),   # ... D=128
+    (1, 2, 130, 32, 128, F32),    # ... D=32 against a wide value head
+    (2, 3, 200, 64, 32, F32),     # ... two column tiles only (half the wavefronts own state)
+    (1, 3, 2500, 64, 64, F32),    # ... several chunks per group
 ]
 
 
@@ -100,7 +106,8 @@ def test_golden_fixtures(ct):
 
 
 @pytest.mark.parametrize("case", [(2, 3, 512, 64, 64, BF), (1, 2, 63, 64, 32, HF), (2, 2, 1000, 128, 128, BF),
-                                  (1, 2, 100, 64, 32, F32), (1, 2, 50, 32, 32, F64), (1, 1, 40, 256, 64, F32)],
+                                  (1, 2, 100, 64, 32, F32), (1, 2, 50, 32, 32, F64), (1, 1, 40, 256, 64, F32),
+                                  (2, 3, 512, 64, 64, F32), (1, 2, 1000, 128, 128, F32), (3, 2, 77, 48, 80, F32)],
                          ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
 def test_noncausal_forward_backward(ct, oracle, case):
     b, h, n, dk, dv, dt = case

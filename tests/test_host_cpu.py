@@ -67,8 +67,14 @@ def test_workspace_queries_are_pure_host_functions():
     assert ws > 0 and ws % (64 * 32 * 4) == 0
     # headline shape: B*H (x2 column halves) already fills the chip -> one group -> no workspace
     assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.BF16) == 0
-    # fp32 takes the generic path -> none either
-    assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F32) == 0
+    # fp32 has MFMA kernels too and is cut the same way; fp64 takes the plain-FMA path -> none
+    assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F32) > 0
+    # (no column halves in fp32: 128 heads are cut into two groups to reach 256 workgroups)
+    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 2 * 128 * 64 * 64 * 4
+    assert L.cott_causal_workspace_bytes(16, 16, 2048, 64, 64, _loader.F32) == 0
+    assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F64) == 0
+    # fp32 non-causal always stages K^T V through the workspace
+    assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.F32) > 0
     assert L.cott_causal_bwd_workspace_bytes(1, 2, 8192, 64, 64, _loader.BF16) > 0
     # non-causal: many heads -> one fused launch per head, no workspace; few heads -> group slots
     assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.BF16) == 0
