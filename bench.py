@@ -22,8 +22,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM-side bytes per launch at the headline shape, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
 # `bench.py --calibration-copy` (counters scaled by their reading for the 256 MiB copy in the same run).
 # A counter run cannot be made from inside this script; the figures and commands are in
-# profiles/scan_kernel_headline_hbm_traffic_pmc.txt.
-MEASURED_TRAFFIC_BYTES = {"scan": 128.10 * 2**20, "scan_grad": 312.78 * 2**20}
+# profiles/headline_kernels_hbm_traffic_pmc.txt.
+MEASURED_TRAFFIC_BYTES = {"scan": 128.11 * 2**20, "scan_grad": 312.33 * 2**20}
 
 
 def parse():
@@ -68,7 +68,7 @@ def cpu_baseline(torch):
     b, h, n, d = 1, 16, 2048, 64
     q, k, v, g = tf.synthetic_inputs((b, h, n, d), seed=0, dtype=torch.float32)
     times = []
-    for it in range(4):
+    for it in range(25):
         qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
         t0 = time.perf_counter()
         tf.causal_cumsum(qa, ka, va).backward(g)
@@ -76,7 +76,7 @@ def cpu_baseline(torch):
     t = statistics.median(times[1:])
     return {"value": b * n / t, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"(B,H,N,D)=({b},{h},{n},{d}) fp32: 1 of the 8 batch elements of the headline shape, torch cumsum "
-                      f"form fwd + autograd bwd, median of 3 after 1 warm-up; {t:.2f} s per pass"}
+                      f"form fwd + autograd bwd, median of 24 passes after 1 warm-up; {t:.2f} s per pass"}
 
 
 def main():
@@ -210,6 +210,21 @@ def run_extras(torch, ct, dev):
                          "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS}
         del q, k, v, do
     ex["long_context_fwd_bwd_B1_H16_D128"] = sweep
+    # fp32 storage at the headline shape (what the backward of an autocast training step runs: the autograd
+    # function saves the fp32 inputs, Cuda_Kernel/Custom_Kernel.py:16,38); fp32 MFMA, peak 157.3 TFLOP/s
+    q, k, v, do = make_inputs(torch, 8, 16, 2048, 64, 64, torch.float32, dev)
+
+    def step32():
+        ct.causal_dot_product(q, k, v)
+        ct.causal_backward(q, k, v, do)
+    s = time_region(torch, step32, 20, 3)
+    byts = 11 * 8 * 16 * 2048 * 64 * 4
+    flops = 28.0 * 8 * 16 * 2048 * 64 * 64   # executed by the chunked form (scores recomputed per gradient)
+    ex["fp32_fwd_bwd_B8_H16_N2048_D64"] = {"us": s * 1e6, "tokens_per_s": 8 * 2048 / s, "GBps": byts / s / 1e9,
+                                           "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS,
+                                           "executed_tflops": flops / s / 1e12,
+                                           "frac_mfma_fp32": flops / s / 1e12 / 157.3}
+    del q, k, v, do
     return ex
 
 

@@ -109,7 +109,8 @@ struct SetPlan {
 
 SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtype) {
     SetPlan p;
-    const long tgt = target_workgroups();
+    // the fp32 kernels are MFMA-bound with four wavefronts per workgroup: two workgroups per CU overlap well
+    const long tgt = target_workgroups() * (dtype == COTT_F32 ? 2 : 1);
     const bool can_split = dtype != COTT_F32 && dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
     const int pol = split_policy();
     p.nchunks = (N + 63) / 64;

@@ -69,9 +69,9 @@ def test_workspace_queries_are_pure_host_functions():
     assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.BF16) == 0
     # fp32 has MFMA kernels too and is cut the same way; fp64 takes the plain-FMA path -> none
     assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F32) > 0
-    # (no column halves in fp32: 128 heads are cut into two groups to reach 256 workgroups)
-    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 2 * 128 * 64 * 64 * 4
-    assert L.cott_causal_workspace_bytes(16, 16, 2048, 64, 64, _loader.F32) == 0
+    # (no column halves in fp32: 128 heads are cut into four groups to reach two workgroups per CU)
+    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 4 * 128 * 64 * 64 * 4
+    assert L.cott_causal_workspace_bytes(32, 16, 2048, 64, 64, _loader.F32) == 0
     assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F64) == 0
     # fp32 non-causal always stages K^T V through the workspace
     assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.F32) > 0
