@@ -5,10 +5,10 @@ include/cottention.h; this package is the torch-facing host side.  `Cuda_Kernel/
 named like the reference's extension (`FastAttention2.kernel`, `FastAttention.forward/backward`,
 `Custom_Kernel.CustomAttention`) so its callers import them unchanged.
 """
-from .ops import (causal_backward, causal_dot_product, decode_step, noncausal_backward,  # noqa: F401
+from .ops import (causal_backward, causal_dot_product, causal_prefill, decode_step, noncausal_backward,  # noqa: F401
                   noncausal_dot_product)
 
-__all__ = ["causal_dot_product", "causal_backward", "noncausal_dot_product", "noncausal_backward", "decode_step",
+__all__ = ["causal_dot_product", "causal_prefill", "causal_backward", "noncausal_dot_product", "noncausal_backward", "decode_step",
            "CustomAttention", "NonCausalAttention"]
 
 

@@ -18,6 +18,7 @@ SIGNATURES = {
     "cott_last_error": (ctypes.c_char_p, []),
     "cott_causal_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_fwd": (_i, [_vp] * 4 + [_i] * 7 + [_vp, _sz, _vp]),
+    "cott_causal_fwd_state": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_causal_bwd_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_workspace_bytes": (_sz, [_i] * 6),

@@ -98,6 +98,8 @@ struct Op {
     const void *A, *B, *C;
     void *O;
     int di, dj, reversed;
+    const void *sin = nullptr;  // (BH,di,dj) state to start from / to receive the final state (causal only)
+    void *sout = nullptr;
 };
 
 // How a set of `nops` ops with the same padded head dims is laid on the chip.
@@ -192,7 +194,8 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
             if (!cott::generic_fits(dtype, ops[i].di))
                 return fail(COTT_ERR_UNSUPPORTED, "%s: head dim %d too large for dtype %d on this build", fn, ops[i].di,
                             dtype);
-            cott::OpDesc d{ops[i].A, ops[i].B, ops[i].C, ops[i].O, ops[i].di, ops[i].dj, ops[i].dj, ops[i].reversed};
+            cott::OpDesc d{ops[i].A, ops[i].B, ops[i].C, ops[i].O, ops[i].di, ops[i].dj, ops[i].dj, ops[i].reversed,
+                           ops[i].sin,  ops[i].sout, ops[i].dj};
             hipError_t e = cott::launch_generic(dtype, causal, d, (int)BH, N, stream);
             if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
         }
@@ -225,6 +228,10 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
                 d.dj = djh;
                 d.ldc = o.dj;
                 d.reversed = o.reversed;
+                const size_t ssz = dtype == COTT_F64 ? 8 : 4;
+                d.sin = o.sin ? static_cast<const char *>(o.sin) + (size_t)h * djh * ssz : nullptr;
+                d.sout = o.sout ? static_cast<char *>(o.sout) + (size_t)h * djh * ssz : nullptr;
+                d.lds = o.dj;
             }
         }
         a.ws = p.ws_bytes ? reinterpret_cast<float *>(ws_cursor) : nullptr;
@@ -316,6 +323,37 @@ int cott_causal_fwd(const void *q, const void *k, const void *v, void *o, int B,
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
     const Op op{q, k, v, o, Dk, Dv, reversed ? 1 : 0};
     return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int cott_causal_fwd_state(const void *q, const void *k, const void *v, void *o, const void *state_in, void *state_out,
+                          int B, int H, int N, int Dk, int Dv, int dtype, void *workspace, size_t workspace_bytes,
+                          void *stream) {
+    const char *fn = "cott_causal_fwd_state";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    const long BH = (long)B * H;
+    if (BH == 0) return COTT_OK;
+    const size_t ssz = dtype == COTT_F64 ? 8 : 4;
+    const uintptr_t smask = dtype == COTT_F64 ? 31u : 15u;
+    if ((reinterpret_cast<uintptr_t>(state_in) & smask) || (reinterpret_cast<uintptr_t>(state_out) & smask))
+        return fail(COTT_ERR_INVALID, "%s: state pointers must be 16-byte (fp64: 32-byte) aligned", fn);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (N == 0) {  // nothing to scan: the state passes through
+        if (state_out && state_in && state_out != state_in) {
+            hipError_t e = hipMemcpyAsync(state_out, state_in, (size_t)BH * Dk * Dv * ssz, hipMemcpyDeviceToDevice, st);
+            if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: state copy failed: %s", fn, hipGetErrorString(e));
+        } else if (state_out && !state_in) {
+            hipError_t e = hipMemsetAsync(state_out, 0, (size_t)BH * Dk * Dv * ssz, st);
+            if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: state clear failed: %s", fn, hipGetErrorString(e));
+        }
+        return COTT_OK;
+    }
+    if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op op{q, k, v, o, Dk, Dv, 0};
+    op.sin = state_in;
+    op.sout = state_out;
+    return run_ops(fn, true, &op, 1, BH, N, dtype, workspace, workspace_bytes, st);
 }
 
 size_t cott_causal_bwd_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype) {

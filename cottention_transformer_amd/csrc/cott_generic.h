@@ -37,7 +37,9 @@ template <class ST, bool CAUSAL>
 __global__ __launch_bounds__(256) void generic_scan_kernel(const typename ST::elem *__restrict__ A,
                                                            const typename ST::elem *__restrict__ B,
                                                            const typename ST::elem *__restrict__ C,
-                                                           typename ST::elem *__restrict__ O, int N, int di, int dj,
+                                                           typename ST::elem *__restrict__ O,
+                                                           const typename ST::acc *__restrict__ sin,
+                                                           typename ST::acc *__restrict__ sout, int N, int di, int dj,
                                                            int CH, int DJT, int nslices, int reversed) {
     typedef typename ST::acc acc_t;
     extern __shared__ __attribute__((aligned(32))) unsigned char smem_raw[];
@@ -55,7 +57,11 @@ __global__ __launch_bounds__(256) void generic_scan_kernel(const typename ST::el
     const int nchunks = (N + CH - 1) / CH;
     const int lda = di + 1;
 
-    for (int x = tid; x < di * DJT; x += 256) sS[x] = (acc_t)0;
+    // start state: zero, or the caller's [di][dj] row-major state of this head
+    for (int x = tid; x < di * DJT; x += 256) {
+        const int i = x / DJT, jj = x % DJT;
+        sS[x] = (sin != nullptr && j0 + jj < dj) ? sin[((size_t)bh * di + i) * dj + j0 + jj] : (acc_t)0;
+    }
 
     auto load_bc = [&](int row0) {
         for (int x = tid; x < CH * di; x += 256) {
@@ -115,6 +121,13 @@ __global__ __launch_bounds__(256) void generic_scan_kernel(const typename ST::el
         if (CAUSAL) {
             __syncthreads();
             update_state();
+        }
+    }
+    if (sout != nullptr) {
+        __syncthreads();
+        for (int x = tid; x < di * DJT; x += 256) {
+            const int i = x / DJT, jj = x % DJT;
+            if (j0 + jj < dj) sout[((size_t)bh * di + i) * dj + j0 + jj] = sS[x];
         }
     }
 }

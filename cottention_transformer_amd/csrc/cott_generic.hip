@@ -46,7 +46,7 @@ hipError_t run_generic(const OpDesc &a, int BH, int N, hipStream_t stream) {
     ProfScope ps(K_GENERIC, stream);
     kern<<<dim3((unsigned)(BH * nslices)), dim3(256), t.bytes, stream>>>(
         static_cast<const E *>(a.A), static_cast<const E *>(a.B), static_cast<const E *>(a.C), static_cast<E *>(a.O),
-        N, a.di, a.dj, t.CH, t.DJT, nslices, a.reversed);
+        static_cast<const typename ST::acc *>(a.sin), static_cast<typename ST::acc *>(a.sout), N, a.di, a.dj, t.CH, t.DJT, nslices, a.reversed);
     return hipGetLastError();
 }
 

@@ -11,6 +11,11 @@ struct OpDesc {
     const void *A, *B, *C;  // A,B: (BH,N,di)  C: (BH,N,ldc)
     void *O;                // (BH,N,ldc)
     int di, dj, ldc, reversed;
+    // Optional hand-over of the recurrence state (causal ops only): (BH,di,lds) row-major, fp32
+    // (fp64 for fp64 tensors), pointers offset to the first column like C and O.
+    const void *sin = nullptr;  // start from this state instead of zero
+    void *sout = nullptr;       // receives the state after the last position
+    int lds = 0;
 };
 
 // A set of ops launched together over the same (BH, N); MFMA path: all share padded head dims.

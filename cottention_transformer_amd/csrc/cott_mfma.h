@@ -26,12 +26,16 @@ constexpr int kXcds = 8;       // workgroup i is dispatched to XCD i % 8
 // One generic op.  A, B: rows of `di` elements, contiguous.  C, O: `dj` columns taken from rows of
 // `ldc` elements (the pointers already include the first column), so a problem can own a column
 // slice of a wider tensor.  gstate: G slots of DI*DJ floats per head (G > 1 or non-causal).
+// sin / sout (either may be null): row-major fp32 [di][lds] state per head, likewise offset to the
+// first column; the scan starts from sin and its last group writes the final state to sout.
 template <class E>
 struct ProblemT {
     const E *A, *B, *C;
     E *O;
     float *gstate;
-    int di, dj, ldc, reversed;
+    const float *sin;
+    float *sout;
+    int di, dj, ldc, reversed, lds;
 };
 
 template <class E>
@@ -303,6 +307,18 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
 #pragma unroll
             for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
         }
+        // accumulator element r of tile (it, jt) is S[16it + 4g + r][16jt + m]
+        if (pr.sin != nullptr) {
+            const float *si = pr.sin + (size_t)wi.bh * di * pr.lds;
+#pragma unroll
+            for (int u = 0; u < TL::TPW; ++u) {
+                const int t = w * TL::TPW + u;
+                const int i0 = 16 * (t / TL::NJT) + 4 * g, j = 16 * (t % TL::NJT) + m;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (i0 + r < di && j < dj) S[u][r] += si[(size_t)(i0 + r) * pr.lds + j];
+            }
+        }
         // 16-bit copy of the state, transposed to [j][i] for the A_blk S product
         auto put_state = [&](u16 *dst) {
 #pragma unroll
@@ -320,6 +336,17 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
             state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
             put_state(sS + (buf ^ 1) * SSZ);
             __syncthreads();
+        }
+        if (pr.sout != nullptr && wi.grp == G - 1) {
+            float *so = pr.sout + (size_t)wi.bh * di * pr.lds;
+#pragma unroll
+            for (int u = 0; u < TL::TPW; ++u) {
+                const int t = w * TL::TPW + u;
+                const int i0 = 16 * (t / TL::NJT) + 4 * g, j = 16 * (t % TL::NJT) + m;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (i0 + r < di && j < dj) so[(size_t)(i0 + r) * pr.lds + j] = S[u][r];
+            }
         }
     } else {
         // ---------------------------------------------------------------- output wavefronts

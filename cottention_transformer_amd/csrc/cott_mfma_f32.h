@@ -219,6 +219,21 @@ __global__ __launch_bounds__(kThreads) void scan_f32_kernel(ProblemSetF32 set, i
         read_state_f32<DI, DJ>(S, pr.gstate + (size_t)wi.bh * G * TL::STATE_FLOATS, w, l);
     else if (pr.gstate != nullptr)
         read_state_f32<DI, DJ>(S, pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS, w, l);
+    if (!APPLY && pr.sin != nullptr) {
+        const float *si = pr.sin + (size_t)wi.bh * di * pr.lds;
+#pragma unroll
+        for (int js = 0; js < TL::JPW; ++js)
+            if (w + 4 * js < TL::NJT) {
+                const int j = 16 * (w + 4 * js) + m;
+#pragma unroll
+                for (int it = 0; it < TL::NIT; ++it)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int i = 16 * it + 4 * g + r;
+                        if (i < di && j < dj) S.v[js][it][r] += si[(size_t)i * pr.lds + j];
+                    }
+            }
+    }
 
     u32x4 ra[TL::VA], rb[APPLY ? 1 : TL::VA], rc[APPLY ? 1 : TL::VC];
     auto load_step = [&](int p) {
@@ -314,6 +329,21 @@ __global__ __launch_bounds__(kThreads) void scan_f32_kernel(ProblemSetF32 set, i
         // (3) state
         if (!APPLY) state_update_f32<DI, DJ>(S, cf, sB, w, g, m);
         __syncthreads();
+    }
+    if (!APPLY && pr.sout != nullptr && wi.grp == G - 1) {
+        float *so = pr.sout + (size_t)wi.bh * di * pr.lds;
+#pragma unroll
+        for (int js = 0; js < TL::JPW; ++js)
+            if (w + 4 * js < TL::NJT) {
+                const int j = 16 * (w + 4 * js) + m;
+#pragma unroll
+                for (int it = 0; it < TL::NIT; ++it)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int i = 16 * it + 4 * g + r;
+                        if (i < di && j < dj) so[(size_t)i * pr.lds + j] = S.v[js][it][r];
+                    }
+            }
     }
 }
 

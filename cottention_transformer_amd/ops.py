@@ -75,6 +75,36 @@ def causal_dot_product(q, k, v, reversed=False):
     return o
 
 
+def causal_prefill(q, k, v, state=None, return_state=True):
+    """Causal forward over a whole prompt (or one piece of a sequence) with the recurrence state handed over:
+    returns (o, state_out) with o[s] = q[s] (state + sum_{s'<=s} k[s'] v[s']^T) and
+    state_out = state + sum_{s'} k[s'] v[s']^T, the tensor `decode_step` continues from.  Replaces the
+    per-token loop over the prompt of GPT_Trainer/GPTCosAttention.py:253-272.
+    state: None (zero) or (B,H,Dk,Dv) fp32 (fp64 for fp64 inputs); it is not modified."""
+    _require_gpu(Q=q, K=k, V=v)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("Q, K and V must have the same dtype")
+    code = _dtype_code(q)
+    sdt = torch.float64 if q.dtype == torch.float64 else torch.float32
+    if state is not None:
+        _require_gpu(state=state)
+        if state.shape != (b, h, dk, dv) or state.dtype != sdt or not state.is_contiguous():
+            raise RuntimeError(f"causal_prefill: state must be a contiguous {sdt} tensor of shape {(b, h, dk, dv)}")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
+    s_out = torch.empty((b, h, dk, dv), dtype=sdt, device=q.device) if return_state else None
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        ws, ws_ptr = _workspace(L.cott_causal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+        rc = L.cott_causal_fwd_state(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                     state.data_ptr() if state is not None else None,
+                                     s_out.data_ptr() if s_out is not None else None, b, h, n, dk, dv, code, ws_ptr,
+                                     ws.numel() if ws is not None else 0, _stream())
+    _check(rc, "cott_causal_fwd_state")
+    return o, s_out
+
+
 def causal_backward(q, k, v, grad_out):
     """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out."""
     _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)

@@ -57,6 +57,20 @@ COTT_API int cott_causal_fwd(const void *q, const void *k, const void *v, void *
                     int B, int H, int N, int Dk, int Dv, int dtype, int reversed,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- causal forward with state hand-over (prefill -> decode, or a sequence fed in pieces) -----
+ *   o[s,j] = sum_i q[s,i] * ( state_in[i,j] + sum_{s' <= s} k[s',i] * v[s',j] )
+ *   state_out[i,j] = state_in[i,j] + sum_{s' < N} k[s',i] * v[s',j]
+ * Replaces the per-token Python loop that the reference runs over a prompt to build its decode
+ * state (GPT_Trainer/GPTCosAttention.py:253-272; generation driver fast_infer.py:111): one call
+ * over the prompt yields the outputs of cott_causal_fwd AND the state that cott_decode_step
+ * continues from.  state_in / state_out: (B,H,Dk,Dv) fp32 (fp64 for COTT_F64), the layout of
+ * cott_decode_step; either may be NULL (start from zero / state not wanted); they may alias.
+ * Workspace: cott_causal_workspace_bytes().  N == 0 copies state_in to state_out. */
+COTT_API int cott_causal_fwd_state(const void *q, const void *k, const void *v, void *o,
+                          const void *state_in, void *state_out,
+                          int B, int H, int N, int Dk, int Dv, int dtype,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- causal backward ------------------------------------------------------------------------
  * (dq, dk, dv) of o = cott_causal_fwd(q,k,v) contracted with d_o.  Replaces the three launches
  * of CustomAttention.backward, Cuda_Kernel/Custom_Kernel.py:106-108 (closed forms :63,:68,:72)

@@ -151,6 +151,51 @@ def test_decode_after_prompt_equals_causal_forward(ct, oracle):
     # the reference's past_KV is the transposed state: (B,H,Dv,Dk) = sum v (x) k   (:264)
     assert rel_l2(state.transpose(-1, -2), np.einsum("bhne,bhnd->bhed", v.double().numpy(), k.double().numpy())) <= 1e-5
 
+PREFILL_CASES = [
+    (2, 3, 200, 64, 64, BF),      # one group, column halves
+    (1, 2, 1023, 64, 64, BF),     # several groups per head: every group starts from prefix + handed-over state
+    (8, 16, 256, 64, 64, BF),     # many heads
+    (1, 2, 130, 128, 128, HF),
+    (2, 2, 257, 48, 80, BF),      # padded head dims: state rows/columns beyond (Dk,Dv) must not be touched
+    (2, 2, 257, 48, 80, F32),
+    (1, 3, 2500, 64, 64, F32),
+    (1, 2, 63, 128, 128, F64),    # plain-FMA path, fp64 state
+    (1, 1, 70, 256, 48, F32),     # plain-FMA path, state slices
+]
+
+
+@pytest.mark.parametrize("case", PREFILL_CASES, ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_prefill_hands_state_to_next_piece_and_to_decode(ct, oracle, case):
+    # GPTCosAttention.py:253-272 builds the decode state token by token; here one call over the prompt returns it.
+    # Ground truth is the pinned causal oracle on the WHOLE sequence: feeding the sequence in two pieces with
+    # the state handed over, then three decode steps, must reproduce its rows.
+    b, h, n, dk, dv, dt = case
+    say("prefill", case)
+    extra = 3
+    q, k, v, _ = inputs(b, h, n + extra, dk, dv, dt, seed=n + 2)
+    ref = oracle.causal(q, k, v)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    n1 = n // 3 + 1
+    o1, s1 = ct.causal_prefill(qd[:, :, :n1], kd[:, :, :n1], vd[:, :, :n1])
+    s1_copy = s1.clone()
+    o2, s2 = ct.causal_prefill(qd[:, :, n1:n], kd[:, :, n1:n], vd[:, :, n1:n], state=s1)
+    assert torch.equal(s1, s1_copy), "input state must not be modified"
+    assert s2.dtype == (F64 if dt == F64 else F32) and s2.shape == (b, h, dk, dv)
+    assert rel_l2(torch.cat([o1, o2], 2), ref[:, :, :n]) <= TOL[dt]
+    kv = np.einsum("bhni,bhnj->bhij", k[:, :, :n].double().numpy(), v[:, :, :n].double().numpy())
+    assert rel_l2(s2, kv) <= (1e-12 if dt == F64 else 2e-6)
+    # one call over the whole prompt gives the same state
+    o, s = ct.causal_prefill(qd[:, :, :n], kd[:, :, :n], vd[:, :, :n])
+    assert rel_l2(o, ref[:, :, :n]) <= TOL[dt] and rel_l2(s, kv) <= (1e-12 if dt == F64 else 2e-6)
+    if dv % 4 == 0:
+        rows = [ct.decode_step(s2, qd[:, :, t], kd[:, :, t], vd[:, :, t]) for t in range(n, n + extra)]
+        assert rel_l2(torch.stack(rows, 2), ref[:, :, n:]) <= TOL[dt]
+    # return_state=False / empty piece
+    o3, none = ct.causal_prefill(qd[:, :, :n1], kd[:, :, :n1], vd[:, :, :n1], return_state=False)
+    assert none is None and torch.equal(o3, o1)
+    oe, se = ct.causal_prefill(qd[:, :, :0], kd[:, :, :0], vd[:, :, :0], state=s1)
+    assert oe.shape == (b, h, 0, dv) and torch.equal(se, s1)
+
 
 def test_padded_rows_and_noncontiguous_inputs(ct, oracle):
     b, h, n, d = 2, 4, 150, 64
