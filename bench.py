@@ -220,6 +220,24 @@ def run_extras(torch, ct, dev):
     s = time_region(torch, step32, 20, 3)
     byts = 11 * 8 * 16 * 2048 * 64 * 4
     flops = 28.0 * 8 * 16 * 2048 * 64 * 64   # executed by the chunked form (scores recomputed per gradient)
+    # fused input preparation (normalise q,k; scale v; mask; fp32 -> bf16) at the headline shape, next to the same
+    # sequence written with torch elementwise ops as the reference module does (GPTCosAttention.py:216-235)
+    keep = torch.rand(8, 2048, device=dev) > 0.1
+    cnt = keep.float().cumsum(-1)
+    sig = torch.sigmoid(torch.randn(16, device=dev))
+    s_f = time_region(torch, lambda: ct.prepare_inputs(q, k, v, keep, cnt, sig, out_dtype=torch.bfloat16), 50, 5)
+
+    def eager_prep():
+        m = keep[:, None, :, None]
+        qh = torch.nn.functional.normalize(q, dim=-1, p=2) * m
+        kh = torch.nn.functional.normalize(k, dim=-1, p=2) * m
+        vs = v / (cnt[:, None, :, None] ** sig.reshape(1, -1, 1, 1)).clamp(min=1) * m
+        return qh.bfloat16(), kh.bfloat16(), vs.bfloat16()
+    s_e = time_region(torch, eager_prep, 20, 3)
+    pb = 3 * 8 * 16 * 2048 * 64 * (4 + 2)
+    ex["input_prep_fwd_B8_H16_N2048_D64_f32_to_bf16"] = {"us": s_f * 1e6, "GBps": pb / s_f / 1e9,
+                                                         "frac_hbm": pb / s_f / 1e9 / HBM_PEAK_GBS,
+                                                         "torch_elementwise_us": s_e * 1e6}
     ex["fp32_fwd_bwd_B8_H16_N2048_D64"] = {"us": s * 1e6, "tokens_per_s": 8 * 2048 / s, "GBps": byts / s / 1e9,
                                            "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS,
                                            "executed_tflops": flops / s / 1e12,

@@ -6,14 +6,14 @@ named like the reference's extension (`FastAttention2.kernel`, `FastAttention.fo
 `Custom_Kernel.CustomAttention`) so its callers import them unchanged.
 """
 from .ops import (causal_backward, causal_dot_product, causal_prefill, decode_step, noncausal_backward,  # noqa: F401
-                  noncausal_dot_product)
+                  noncausal_dot_product, prepare_inputs, prepare_inputs_backward)
 
 __all__ = ["causal_dot_product", "causal_prefill", "causal_backward", "noncausal_dot_product", "noncausal_backward", "decode_step",
-           "CustomAttention", "NonCausalAttention"]
+           "prepare_inputs", "prepare_inputs_backward", "CustomAttention", "NonCausalAttention", "PrepareInputs"]
 
 
 def __getattr__(name):
-    if name in ("CustomAttention", "NonCausalAttention"):
+    if name in ("CustomAttention", "NonCausalAttention", "PrepareInputs"):
         from . import autograd
         return getattr(autograd, name)
     raise AttributeError(name)

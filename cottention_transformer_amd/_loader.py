@@ -19,6 +19,8 @@ SIGNATURES = {
     "cott_causal_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_fwd": (_i, [_vp] * 4 + [_i] * 7 + [_vp, _sz, _vp]),
     "cott_causal_fwd_state": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_prep_fwd": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
+    "cott_prep_bwd": (_i, [_vp] * 13 + [_i] * 7 + [_vp]),
     "cott_causal_bwd_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_workspace_bytes": (_sz, [_i] * 6),
@@ -30,7 +32,8 @@ SIGNATURES = {
     "cott_kernel_name": (ctypes.c_char_p, [_i]),
 }
 
-KERNEL_IDS = {"group_state": 0, "state_prefix": 1, "scan": 2, "apply": 3, "scan_grad": 4, "generic": 5, "decode": 6}
+KERNEL_IDS = {"group_state": 0, "state_prefix": 1, "scan": 2, "apply": 3, "scan_grad": 4, "generic": 5, "decode": 6,
+              "prep": 7}
 
 
 def profile_enable(on):

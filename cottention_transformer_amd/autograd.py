@@ -60,3 +60,25 @@ class NonCausalAttention(torch.autograd.Function):
         Q, K, V = ctx.saved_tensors
         g = grad_output.contiguous().to(Q.dtype)
         return ops.noncausal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g)
+
+
+class PrepareInputs(torch.autograd.Function):
+    """(q, k, v, keep, cnt, sig, out_dtype) -> (q_hat, k_hat, v_scaled): the normalise / value-scale / mask
+    steps in front of the attention op (GPT_Trainer/GPTCosAttention.py:216-241) as one fused operator with a
+    fused backward.  `sig` = sigmoid(norm_const) per head, differentiable; keep and cnt are constants."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, keep, cnt, sig, out_dtype):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        ctx.save_for_backward(q, k, v, keep, cnt, sig)
+        return ops.prepare_inputs(q, k, v, keep, cnt, sig, out_dtype)
+
+    @staticmethod
+    def backward(ctx, gq, gk, gv):
+        q, k, v, keep, cnt, sig = ctx.saved_tensors
+        want = sig is not None and ctx.needs_input_grad[5]
+        dq, dk, dv, dsig = ops.prepare_inputs_backward(q, k, v, gq.contiguous(), gk.contiguous(), gv.contiguous(), keep,
+                                                       cnt, sig, want_dsig=want)
+        if dsig is not None:
+            dsig = dsig.to(sig.dtype)
+        return dq, dk, dv, None, None, dsig, None

@@ -302,7 +302,7 @@ int cott_profile_read(int kernel_id, double *total_ms, long *launches) {
 const char *cott_kernel_name(int kernel_id) {
     static const char *names[cott::K_COUNT] = {"group_state_kernel", "state_prefix_kernel", "scan_kernel<causal>",
                                                "scan_kernel<apply>", "scan_kernel<causal> (dQ,dK,dV set)", "generic_scan_kernel",
-                                               "decode_kernel"};
+                                               "decode_kernel", "prep_kernel"};
     return (kernel_id >= 0 && kernel_id < cott::K_COUNT) ? names[kernel_id] : "";
 }
 
@@ -429,6 +429,55 @@ int cott_decode_step(void *state, const void *q, const void *k, const void *v, v
     if (!aligned16(state) || (dtype == COTT_F64 && (reinterpret_cast<uintptr_t>(state) & 31u)))
         return fail(COTT_ERR_INVALID, "%s: state must be 16-byte (fp64: 32-byte) aligned", fn);
     hipError_t e = cott::launch_decode(dtype, state, q, k, v, o, (int)BH, Dk, Dv, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
+    return COTT_OK;
+}
+
+namespace {
+int check_prep(const char *fn, int B, int H, int N, int Dk, int Dv, int d0, int d1) {
+    if (elem_size(d0) == 0 || elem_size(d1) == 0) return fail(COTT_ERR_INVALID, "%s: unknown dtype", fn);
+    if (B < 0 || H < 0 || N < 0 || Dk < 1 || Dv < 1) return fail(COTT_ERR_INVALID, "%s: bad size", fn);
+    if (Dk % 4 != 0 || Dv % 4 != 0) return fail(COTT_ERR_UNSUPPORTED, "%s: head dims must be multiples of 4", fn);
+    if (Dk > 1024 || Dv > 1024) return fail(COTT_ERR_UNSUPPORTED, "%s: head dims above 1024", fn);
+    if ((d0 == COTT_F64) != (d1 == COTT_F64)) return fail(COTT_ERR_UNSUPPORTED, "%s: fp64 only converts to fp64", fn);
+    return COTT_OK;
+}
+}  // namespace
+
+int cott_prep_fwd(const void *q, const void *k, const void *v, void *q_out, void *k_out, void *v_out,
+                  const unsigned char *keep, const float *cnt, const float *sig, int B, int H, int N, int Dk, int Dv,
+                  int in_dtype, int out_dtype, void *stream) {
+    const char *fn = "cott_prep_fwd";
+    if (int rc = check_prep(fn, B, H, N, Dk, Dv, in_dtype, out_dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (!q || !k || !v || !q_out || !k_out || !v_out) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(q_out) || !aligned16(k_out) || !aligned16(v_out))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    if ((cnt == nullptr) != (sig == nullptr)) return fail(COTT_ERR_INVALID, "%s: cnt and sig go together", fn);
+    const void *x[3] = {q, k, v};
+    void *y[3] = {q_out, k_out, v_out};
+    hipError_t e = cott::launch_prep(false, x, nullptr, y, keep, cnt, sig, nullptr, B, H, N, Dk, Dv, in_dtype, out_dtype,
+                                     out_dtype, 1e-12f, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
+    return COTT_OK;
+}
+
+int cott_prep_bwd(const void *q, const void *k, const void *v, const void *gq, const void *gk, const void *gv, void *dq,
+                  void *dk, void *dv, float *dsig_rows, const unsigned char *keep, const float *cnt, const float *sig,
+                  int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream) {
+    const char *fn = "cott_prep_bwd";
+    if (int rc = check_prep(fn, B, H, N, Dk, Dv, in_dtype, grad_dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (!q || !k || !v || !gq || !gk || !gv || !dq || !dk || !dv) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(gq) || !aligned16(gk) || !aligned16(gv) ||
+        !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    if ((cnt == nullptr) != (sig == nullptr)) return fail(COTT_ERR_INVALID, "%s: cnt and sig go together", fn);
+    const void *x[3] = {q, k, v};
+    const void *g[3] = {gq, gk, gv};
+    void *y[3] = {dq, dk, dv};
+    hipError_t e = cott::launch_prep(true, x, g, y, keep, cnt, sig, dsig_rows, B, H, N, Dk, Dv, in_dtype, in_dtype,
+                                     grad_dtype, 1e-12f, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
     return COTT_OK;
 }

@@ -30,7 +30,7 @@ struct SetArgs {
 };
 
 // Kernel families, as reported by cott_profile_read().
-enum KernelId { K_GROUP_STATE = 0, K_STATE_PREFIX, K_SCAN, K_APPLY, K_SCAN_GRAD, K_GENERIC, K_DECODE, K_COUNT };
+enum KernelId { K_GROUP_STATE = 0, K_STATE_PREFIX, K_SCAN, K_APPLY, K_SCAN_GRAD, K_GENERIC, K_DECODE, K_PREP, K_COUNT };
 
 // While profiling is enabled (cott_profile_enable), brackets the launches made in its lifetime
 // with a pair of HIP events on the launch stream; otherwise does nothing.
@@ -65,6 +65,11 @@ hipError_t launch_noncausal_mfma_f32(const SetArgs &a);
 // Returns hipErrorInvalidValue if no tiling fits LDS.
 hipError_t launch_generic(int dtype, bool causal, const OpDesc &op, int BH, int N, hipStream_t stream);
 bool generic_fits(int dtype, int di);
+
+// Fused input preparation (backward = false) or its backward; see cott_prep.hip.
+hipError_t launch_prep(bool backward, const void *const x[3], const void *const g[3], void *const y[3],
+                       const unsigned char *keep, const float *cnt, const float *sig, float *dsig_rows, int B, int H, int N,
+                       int dk, int dv, int x_dtype, int y_dtype, int g_dtype, float eps, hipStream_t stream);
 
 hipError_t launch_decode(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH,
                          int dk, int dv, hipStream_t stream);

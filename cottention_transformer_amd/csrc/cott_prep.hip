@@ -1,0 +1,270 @@
+// Fused input preparation of the cosine-attention module and its backward: L2-normalise the rows
+// of q and k, scale the rows of v by 1 / max(cnt^sig, 1), multiply all three by the 0/1 keep mask
+// and convert to the dtype the attention kernels run in -- one pass over each tensor
+// (GPT_Trainer/GPTCosAttention.py:216-241, BERT_Trainer/BertCosAttention.py:162-178 do this with
+// eight separate elementwise / reduction kernels).  Bandwidth-bound: every element is read once
+// and written once, rows are reduced with lane shuffles inside a wavefront.
+#include "cott_common.h"
+#include "cott_launch.h"
+#include "../../include/cottention.h"
+
+namespace cott {
+namespace {
+
+constexpr int kPrepThreads = 256;
+constexpr int kMaxVec = 4;  // a lane holds up to kMaxVec groups of 4 elements of its row: rows of up to 1024 elements
+
+template <class ACC>
+struct Vec4 {
+    ACC x[4];
+};
+
+template <class ACC>
+__device__ __forceinline__ Vec4<ACC> load4(const void *base, int dtype, size_t idx) {
+    Vec4<ACC> r;
+    switch (dtype) {
+        case COTT_F32: {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(static_cast<const float *>(base) + idx);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r.x[i] = (ACC)v[i];
+            break;
+        }
+        case COTT_F64: {
+            const double *p = static_cast<const double *>(base) + idx;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r.x[i] = (ACC)p[i];
+            break;
+        }
+        case COTT_F16: {
+            const u32x2 v = *reinterpret_cast<const u32x2 *>(static_cast<const u16 *>(base) + idx);
+            r.x[0] = (ACC)Fp16::to_float((u16)(v.x & 0xffffu));
+            r.x[1] = (ACC)Fp16::to_float((u16)(v.x >> 16));
+            r.x[2] = (ACC)Fp16::to_float((u16)(v.y & 0xffffu));
+            r.x[3] = (ACC)Fp16::to_float((u16)(v.y >> 16));
+            break;
+        }
+        default: {
+            const u32x2 v = *reinterpret_cast<const u32x2 *>(static_cast<const u16 *>(base) + idx);
+            r.x[0] = (ACC)Bf16::to_float((u16)(v.x & 0xffffu));
+            r.x[1] = (ACC)Bf16::to_float((u16)(v.x >> 16));
+            r.x[2] = (ACC)Bf16::to_float((u16)(v.y & 0xffffu));
+            r.x[3] = (ACC)Bf16::to_float((u16)(v.y >> 16));
+            break;
+        }
+    }
+    return r;
+}
+
+template <class ACC>
+__device__ __forceinline__ void store4(void *base, int dtype, size_t idx, const Vec4<ACC> &v) {
+    switch (dtype) {
+        case COTT_F32: {
+            f32x4 o = {(float)v.x[0], (float)v.x[1], (float)v.x[2], (float)v.x[3]};
+            *reinterpret_cast<f32x4 *>(static_cast<float *>(base) + idx) = o;
+            break;
+        }
+        case COTT_F64: {
+            double *p = static_cast<double *>(base) + idx;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[i] = (double)v.x[i];
+            break;
+        }
+        case COTT_F16: {
+            u32x2 o = {Fp16::pack2((float)v.x[0], (float)v.x[1]), Fp16::pack2((float)v.x[2], (float)v.x[3])};
+            *reinterpret_cast<u32x2 *>(static_cast<u16 *>(base) + idx) = o;
+            break;
+        }
+        default: {
+            u32x2 o = {Bf16::pack2((float)v.x[0], (float)v.x[1]), Bf16::pack2((float)v.x[2], (float)v.x[3])};
+            *reinterpret_cast<u32x2 *>(static_cast<u16 *>(base) + idx) = o;
+            break;
+        }
+    }
+}
+
+// Sum over the `lpr` (power of two, <= 64) consecutive lanes that hold one row.
+template <class ACC>
+__device__ __forceinline__ ACC row_sum(ACC v, int lpr) {
+    for (int off = 1; off < lpr; off <<= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+struct PrepArgs {
+    const void *x[3];    // q, k, v as given
+    const void *g[3];    // backward: gradients with respect to the prepared tensors
+    void *y[3];          // forward: prepared tensors; backward: gradients with respect to q, k, v
+    const uint8_t *keep; // (B,N) 0/1 or null
+    const float *cnt;    // (B,N) or null
+    const float *sig;    // (H) or null
+    float *dsig_rows;    // backward: (B,H,N) per-row derivative with respect to sig[h], or null
+    long rows;           // B*H*N
+    int H, N, dk, dv;
+    int x_dtype, y_dtype, g_dtype;
+    int lpr[3];          // lanes per row of q, k, v
+    float eps;
+};
+
+__device__ __forceinline__ float pow_pos(float c, float s) { return c > 0.f ? expf(s * logf(c)) : 0.f; }
+__device__ __forceinline__ double pow_pos(double c, double s) { return c > 0.0 ? exp(s * log(c)) : 0.0; }
+
+// blockIdx.y selects the tensor (0 q, 1 k, 2 v).  A row of D elements lives in lpr consecutive
+// lanes, 4 elements per lane and group; groups c = 0..NV-1 cover D up to 4*64*NV.  Each lane group
+// handles R rows (row, row + stride, ...) whose loads are all issued before the first use, so that
+// enough bytes are in flight per wavefront to cover the memory latency.
+template <class ACC, bool BACKWARD, int NV, int R>
+__global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
+    const int t = blockIdx.y;
+    const int D = t < 2 ? a.dk : a.dv;
+    const int lpr = a.lpr[t];
+    const int rpb = kPrepThreads / lpr;
+    const long row0 = ((long)blockIdx.x * R) * rpb + threadIdx.x / lpr;
+    const int lane = threadIdx.x % lpr;
+
+    Vec4<ACC> x[R][NV], g[R][NV];
+    long rr[R];
+    bool act[R];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const long row = row0 + (long)u * rpb;
+        act[u] = row < a.rows;
+        rr[u] = act[u] ? row : 0;
+#pragma unroll
+        for (int c = 0; c < NV; ++c) {
+            const int col = 4 * (lane + c * lpr);
+            if (act[u] && col < D) {
+                x[u][c] = load4<ACC>(a.x[t], a.x_dtype, (size_t)rr[u] * D + col);
+                if (BACKWARD) g[u][c] = load4<ACC>(a.g[t], a.g_dtype, (size_t)rr[u] * D + col);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    x[u][c].x[i] = 0;
+                    if (BACKWARD) g[u][c].x[i] = 0;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const long r = rr[u];
+        const int s = (int)(r % a.N);
+        const long bh = r / a.N;
+        const int h = (int)(bh % a.H);
+        const long b = bh / a.H;
+        const ACC keep = (a.keep == nullptr || a.keep[b * a.N + s] != 0) ? (ACC)1 : (ACC)0;
+        ACC ss = 0, dot = 0;
+#pragma unroll
+        for (int c = 0; c < NV; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                ss += x[u][c].x[i] * x[u][c].x[i];
+                if (BACKWARD) dot += x[u][c].x[i] * g[u][c].x[i];
+            }
+        ACC mul_x = 0, mul_g = 0;  // y = mul_x * x (forward);  dx = mul_g * g + mul_x * x (backward)
+        if (t < 2) {
+            ss = row_sum(ss, lpr);
+            const ACC nrm = sqrt(ss);
+            const ACC den = nrm > (ACC)a.eps ? nrm : (ACC)a.eps;
+            if (!BACKWARD) {
+                mul_x = keep / den;
+            } else {
+                dot = row_sum(dot, lpr);
+                mul_g = keep / den;
+                // d/dx of x / max(|x|, eps): the norm term only exists where the norm is not clamped
+                mul_x = nrm > (ACC)a.eps ? -keep * dot / (nrm * nrm * nrm) : (ACC)0;
+            }
+        } else {
+            ACC scale = 1;
+            bool scaled = false;
+            ACC c = 0;
+            if (a.cnt != nullptr && a.sig != nullptr) {
+                c = (ACC)a.cnt[b * a.N + s];
+                const ACC p = pow_pos(c, (ACC)a.sig[h]);
+                if (p > (ACC)1) {
+                    scale = (ACC)1 / p;
+                    scaled = true;
+                }
+            }
+            if (!BACKWARD) {
+                mul_x = keep * scale;
+            } else {
+                mul_g = keep * scale;
+                if (a.dsig_rows != nullptr) {
+                    // y = x c^-sig  ->  dy/dsig = -ln(c) y ; zero where the scale is clamped to 1
+                    dot = row_sum(dot, lpr);
+                    if (act[u] && lane == 0) a.dsig_rows[r] = scaled ? (float)(-log(c) * keep * scale * dot) : 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NV; ++c) {
+            const int col = 4 * (lane + c * lpr);
+            if (act[u] && col < D) {
+                Vec4<ACC> y;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    y.x[i] = BACKWARD ? mul_g * g[u][c].x[i] + mul_x * x[u][c].x[i] : mul_x * x[u][c].x[i];
+                store4<ACC>(a.y[t], BACKWARD ? a.x_dtype : a.y_dtype, (size_t)r * D + col, y);
+            }
+        }
+    }
+}
+
+int lanes_per_row(int d) {
+    int l = 1;
+    while (4 * l < d && l < 64) l <<= 1;
+    return l;
+}
+
+}  // namespace
+
+hipError_t launch_prep(bool backward, const void *const x[3], const void *const g[3], void *const y[3],
+                       const uint8_t *keep, const float *cnt, const float *sig, float *dsig_rows, int B, int H, int N,
+                       int dk, int dv, int x_dtype, int y_dtype, int g_dtype, float eps, hipStream_t stream) {
+    PrepArgs a;
+    for (int i = 0; i < 3; ++i) {
+        a.x[i] = x[i];
+        a.g[i] = g ? g[i] : nullptr;
+        a.y[i] = y[i];
+    }
+    a.keep = keep;
+    a.cnt = cnt;
+    a.sig = sig;
+    a.dsig_rows = dsig_rows;
+    a.rows = (long)B * H * N;
+    a.H = H;
+    a.N = N;
+    a.dk = dk;
+    a.dv = dv;
+    a.x_dtype = x_dtype;
+    a.y_dtype = y_dtype;
+    a.g_dtype = g_dtype;
+    a.lpr[0] = a.lpr[1] = lanes_per_row(dk);
+    a.lpr[2] = lanes_per_row(dv);
+    a.eps = eps;
+    // one grid for the three tensors; rows per block differ per tensor, size x for the largest need
+    const int big = dk > dv ? dk : dv;
+    const bool wide = big > 256;              // more than one element group per lane
+    const int R = wide ? 1 : 4;
+    const int min_rows = R * kPrepThreads / (a.lpr[0] > a.lpr[2] ? a.lpr[0] : a.lpr[2]);
+    const long blocks = (a.rows + min_rows - 1) / min_rows;
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    ProfScope prof(K_PREP, stream);
+    const dim3 grid((unsigned)blocks, 3), blk(kPrepThreads);
+    const bool f64 = x_dtype == COTT_F64;
+#define COTT_PREP(ACC, BWD) \
+    do { \
+        if (wide) prep_kernel<ACC, BWD, kMaxVec, 1><<<grid, blk, 0, stream>>>(a); \
+        else prep_kernel<ACC, BWD, 1, 4><<<grid, blk, 0, stream>>>(a); \
+    } while (0)
+    if (backward) {
+        if (f64) COTT_PREP(double, true);
+        else COTT_PREP(float, true);
+    } else {
+        if (f64) COTT_PREP(double, false);
+        else COTT_PREP(float, false);
+    }
+#undef COTT_PREP
+    return hipGetLastError();
+}
+
+}  // namespace cott

@@ -192,3 +192,70 @@ def decode_step(state, q, k, v, out=None):
                                 dv, code, _stream())
     _check(rc, "cott_decode_step")
     return out
+
+
+def _prep_side_inputs(b, h, n, keep, cnt, sig, device):
+    if keep is not None:
+        if keep.shape != (b, n):
+            raise RuntimeError(f"keep must have shape {(b, n)}, got {tuple(keep.shape)}")
+        keep = keep.to(device=device, dtype=torch.uint8).contiguous()
+    if (cnt is None) != (sig is None):
+        raise RuntimeError("cnt and sig are given together (or neither)")
+    if cnt is not None:
+        if cnt.shape != (b, n) or sig.shape != (h,):
+            raise RuntimeError(f"cnt must have shape {(b, n)} and sig {(h,)}")
+        cnt = cnt.to(device=device, dtype=torch.float32).contiguous()
+        sig = sig.detach().to(device=device, dtype=torch.float32).contiguous()
+    return keep, cnt, sig
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None):
+    """Fused input preparation of the cosine-attention module, one pass per tensor:
+        q_out = keep * q / max(|q|, 1e-12),  k_out likewise,  v_out = keep * v / max(cnt ** sig[h], 1)
+    converted to `out_dtype` (default: the input dtype).  Replaces GPT_Trainer/GPTCosAttention.py:216-241
+    and BERT_Trainer/BertCosAttention.py:162-178.  keep: (B,N) bool/0-1, True = real token; cnt: (B,N) number of
+    kept keys each position attends to; sig: (H,) = sigmoid(norm_const)."""
+    _require_gpu(Q=q, K=k, V=v)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("Q, K and V must have the same dtype")
+    code = _dtype_code(q)
+    out_dtype = out_dtype or q.dtype
+    if out_dtype not in _DTYPES:
+        raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
+    keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    qo, ko, vo = (torch.empty(t.shape, dtype=out_dtype, device=t.device) for t in (q, k, v))
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        rc = L.cott_prep_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), qo.data_ptr(), ko.data_ptr(), vo.data_ptr(),
+                             _ptr(keep), _ptr(cnt), _ptr(sig), b, h, n, dk, dv, code, _DTYPES[out_dtype], _stream())
+    _check(rc, "cott_prep_fwd")
+    return qo, ko, vo
+
+
+def prepare_inputs_backward(q, k, v, gq, gk, gv, keep=None, cnt=None, sig=None, want_dsig=False):
+    """Gradients of `prepare_inputs` with respect to q, k, v (in their dtype) and, if asked, to sig (H,)."""
+    _require_gpu(Q=q, K=k, V=v, gq=gq, gk=gk, gv=gv)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if gq.shape != q.shape or gk.shape != k.shape or gv.shape != v.shape:
+        raise RuntimeError("gradient shapes must match q, k, v")
+    if not (q.dtype == k.dtype == v.dtype) or not (gq.dtype == gk.dtype == gv.dtype):
+        raise RuntimeError("q, k, v share one dtype and their gradients share one dtype")
+    code, gcode = _dtype_code(q), _dtype_code(gq)
+    keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
+    q, k, v, gq, gk, gv = (t.contiguous() for t in (q, k, v, gq, gk, gv))
+    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    rows = torch.empty((b, h, n), dtype=torch.float32, device=q.device) if (want_dsig and sig is not None) else None
+    L = _loader.lib()
+    with torch.cuda.device(q.device):
+        rc = L.cott_prep_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
+                             dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), _ptr(rows), _ptr(keep), _ptr(cnt), _ptr(sig),
+                             b, h, n, dk, dv, code, gcode, _stream())
+    _check(rc, "cott_prep_bwd")
+    dsig = rows.sum(dim=(0, 2)) if rows is not None else None
+    return dq, dk_, dv_, dsig

@@ -106,13 +106,33 @@ COTT_API int cott_noncausal_bwd(const void *q, const void *k, const void *v, con
 COTT_API int cott_decode_step(void *state, const void *q, const void *k, const void *v, void *o,
                      int B, int H, int Dk, int Dv, int dtype, void *stream);
 
+/* ---- fused input preparation (the elementwise work the module does before the attention op) --
+ *   q_out = keep * q / max(|q|_2, 1e-12)     (rows of Dk; same for k)
+ *   v_out = keep * v / max(cnt^sig[h], 1)    (rows of Dv)
+ * in one pass per tensor, converting in_dtype -> out_dtype on the way.  Replaces the eight
+ * elementwise / reduction kernels of GPT_Trainer/GPTCosAttention.py:216-241 (normalize :216-217,
+ * value scaling :222-228, mask multiplies :232-235) and BERT_Trainer/BertCosAttention.py:162-178
+ * (for a 0/1 mask the order mask/normalise/scale does not matter).
+ * keep: (B,N) bytes, 0 = padded position, or NULL.  cnt: (B,N) fp32, the number of kept keys a
+ * position attends to (GPT: running count, :228; BERT: the total, :178) and sig: (H) fp32 =
+ * sigmoid(norm_const); both NULL = no value scaling.  fp64 converts only to fp64.
+ * cott_prep_bwd: gq,gk,gv = gradients wrt the outputs (grad_dtype); dq,dk,dv = gradients wrt the
+ * inputs (in_dtype); dsig_rows (B,H,N) fp32 or NULL receives per-row d/dsig[h] (sum it over B,N). */
+COTT_API int cott_prep_fwd(const void *q, const void *k, const void *v, void *q_out, void *k_out, void *v_out,
+                  const unsigned char *keep, const float *cnt, const float *sig,
+                  int B, int H, int N, int Dk, int Dv, int in_dtype, int out_dtype, void *stream);
+COTT_API int cott_prep_bwd(const void *q, const void *k, const void *v,
+                  const void *gq, const void *gk, const void *gv, void *dq, void *dk, void *dv,
+                  float *dsig_rows, const unsigned char *keep, const float *cnt, const float *sig,
+                  int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream);
+
 /* ---- per-kernel timing -----------------------------------------------------------------------
  * While enabled, every kernel launch made by the entry points above is bracketed by a pair of HIP
  * events on the launch stream (this is the one place the library creates HIP objects).
  * cott_profile_read() waits for the recorded launches of one kernel family, returns their summed
  * duration and count, and forgets them.  Kernel ids: 0 group_state, 1 state_prefix, 2 causal scan
  * (forward launch), 3 non-causal apply, 4 causal scan (the launch that computes dQ, dK and dV together),
- * 5 generic scan, 6 decode.  Stands where the reference wraps
+ * 5 generic scan, 6 decode, 7 input preparation.  Stands where the reference wraps
  * its kernel call in torch.autograd.profiler (Cuda_Kernel/Custom_Kernel.py:165-179). */
 COTT_API int cott_profile_enable(int on);
 COTT_API int cott_profile_read(int kernel_id, double *total_ms, long *launches);

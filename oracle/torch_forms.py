@@ -66,3 +66,38 @@ def synthetic_inputs(shape_qk, dv=None, seed=0, dtype=torch.float32, with_grad_o
     if with_grad_out:
         out.append(torch.randn(b, h, n, dv, generator=gen).to(dtype))
     return out
+
+
+def input_prep_gpt(q, k, v, keep=None, sig=None):
+    """CPU statement of the module-side preparation in front of the causal op, in the reference's order
+    (GPT_Trainer/GPTCosAttention.py:216-235): L2-normalise q and k (:216-217); divide v by
+    clamp(cnt ** sig, min=1) with cnt[b,s] = number of kept keys at positions <= s (:228, causal mask times
+    padding mask, summed over keys); multiply q, k, v by the keep mask (:232-235).
+    q,k: (B,H,N,Dk), v: (B,H,N,Dv), keep: (B,N) bool (True = real token) or None, sig: (H,) or None.
+    Returns (q_hat, k_hat, v_scaled, cnt)."""
+    b, h, n, _ = q.shape
+    km = torch.ones(b, n, dtype=torch.bool) if keep is None else keep.bool()
+    qh = torch.nn.functional.normalize(q, dim=-1, p=2)
+    kh = torch.nn.functional.normalize(k, dim=-1, p=2)
+    causal = torch.tril(torch.ones(n, n, dtype=q.dtype))                       # [s, t] = 1 for t <= s
+    cnt = (causal[None, None] * km[:, None, None, :].to(q.dtype)).sum(-1, keepdim=True)   # (B,1,N,1)
+    vs = v
+    if sig is not None:
+        vs = v / (cnt ** sig.reshape(1, h, 1, 1)).clamp(min=1)
+    m = km[:, None, :, None].to(q.dtype)
+    return qh * m, kh * m, vs * m, cnt.reshape(b, n)
+
+
+def input_prep_bert(q, k, v, keep=None, sig=None):
+    """Same for the non-causal module, in ITS order (BERT_Trainer/BertCosAttention.py:162-178): mask first
+    (:164-167), normalise (:171-172), divide v by clamp(total_kept ** sig, min=1) (:178)."""
+    b, h, n, _ = q.shape
+    km = torch.ones(b, n, dtype=torch.bool) if keep is None else keep.bool()
+    m = km[:, None, :, None].to(q.dtype)
+    qh = torch.nn.functional.normalize(q * m, dim=-1, p=2)
+    kh = torch.nn.functional.normalize(k * m, dim=-1, p=2)
+    cnt = km.sum(-1).to(q.dtype).reshape(b, 1, 1, 1)
+    vs = v * m
+    if sig is not None:
+        vs = vs / (cnt ** sig.reshape(1, h, 1, 1)).clamp(min=1)
+    return qh, kh, vs, cnt.reshape(b, 1).expand(b, n).contiguous()

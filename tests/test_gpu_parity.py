@@ -303,3 +303,84 @@ def test_headline_shape_properties(ct, oracle):
     # linearity in V (exact in exact arithmetic; bf16 output rounding bounds the defect)
     out2 = ct.causal_dot_product(qd, kd, (2 * vd))
     assert rel_l2(out2, (2 * out).double().cpu().numpy()) <= 1e-2
+
+
+PREP_CASES = [
+    # b, h, n, dk, dv, in dtype, out dtype, masked
+    (2, 3, 200, 64, 64, F32, BF, True),     # the autocast module: fp32 projections in, bf16 operands out
+    (2, 3, 200, 64, 64, F32, F32, True),
+    (1, 2, 63, 128, 128, F64, F64, True),
+    (2, 2, 257, 48, 80, BF, BF, True),      # rows that do not fill a power-of-two lane group
+    (1, 2, 130, 32, 128, HF, HF, False),
+    (1, 1, 70, 256, 40, F32, HF, True),
+    (1, 2, 33, 1024, 512, F32, F32, True),  # several element groups per lane
+    (8, 16, 256, 64, 64, F32, BF, False),
+]
+
+
+@pytest.mark.parametrize("case", PREP_CASES,
+                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1] + "-" + str(c[6]).split(".")[-1])
+def test_fused_input_preparation_forward_and_backward(ct, case):
+    # GPT_Trainer/GPTCosAttention.py:216-235 and BERT_Trainer/BertCosAttention.py:162-178 against their CPU statement
+    # (oracle/torch_forms.py, pinned by loops in tests/test_oracle_pinning.py), gradients by torch.autograd in fp64.
+    from oracle import torch_forms as tf
+    b, h, n, dk, dv, dt_in, dt_out, masked = case
+    say("prep", case)
+    g = torch.Generator().manual_seed(n + dk)
+    q, k = (torch.randn(b, h, n, dk, generator=g).to(dt_in) for _ in range(2))
+    v = torch.randn(b, h, n, dv, generator=g).to(dt_in)
+    q[0, 0, 1] = 0                                             # a zero row: norm clamp, gradient passes as g / eps
+    keep = (torch.rand(b, n, generator=g) > 0.2) if masked else None
+    sig = torch.sigmoid(torch.randn(h, generator=g)).double()
+    q64, k64, v64 = (t.clone().double().requires_grad_(True) for t in (q, k, v))
+    sig64 = sig.clone().requires_grad_(True)
+    for form in (tf.input_prep_gpt, tf.input_prep_bert):
+        rq, rk, rv, cnt = form(q64, k64, v64, keep, sig64)
+        oq, ok, ov = ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), None if keep is None else keep.to(DEV),
+                                       cnt.float().to(DEV), sig.float().to(DEV), out_dtype=dt_out)
+        assert oq.dtype == dt_out and ov.shape == v.shape
+        for got, ref in ((oq, rq), (ok, rk), (ov, rv)):
+            assert rel_l2(got, ref.detach().numpy()) <= TOL[dt_out]
+        if keep is not None:
+            assert torch.all(oq[~keep.to(DEV)[:, None, :].expand(b, h, n)] == 0)
+        # backward: upstream gradients in the output dtype
+        gq, gk = (torch.randn(b, h, n, dk, generator=g).to(dt_out) for _ in range(2))
+        gv = torch.randn(b, h, n, dv, generator=g).to(dt_out)
+        gq[0, 0, 1] = 0                                        # keeps the g / eps term of the zero row finite
+        grads = torch.autograd.grad([rq, rk, rv], [q64, k64, v64, sig64], [gq.double(), gk.double(), gv.double()])
+        dq, dk_, dv_, dsig = ct.prepare_inputs_backward(q.to(DEV), k.to(DEV), v.to(DEV), gq.to(DEV), gk.to(DEV), gv.to(DEV),
+                                                        None if keep is None else keep.to(DEV), cnt.float().to(DEV),
+                                                        sig.float().to(DEV), want_dsig=True)
+        assert dq.dtype == dt_in
+        tol_in = max(TOL[dt_in], TOL[dt_out])
+        for got, ref in ((dq, grads[0]), (dk_, grads[1]), (dv_, grads[2])):
+            assert rel_l2(got, ref.numpy()) <= tol_in
+        assert rel_l2(dsig, grads[3].numpy()) <= max(tol_in, 1e-4)
+    # no value scaling: cnt and sig omitted
+    oq, ok, ov = ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), out_dtype=dt_out)
+    assert rel_l2(ov, v.double().numpy()) <= TOL[dt_out]
+
+
+def test_prepare_inputs_autograd_function_feeds_attention(ct, oracle):
+    # module-shaped use: fp32 projections -> fused prep (bf16 out) -> causal op, gradients back to q, k, v, norm_const
+    from oracle import torch_forms as tf
+    b, h, n, d = 2, 4, 192, 64
+    g = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(b, h, n, d, generator=g) for _ in range(3))
+    keep = torch.rand(b, n, generator=g) > 0.1
+    norm_const = torch.randn(h, generator=g)
+    go = torch.randn(b, h, n, d, generator=g)
+    # CPU reference in fp64
+    q64, k64, v64, c64 = (t.double().requires_grad_(True) for t in (q, k, v, norm_const))
+    rq, rk, rv, cnt = tf.input_prep_gpt(q64, k64, v64, keep, torch.sigmoid(c64))
+    ro = tf.causal_cumsum(rq, rk, rv)
+    ref_grads = torch.autograd.grad(ro, [q64, k64, v64, c64], go.double())
+    # HIP path
+    qd, kd, vd, cd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, norm_const))
+    oq, ok, ov = ct.PrepareInputs.apply(qd, kd, vd, keep.to(DEV), cnt.float().to(DEV), torch.sigmoid(cd), torch.bfloat16)
+    out = ct.CustomAttention.apply(oq, ok, ov)
+    assert rel_l2(out, ro.detach().numpy()) <= 2e-2
+    out.backward(go.to(DEV).to(out.dtype))
+    for got, ref in zip((qd.grad, kd.grad, vd.grad, cd.grad), ref_grads):
+        assert got.dtype == torch.float32
+        assert rel_l2(got, ref.numpy()) <= 2e-2

@@ -183,3 +183,35 @@ def test_linearity_in_each_operand(oracle):
     A, B, C, A2 = rnd(1, 9, 4, seed=1), rnd(1, 9, 4, seed=2), rnd(1, 9, 5, seed=3), rnd(1, 9, 4, seed=4)
     assert np.allclose(oracle.causal(A + 2 * A2, B, C), oracle.causal(A, B, C) + 2 * oracle.causal(A2, B, C))
     assert np.allclose(oracle.causal(A, B + 2 * A2, C), oracle.causal(A, B, C) + 2 * oracle.causal(A, A2, C))
+
+
+def test_input_prep_forms_against_hand_written_loops():
+    # The CPU statement of the module-side preparation (oracle/torch_forms.py) against plain loops written here,
+    # on an input with padded positions, a zero row (norm clamp) and counts on both sides of the clamp at 1.
+    b, h, n, dk, dv = 2, 3, 7, 4, 5
+    g = torch.Generator().manual_seed(5)
+    q, k = torch.randn(b, h, n, dk, generator=g, dtype=torch.float64), torch.randn(b, h, n, dk, generator=g, dtype=torch.float64)
+    v = torch.randn(b, h, n, dv, generator=g, dtype=torch.float64)
+    q[0, 1, 2] = 0.0
+    keep = torch.tensor([[1, 1, 0, 1, 1, 0, 1], [0, 1, 1, 1, 1, 1, 1]], dtype=torch.bool)
+    sig = torch.tensor([0.3, 0.5, 0.9], dtype=torch.float64)
+    qh, kh, vs, cnt = tf.input_prep_gpt(q, k, v, keep, sig)
+    for bi in range(b):
+        run = 0
+        for s in range(n):
+            run += int(keep[bi, s])
+            assert cnt[bi, s] == run
+            for hi in range(h):
+                for x, xh in ((q, qh), (k, kh)):
+                    nrm = float(np.sqrt(sum(float(e) ** 2 for e in x[bi, hi, s])))
+                    want = [float(e) / max(nrm, 1e-12) * int(keep[bi, s]) for e in x[bi, hi, s]]
+                    assert np.allclose(xh[bi, hi, s].numpy(), want, rtol=1e-13, atol=0)
+                scale = max(run ** float(sig[hi]), 1.0)
+                want = [float(e) / scale * int(keep[bi, s]) for e in v[bi, hi, s]]
+                assert np.allclose(vs[bi, hi, s].numpy(), want, rtol=1e-13, atol=0)
+    # the non-causal module masks first and uses the total count; for 0/1 masks only the count differs
+    qb, kb, vb, cntb = tf.input_prep_bert(q, k, v, keep, sig)
+    assert torch.equal(qb, qh) and torch.equal(kb, kh)
+    assert torch.equal(cntb, keep.sum(-1, keepdim=True).expand(b, n).to(torch.float64))
+    tot = keep.sum(-1).to(torch.float64).reshape(b, 1, 1, 1)
+    assert torch.allclose(vb, v * keep[:, None, :, None] / (tot ** sig.reshape(1, h, 1, 1)).clamp(min=1), rtol=1e-13, atol=0)
