@@ -101,3 +101,88 @@ def input_prep_bert(q, k, v, keep=None, sig=None):
     if sig is not None:
         vs = vs / (cnt ** sig.reshape(1, h, 1, 1)).clamp(min=1)
     return qh, kh, vs, cnt.reshape(b, 1).expand(b, n).contiguous()
+
+
+# ---- module level: the attention blocks around the op, as the reference writes them, in plain torch -------------
+
+def gptj_sinusoid_table(num_pos, dim):
+    """GPT-J rotary table (transformers.models.gptj.modeling_gptj.create_sinusoidal_positions, imported by the
+    reference at GPT_Trainer/GPTCosAttention.py:7): columns [sin(p f_0..f_{dim/2-1}) | cos(...)], f_i = 10000^(-2i/dim)."""
+    freqs = torch.tensor([10000.0 ** (-(2 * i) / dim) for i in range(dim // 2)], dtype=torch.float32)
+    ang = torch.outer(torch.arange(num_pos, dtype=torch.float32), freqs)
+    return torch.cat((ang.sin(), ang.cos()), dim=1)
+
+
+def gptj_rotate(x, sin, cos):
+    """apply_rotary_pos_emb of GPT-J: x*cos + rotate_every_two(x)*sin with sin/cos repeated pairwise.
+    x: (B,S,H,R); sin, cos: (B,S,R/2)."""
+    sin = torch.repeat_interleave(sin[:, :, None, :], 2, 3)
+    cos = torch.repeat_interleave(cos[:, :, None, :], 2, 3)
+    rot = torch.stack((-x[..., 1::2], x[..., ::2]), dim=-1).flatten(-2)
+    return x * cos + rot * sin
+
+
+def _gpt_qkv(hidden, wq, wk, wv, num_heads, rotary_dim, max_pos, position_ids):
+    b, s, e = hidden.shape
+    d = e // num_heads
+    q = (hidden @ wq.T).view(b, s, num_heads, d)
+    k = (hidden @ wk.T).view(b, s, num_heads, d)
+    v = (hidden @ wv.T).view(b, s, num_heads, d).permute(0, 2, 1, 3)
+    table = gptj_sinusoid_table(max_pos, rotary_dim or e).to(hidden.dtype)
+    sincos = table[position_ids]
+    sin, cos = torch.split(sincos, sincos.shape[-1] // 2, dim=-1)
+    if rotary_dim is not None:
+        k = torch.cat([gptj_rotate(k[..., :rotary_dim], sin, cos), k[..., rotary_dim:]], dim=-1)
+        q = torch.cat([gptj_rotate(q[..., :rotary_dim], sin, cos), q[..., rotary_dim:]], dim=-1)
+    else:
+        k, q = gptj_rotate(k, sin, cos), gptj_rotate(q, sin, cos)
+    return q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v
+
+
+def gpt_attention_block(hidden, wq, wk, wv, wo, norm_const, num_heads, rotary_dim, max_pos, keep=None, position_ids=None):
+    """Training/evaluation path of the GPT block (GPT_Trainer/GPTCosAttention.py:429-506 with _cos_attn :200-282):
+    projections, rotary, input preparation, causal cosine attention, merge heads, output projection.
+    hidden: (B,S,E); weights as nn.Linear stores them; norm_const: (H,); keep: (B,S) bool."""
+    b, s, e = hidden.shape
+    if position_ids is None:
+        position_ids = torch.arange(s)[None, :].expand(b, s)
+    q, k, v = _gpt_qkv(hidden, wq, wk, wv, num_heads, rotary_dim, max_pos, position_ids)
+    qh, kh, vs, _ = input_prep_gpt(q, k, v, keep, torch.sigmoid(norm_const))
+    out = causal_cumsum(qh, kh, vs)
+    return out.permute(0, 2, 1, 3).reshape(b, s, e) @ wo.T
+
+
+def gpt_attention_block_recurrent(hidden, wq, wk, wv, wo, norm_const, num_heads, rotary_dim, max_pos, state, cur_s,
+                                  keep=None, position_ids=None):
+    """Recurrent-inference path (:222-223 value scaling by absolute position, :253-272 per-token loop).
+    state: (B,H,Dv,Dk) as the reference keeps it (sum of v (x) k); returns (output, state, cur_s)."""
+    b, s, e = hidden.shape
+    if position_ids is None:
+        position_ids = torch.arange(cur_s - 1, cur_s - 1 + s)[None, :].expand(b, s)
+    q, k, v = _gpt_qkv(hidden, wq, wk, wv, num_heads, rotary_dim, max_pos, position_ids)
+    q = torch.nn.functional.normalize(q, dim=-1, p=2)
+    k = torch.nn.functional.normalize(k, dim=-1, p=2)
+    pos = (cur_s + torch.arange(s)).reshape(1, 1, -1, 1).to(hidden.dtype)
+    v = v / (pos ** torch.sigmoid(norm_const).reshape(1, num_heads, 1, 1)).clamp(min=1)
+    if keep is not None:
+        m = keep[:, None, :, None].to(hidden.dtype)
+        q, k, v = q * m, k * m, v * m
+    out = torch.zeros_like(v)
+    for t in range(s):
+        state = state + v[:, :, t].unsqueeze(-1) * k[:, :, t].unsqueeze(-2)
+        out[:, :, t] = (q[:, :, t].unsqueeze(-2) * state).sum(-1)
+        cur_s += 1
+    return out.permute(0, 2, 1, 3).reshape(b, s, e) @ wo.T, state, cur_s
+
+
+def bert_attention_block(hidden, wq, bq, wk, bk, wv, bv, norm_const, num_heads, keep=None):
+    """BERT self-attention block (BERT_Trainer/BertCosAttention.py:104-334): projections with bias, mask, normalise,
+    value scaling by the number of real tokens, Q (K^T V), merge heads."""
+    b, s, e = hidden.shape
+    d = e // num_heads
+
+    def heads(x):
+        return x.view(b, s, num_heads, d).permute(0, 2, 1, 3)
+    q, k, v = heads(hidden @ wq.T + bq), heads(hidden @ wk.T + bk), heads(hidden @ wv.T + bv)
+    qh, kh, vs, _ = input_prep_bert(q, k, v, keep, torch.sigmoid(norm_const))
+    return noncausal_einsum(qh, kh, vs).permute(0, 2, 1, 3).reshape(b, s, e)

@@ -1,0 +1,133 @@
+"""GPU parity of the module-level drop-ins (cottention_transformer_amd/modules.py) against the CPU statements of the
+reference's attention blocks (oracle/torch_forms.py) with identical weights and inputs."""
+import os
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from util import rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def mods():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from cottention_transformer_amd import _loader, modules
+    assert os.path.exists(_loader.lib_path()), "libcottention_hip.so must be prebuilt in-tree"
+    _loader.lib()
+    return modules
+
+
+def gpt_cfg(e=256, heads=4, rot=32, max_pos=512, fast=False):
+    return SimpleNamespace(max_position_embeddings=max_pos, attn_pdrop=0.0, resid_pdrop=0.0, hidden_size=e,
+                           num_attention_heads=heads, rotary_dim=rot, fast_inference=fast)
+
+
+def additive_mask(keep):
+    # what the surrounding HF model hands to the block: 0 at real tokens, a large negative number at padding
+    return ((~keep).float() * torch.finfo(torch.float32).min)[:, None, None, :]
+
+
+def gpt_reference(tf, m, hidden, keep, **kw):
+    w = [getattr(m, n).weight.detach().double().cpu() for n in ("q_proj", "k_proj", "v_proj", "out_proj")]
+    nc = m.norm_const.detach().double().cpu().reshape(-1)
+    return w, nc
+
+
+@pytest.mark.parametrize("autocast", [False, True], ids=["fp32", "autocast-bf16"])
+def test_gpt_block_forward_backward(mods, autocast):
+    from oracle import torch_forms as tf
+    say("gpt block", autocast)
+    torch.manual_seed(0)
+    cfg = gpt_cfg()
+    m = mods.GPTCosAttention(cfg).to(DEV)
+    with torch.no_grad():
+        m.norm_const.copy_(torch.tensor([0.2, 0.5, -0.4, 1.0]).reshape(1, 4, 1, 1))
+    b, s = 2, 200
+    g = torch.Generator().manual_seed(1)
+    hidden = torch.randn(b, s, cfg.hidden_size, generator=g)
+    keep = torch.rand(b, s, generator=g) > 0.15
+    gout = torch.randn(b, s, cfg.hidden_size, generator=g)
+    # CPU reference in fp64 with the same weights
+    w = [getattr(m, n).weight.detach().double().cpu().requires_grad_(True) for n in ("q_proj", "k_proj", "v_proj", "out_proj")]
+    nc = m.norm_const.detach().double().cpu().reshape(-1).requires_grad_(True)
+    h64 = hidden.double().requires_grad_(True)
+    ref = tf.gpt_attention_block(h64, *w, nc, cfg.num_attention_heads, cfg.rotary_dim, cfg.max_position_embeddings, keep)
+    ref_grads = torch.autograd.grad(ref, [h64, *w, nc], gout.double())
+    # HIP path
+    hd = hidden.to(DEV).requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        out, present = m(hd, attention_mask=additive_mask(keep).to(DEV))
+    assert present is None and out.shape == hidden.shape
+    tol = 3e-2 if autocast else 1e-4
+    assert rel_l2(out.float(), ref.detach().numpy()) <= tol
+    out.backward(gout.to(DEV).to(out.dtype))
+    got = [hd.grad, m.q_proj.weight.grad, m.k_proj.weight.grad, m.v_proj.weight.grad, m.out_proj.weight.grad,
+           m.norm_const.grad.reshape(-1)]
+    for name, a, r in zip(("hidden", "wq", "wk", "wv", "wo", "norm_const"), got, ref_grads):
+        assert rel_l2(a.float(), r.numpy()) <= tol, name
+
+
+def test_gpt_block_recurrent_inference(mods):
+    # GPTCosAttention.py:77-87,222-223,253-272: a prompt, then single tokens, against the per-token loop on the CPU
+    from oracle import torch_forms as tf
+    say("gpt recurrent")
+    torch.manual_seed(0)
+    cfg = gpt_cfg(fast=True)
+    m = mods.GPTCosAttention(cfg).to(DEV).eval()
+    b, s, extra = 2, 70, 3
+    g = torch.Generator().manual_seed(4)
+    hidden = torch.randn(b, s + extra, cfg.hidden_size, generator=g)
+    w = [getattr(m, n).weight.detach().double().cpu() for n in ("q_proj", "k_proj", "v_proj", "out_proj")]
+    nc = m.norm_const.detach().double().cpu().reshape(-1)
+    d = cfg.hidden_size // cfg.num_attention_heads
+    state = torch.zeros(b, cfg.num_attention_heads, d, d, dtype=torch.float64)
+    ref, state, cur = tf.gpt_attention_block_recurrent(hidden.double(), *w, nc, cfg.num_attention_heads, cfg.rotary_dim,
+                                                       cfg.max_position_embeddings, state, 1)
+    with torch.no_grad():
+        outs = [m(hidden[:, :s].to(DEV))[0]]
+        for t in range(s, s + extra):
+            outs.append(m(hidden[:, t:t + 1].to(DEV))[0])
+    assert m.cur_s == cur
+    assert rel_l2(torch.cat(outs, 1), ref.numpy()) <= 1e-4
+    assert rel_l2(m.state.transpose(-1, -2), state.numpy()) <= 1e-5     # the reference keeps v (x) k
+    m.reset_state()
+    assert m.state is None and m.cur_s == 1
+
+
+@pytest.mark.parametrize("autocast", [False, True], ids=["fp32", "autocast-bf16"])
+def test_bert_block_forward_backward(mods, autocast):
+    from oracle import torch_forms as tf
+    say("bert block", autocast)
+    torch.manual_seed(0)
+    cfg = SimpleNamespace(hidden_size=256, num_attention_heads=4, attention_probs_dropout_prob=0.0, is_decoder=False)
+    m = mods.BertCosAttention(cfg).to(DEV)
+    b, s = 3, 128
+    g = torch.Generator().manual_seed(2)
+    hidden = torch.randn(b, s, cfg.hidden_size, generator=g)
+    keep = torch.arange(s)[None, :] < torch.tensor([128, 90, 17])[:, None]
+    gout = torch.randn(b, s, cfg.hidden_size, generator=g)
+    names = ("query", "key", "value")
+    w = [getattr(m, n).weight.detach().double().cpu().requires_grad_(True) for n in names]
+    bias = [getattr(m, n).bias.detach().double().cpu().requires_grad_(True) for n in names]
+    nc = m.norm_const.detach().double().cpu().reshape(-1).requires_grad_(True)
+    h64 = hidden.double().requires_grad_(True)
+    ref = tf.bert_attention_block(h64, w[0], bias[0], w[1], bias[1], w[2], bias[2], nc, cfg.num_attention_heads, keep)
+    ref_grads = torch.autograd.grad(ref, [h64, *w, nc], gout.double())
+    hd = hidden.to(DEV).requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        (out,) = m(hd, attention_mask=additive_mask(keep).to(DEV))
+    tol = 3e-2 if autocast else 1e-4
+    assert rel_l2(out.float(), ref.detach().numpy()) <= tol
+    out.backward(gout.to(DEV).to(out.dtype))
+    got = [hd.grad, m.query.weight.grad, m.key.weight.grad, m.value.weight.grad, m.norm_const.grad.reshape(-1)]
+    for name, a, r in zip(("hidden", "wq", "wk", "wv", "norm_const"), got, ref_grads):
+        assert rel_l2(a.float(), r.numpy()) <= tol, name
