@@ -238,6 +238,27 @@ def run_extras(torch, ct, dev):
     ex["input_prep_fwd_B8_H16_N2048_D64_f32_to_bf16"] = {"us": s_f * 1e6, "GBps": pb / s_f / 1e9,
                                                          "frac_hbm": pb / s_f / 1e9 / HBM_PEAK_GBS,
                                                          "torch_elementwise_us": s_e * 1e6}
+    del keep, cnt, sig
+    # whole GPT attention block (projections, rotary, preparation, attention, output projection), fwd+bwd under
+    # bf16 autocast at the GPT-300M shape; second figure: same block with rotary / head permute as torch ops
+    from types import SimpleNamespace
+    from cottention_transformer_amd import modules
+    cfg = SimpleNamespace(max_position_embeddings=2048, attn_pdrop=0.0, resid_pdrop=0.0, hidden_size=1024,
+                          num_attention_heads=16, rotary_dim=64)
+    blk = modules.GPTCosAttention(cfg).to(dev)
+    hid = torch.randn(8, 2048, 1024, device=dev, requires_grad=True)
+    gout = torch.randn(8, 2048, 1024, device=dev, dtype=torch.bfloat16)
+
+    def block_step(use_cache):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = blk(hid, use_cache=use_cache)[0]
+        out.backward(gout)
+    s_fused = time_region(torch, lambda: block_step(False), 20, 3)
+    s_torch = time_region(torch, lambda: block_step(True), 20, 3)
+    ex["gpt_block_fwd_bwd_B8_S2048_E1024_H16_autocast_bf16"] = {
+        "us": s_fused * 1e6, "tokens_per_s": 8 * 2048 / s_fused,
+        "us_with_rotary_and_permute_as_torch_ops": s_torch * 1e6}
+    del blk, hid, gout
     ex["fp32_fwd_bwd_B8_H16_N2048_D64"] = {"us": s * 1e6, "tokens_per_s": 8 * 2048 / s, "GBps": byts / s / 1e9,
                                            "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS,
                                            "executed_tflops": flops / s / 1e12,

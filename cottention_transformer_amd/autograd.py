@@ -63,22 +63,26 @@ class NonCausalAttention(torch.autograd.Function):
 
 
 class PrepareInputs(torch.autograd.Function):
-    """(q, k, v, keep, cnt, sig, out_dtype) -> (q_hat, k_hat, v_scaled): the normalise / value-scale / mask
-    steps in front of the attention op (GPT_Trainer/GPTCosAttention.py:216-241) as one fused operator with a
-    fused backward.  `sig` = sigmoid(norm_const) per head, differentiable; keep and cnt are constants."""
+    """(q, k, v, keep, cnt, sig, out_dtype[, rot_table, position_ids, bnhd]) -> (q_hat, k_hat, v_scaled), (B,H,N,D):
+    the normalise / value-scale / mask steps in front of the attention op (GPT_Trainer/GPTCosAttention.py:216-241),
+    optionally with the rotary embedding and the head permute before them (:453-475), as one fused operator with a
+    fused backward.  `sig` = sigmoid(norm_const) per head, differentiable; the other side inputs are constants."""
 
     @staticmethod
-    def forward(ctx, q, k, v, keep, cnt, sig, out_dtype):
+    def forward(ctx, q, k, v, keep, cnt, sig, out_dtype, rot_table=None, position_ids=None, bnhd=False):
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        ctx.save_for_backward(q, k, v, keep, cnt, sig)
-        return ops.prepare_inputs(q, k, v, keep, cnt, sig, out_dtype)
+        ctx.save_for_backward(q, k, v, keep, cnt, sig, rot_table, position_ids)
+        ctx.bnhd = bool(bnhd)
+        rotary = (rot_table, position_ids) if rot_table is not None else None
+        return ops.prepare_inputs(q, k, v, keep, cnt, sig, out_dtype, rotary=rotary, bnhd=bnhd)
 
     @staticmethod
     def backward(ctx, gq, gk, gv):
-        q, k, v, keep, cnt, sig = ctx.saved_tensors
+        q, k, v, keep, cnt, sig, rot_table, position_ids = ctx.saved_tensors
         want = sig is not None and ctx.needs_input_grad[5]
+        rotary = (rot_table, position_ids) if rot_table is not None else None
         dq, dk, dv, dsig = ops.prepare_inputs_backward(q, k, v, gq.contiguous(), gk.contiguous(), gv.contiguous(), keep,
-                                                       cnt, sig, want_dsig=want)
+                                                       cnt, sig, want_dsig=want, rotary=rotary, bnhd=ctx.bnhd)
         if dsig is not None:
             dsig = dsig.to(sig.dtype)
-        return dq, dk, dv, None, None, dsig, None
+        return dq, dk, dv, None, None, dsig, None, None, None, None

@@ -442,13 +442,23 @@ int check_prep(const char *fn, int B, int H, int N, int Dk, int Dv, int d0, int 
     if ((d0 == COTT_F64) != (d1 == COTT_F64)) return fail(COTT_ERR_UNSUPPORTED, "%s: fp64 only converts to fp64", fn);
     return COTT_OK;
 }
+int check_rotary(const char *fn, const float *table, const long long *pos, int R, int rows, int Dk) {
+    if (table == nullptr && pos == nullptr) return COTT_OK;
+    if (table == nullptr || pos == nullptr) return fail(COTT_ERR_INVALID, "%s: rotary table and positions go together", fn);
+    if (R < 4 || R % 4 != 0 || R > Dk)
+        return fail(COTT_ERR_INVALID, "%s: rotary_dim must be a multiple of 4 in [4, Dk] (got %d)", fn, R);
+    if (rows < 1) return fail(COTT_ERR_INVALID, "%s: empty rotary table", fn);
+    return COTT_OK;
+}
 }  // namespace
 
-int cott_prep_fwd(const void *q, const void *k, const void *v, void *q_out, void *k_out, void *v_out,
-                  const unsigned char *keep, const float *cnt, const float *sig, int B, int H, int N, int Dk, int Dv,
-                  int in_dtype, int out_dtype, void *stream) {
-    const char *fn = "cott_prep_fwd";
+int cott_prep_ex_fwd(const void *q, const void *k, const void *v, void *q_out, void *k_out, void *v_out,
+                     const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
+                     const long long *pos, int rotary_dim, int table_rows, int in_bnhd, int B, int H, int N, int Dk,
+                     int Dv, int in_dtype, int out_dtype, void *stream) {
+    const char *fn = "cott_prep_ex_fwd";
     if (int rc = check_prep(fn, B, H, N, Dk, Dv, in_dtype, out_dtype)) return rc;
+    if (int rc = check_rotary(fn, rot_table, pos, rotary_dim, table_rows, Dk)) return rc;
     if ((long)B * H * N == 0) return COTT_OK;
     if (!q || !k || !v || !q_out || !k_out || !v_out) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(q_out) || !aligned16(k_out) || !aligned16(v_out))
@@ -457,16 +467,19 @@ int cott_prep_fwd(const void *q, const void *k, const void *v, void *q_out, void
     const void *x[3] = {q, k, v};
     void *y[3] = {q_out, k_out, v_out};
     hipError_t e = cott::launch_prep(false, x, nullptr, y, keep, cnt, sig, nullptr, B, H, N, Dk, Dv, in_dtype, out_dtype,
-                                     out_dtype, 1e-12f, static_cast<hipStream_t>(stream));
+                                     out_dtype, 1e-12f, in_bnhd ? 1 : 0, rot_table, pos, rot_table ? rotary_dim : 0,
+                                     static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
     return COTT_OK;
 }
 
-int cott_prep_bwd(const void *q, const void *k, const void *v, const void *gq, const void *gk, const void *gv, void *dq,
-                  void *dk, void *dv, float *dsig_rows, const unsigned char *keep, const float *cnt, const float *sig,
-                  int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream) {
-    const char *fn = "cott_prep_bwd";
+int cott_prep_ex_bwd(const void *q, const void *k, const void *v, const void *gq, const void *gk, const void *gv,
+                     void *dq, void *dk, void *dv, float *dsig_rows, const unsigned char *keep, const float *cnt,
+                     const float *sig, const float *rot_table, const long long *pos, int rotary_dim, int table_rows,
+                     int in_bnhd, int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream) {
+    const char *fn = "cott_prep_ex_bwd";
     if (int rc = check_prep(fn, B, H, N, Dk, Dv, in_dtype, grad_dtype)) return rc;
+    if (int rc = check_rotary(fn, rot_table, pos, rotary_dim, table_rows, Dk)) return rc;
     if ((long)B * H * N == 0) return COTT_OK;
     if (!q || !k || !v || !gq || !gk || !gv || !dq || !dk || !dv) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(gq) || !aligned16(gk) || !aligned16(gv) ||
@@ -477,9 +490,24 @@ int cott_prep_bwd(const void *q, const void *k, const void *v, const void *gq, c
     const void *g[3] = {gq, gk, gv};
     void *y[3] = {dq, dk, dv};
     hipError_t e = cott::launch_prep(true, x, g, y, keep, cnt, sig, dsig_rows, B, H, N, Dk, Dv, in_dtype, in_dtype,
-                                     grad_dtype, 1e-12f, static_cast<hipStream_t>(stream));
+                                     grad_dtype, 1e-12f, in_bnhd ? 1 : 0, rot_table, pos, rot_table ? rotary_dim : 0,
+                                     static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
     return COTT_OK;
+}
+
+int cott_prep_fwd(const void *q, const void *k, const void *v, void *q_out, void *k_out, void *v_out,
+                  const unsigned char *keep, const float *cnt, const float *sig, int B, int H, int N, int Dk, int Dv,
+                  int in_dtype, int out_dtype, void *stream) {
+    return cott_prep_ex_fwd(q, k, v, q_out, k_out, v_out, keep, cnt, sig, nullptr, nullptr, 0, 0, 0, B, H, N, Dk, Dv,
+                            in_dtype, out_dtype, stream);
+}
+
+int cott_prep_bwd(const void *q, const void *k, const void *v, const void *gq, const void *gk, const void *gv, void *dq,
+                  void *dk, void *dv, float *dsig_rows, const unsigned char *keep, const float *cnt, const float *sig,
+                  int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream) {
+    return cott_prep_ex_bwd(q, k, v, gq, gk, gv, dq, dk, dv, dsig_rows, keep, cnt, sig, nullptr, nullptr, 0, 0, 0, B, H,
+                            N, Dk, Dv, in_dtype, grad_dtype, stream);
 }
 
 }  // extern "C"

@@ -102,7 +102,25 @@ struct PrepArgs {
     int x_dtype, y_dtype, g_dtype;
     int lpr[3];          // lanes per row of q, k, v
     float eps;
+    // Optional extras: q, k, v given as (B,N,H,D) (the layout the projections produce) instead of
+    // (B,H,N,D), and the GPT-J rotary embedding applied to the first R columns of q and k.
+    int x_bnhd;           // 1: x (and, backward, y) are (B,N,H,D); g (backward) / y (forward) stay (B,H,N,D)
+    const float *rot;     // (P,R) table, row p = [sin(p f_0..f_{R/2-1}) | cos(...)], or null
+    const long long *pos; // (B,N) row of the table per position
+    int R;
 };
+
+// Rotates the pairs (v[0],v[1]) and (v[2],v[3]) by +angle (inverse = false) or -angle.
+template <class ACC>
+__device__ __forceinline__ void rotate4(Vec4<ACC> &v, const float *sc, int half, bool inverse) {
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const ACC s = inverse ? -(ACC)sc[p] : (ACC)sc[p], c = (ACC)sc[half + p];
+        const ACC e = v.x[2 * p], o = v.x[2 * p + 1];
+        v.x[2 * p] = e * c - o * s;
+        v.x[2 * p + 1] = o * c + e * s;
+    }
+}
 
 __device__ __forceinline__ float pow_pos(float c, float s) { return c > 0.f ? expf(s * logf(c)) : 0.f; }
 __device__ __forceinline__ double pow_pos(double c, double s) { return c > 0.0 ? exp(s * log(c)) : 0.0; }
@@ -122,17 +140,22 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
 
     Vec4<ACC> x[R][NV], g[R][NV];
     long rr[R];
+    size_t xoff[R];
     bool act[R];
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const long row = row0 + (long)u * rpb;
         act[u] = row < a.rows;
         rr[u] = act[u] ? row : 0;
+        {
+            const long bh_ = rr[u] / a.N, s_ = rr[u] % a.N;
+            xoff[u] = a.x_bnhd ? (size_t)(((bh_ / a.H) * a.N + s_) * a.H + bh_ % a.H) * D : (size_t)rr[u] * D;
+        }
 #pragma unroll
         for (int c = 0; c < NV; ++c) {
             const int col = 4 * (lane + c * lpr);
             if (act[u] && col < D) {
-                x[u][c] = load4<ACC>(a.x[t], a.x_dtype, (size_t)rr[u] * D + col);
+                x[u][c] = load4<ACC>(a.x[t], a.x_dtype, xoff[u] + col);
                 if (BACKWARD) g[u][c] = load4<ACC>(a.g[t], a.g_dtype, (size_t)rr[u] * D + col);
             } else {
 #pragma unroll
@@ -151,6 +174,18 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
         const int h = (int)(bh % a.H);
         const long b = bh / a.H;
         const ACC keep = (a.keep == nullptr || a.keep[b * a.N + s] != 0) ? (ACC)1 : (ACC)0;
+        const bool rotary = t < 2 && a.rot != nullptr;
+        const float *sc = rotary ? a.rot + (size_t)a.pos[b * a.N + s] * a.R : nullptr;
+        // y = keep R x / |R x| with R the block rotation built from the table (orthogonal only up to the table's
+        // rounding, so the norm is taken after the rotation).  Backward: dx = R^T J^T g with J the Jacobian of
+        // the normalisation at x' = R x: the usual combination of g and x', rotated back at the end.
+        if (rotary) {
+#pragma unroll
+            for (int c = 0; c < NV; ++c) {
+                const int col = 4 * (lane + c * lpr);
+                if (col < a.R) rotate4(x[u][c], sc + col / 2, a.R / 2, false);
+            }
+        }
         ACC ss = 0, dot = 0;
 #pragma unroll
         for (int c = 0; c < NV; ++c)
@@ -203,7 +238,8 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     y.x[i] = BACKWARD ? mul_g * g[u][c].x[i] + mul_x * x[u][c].x[i] : mul_x * x[u][c].x[i];
-                store4<ACC>(a.y[t], BACKWARD ? a.x_dtype : a.y_dtype, (size_t)r * D + col, y);
+                if (BACKWARD && rotary && col < a.R) rotate4(y, sc + col / 2, a.R / 2, true);
+                store4<ACC>(a.y[t], BACKWARD ? a.x_dtype : a.y_dtype, (BACKWARD ? xoff[u] : (size_t)r * D) + col, y);
             }
         }
     }
@@ -219,8 +255,13 @@ int lanes_per_row(int d) {
 
 hipError_t launch_prep(bool backward, const void *const x[3], const void *const g[3], void *const y[3],
                        const uint8_t *keep, const float *cnt, const float *sig, float *dsig_rows, int B, int H, int N,
-                       int dk, int dv, int x_dtype, int y_dtype, int g_dtype, float eps, hipStream_t stream) {
+                       int dk, int dv, int x_dtype, int y_dtype, int g_dtype, float eps, int x_bnhd, const float *rot,
+                       const long long *pos, int R, hipStream_t stream) {
     PrepArgs a;
+    a.x_bnhd = x_bnhd;
+    a.rot = rot;
+    a.pos = pos;
+    a.R = R;
     for (int i = 0; i < 3; ++i) {
         a.x[i] = x[i];
         a.g[i] = g ? g[i] : nullptr;
@@ -244,8 +285,8 @@ hipError_t launch_prep(bool backward, const void *const x[3], const void *const 
     // one grid for the three tensors; rows per block differ per tensor, size x for the largest need
     const int big = dk > dv ? dk : dv;
     const bool wide = big > 256;              // more than one element group per lane
-    const int R = wide ? 1 : 4;
-    const int min_rows = R * kPrepThreads / (a.lpr[0] > a.lpr[2] ? a.lpr[0] : a.lpr[2]);
+    const int rows_per_group = wide ? 1 : 4;
+    const int min_rows = rows_per_group * kPrepThreads / (a.lpr[0] > a.lpr[2] ? a.lpr[0] : a.lpr[2]);
     const long blocks = (a.rows + min_rows - 1) / min_rows;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     ProfScope prof(K_PREP, stream);

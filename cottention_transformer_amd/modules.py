@@ -104,17 +104,23 @@ class GPTCosAttention(nn.Module):
             key, query = apply_rotary(key, sin, cos), apply_rotary(query, sin, cos)
         return query, key
 
-    def _cos_attn(self, query, key, value, attention_mask=None, head_mask=None):
-        """query, key, value: (B,H,S,D).  GPTCosAttention.py:200-282."""
-        b, h, s, _ = query.shape
+    def _cos_attn(self, query, key, value, attention_mask=None, head_mask=None, rotary=None, bnhd=False):
+        """GPTCosAttention.py:200-282.  query, key, value: (B,H,S,D), already rotated -- or, with `bnhd`, (B,S,H,D)
+        as the projections produce them, with rotary=(table, position_ids) still to be applied; in that case the
+        rotation, the head permute and the preparation steps are one fused pass."""
+        if bnhd:
+            b, s, h, _ = query.shape
+        else:
+            b, h, s, _ = query.shape
         query, key, value = _common_dtype(query, key, value)
         keep = _keep_from_additive_mask(attention_mask, b, s, query.device)
         sig = self.norm_const.sigmoid().reshape(h)
+        table, pos = rotary if rotary is not None else (None, None)
         if self.fast_inference:
             # value scaling by absolute position (:223), then the recurrence (:253-272) from the stored state
             cnt = (self.cur_s + torch.arange(s, device=query.device, dtype=torch.float32)).expand(b, s)
             dt = query.dtype
-            q, k, v = ops.prepare_inputs(query, key, value, keep, cnt, sig, out_dtype=dt)
+            q, k, v = ops.prepare_inputs(query, key, value, keep, cnt, sig, out_dtype=dt, rotary=rotary, bnhd=bnhd)
             if self.state is None:
                 self.state = torch.zeros(b, h, q.shape[-1], v.shape[-1], device=q.device,
                                          dtype=torch.float64 if dt == torch.float64 else torch.float32)
@@ -126,26 +132,35 @@ class GPTCosAttention(nn.Module):
             return out, out
         cnt = keep.to(torch.float32).cumsum(-1)                        # kept keys at positions <= s (:228)
         dt = _autocast_target(query)
-        q, k, v = PrepareInputs.apply(query, key, value, keep, cnt, sig, dt)
+        q, k, v = PrepareInputs.apply(query, key, value, keep, cnt, sig, dt, table, pos, bnhd)
         out = CustomAttention.apply(q, k, v)
         return out, out
 
     def forward(self, hidden_states, layer_past=None, attention_mask=None, position_ids=None, head_mask=None,
                 use_cache=False, output_attentions=False):
-        query = self._split_heads(self.q_proj(hidden_states))
+        query = self._split_heads(self.q_proj(hidden_states))          # (B,S,H,D)
         key = self._split_heads(self.k_proj(hidden_states))
-        value = self._split_heads(self.v_proj(hidden_states)).permute(0, 2, 1, 3)
+        value = self._split_heads(self.v_proj(hidden_states))
         if position_ids is None:
             start = self.cur_s - 1 if self.fast_inference else 0
             position_ids = torch.arange(start, start + hidden_states.shape[1], device=hidden_states.device)
             position_ids = position_ids[None, :].expand(hidden_states.shape[0], -1)
-        query, key = self._rotate(query, key, position_ids)
-        key, query = key.permute(0, 2, 1, 3), query.permute(0, 2, 1, 3)
-        if layer_past is not None:
-            key = torch.cat((layer_past[0], key), dim=-2)
-            value = torch.cat((layer_past[1], value), dim=-2)
-        present = (key.to(hidden_states.dtype), value) if use_cache is True else None
-        attn_output, attn_weights = self._cos_attn(query, key, value, attention_mask, head_mask)
+        if layer_past is None and use_cache is not True and self.rotary_dim is not None and self.rotary_dim % 4 == 0:
+            # nobody needs the rotated keys themselves: rotation, head permute and preparation in one pass
+            table = self.embed_positions
+            if table.device != hidden_states.device:
+                table = self.embed_positions = table.to(hidden_states.device)
+            present = None
+            attn_output, attn_weights = self._cos_attn(query, key, value, attention_mask, head_mask,
+                                                       rotary=(table, position_ids), bnhd=True)
+        else:
+            query, key = self._rotate(query, key, position_ids)
+            key, query, value = key.permute(0, 2, 1, 3), query.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3)
+            if layer_past is not None:
+                key = torch.cat((layer_past[0], key), dim=-2)
+                value = torch.cat((layer_past[1], value), dim=-2)
+            present = (key.to(hidden_states.dtype), value) if use_cache is True else None
+            attn_output, attn_weights = self._cos_attn(query, key, value, attention_mask, head_mask)
         if not _autocast_on():
             attn_output = attn_output.to(hidden_states.dtype)
         attn_output = attn_output.permute(0, 2, 1, 3).contiguous()
@@ -185,15 +200,17 @@ class BertCosAttention(nn.Module):
             raise NotImplementedError("cross-attention and cached keys are not implemented for cosine attention")
         if head_mask is not None:
             raise NotImplementedError
-        query_layer = self.transpose_for_scores(self.query(hidden_states))
-        key_layer = self.transpose_for_scores(self.key(hidden_states))
-        value_layer = self.transpose_for_scores(self.value(hidden_states))
-        b, h, s, _ = query_layer.shape
+        split = hidden_states.shape[:-1] + (self.num_attention_heads, self.attention_head_size)
+        query_layer = self.query(hidden_states).view(split)            # (B,S,H,D); the head permute of
+        key_layer = self.key(hidden_states).view(split)                # transpose_for_scores happens inside
+        value_layer = self.value(hidden_states).view(split)            # the preparation pass
+        b, s, h, _ = query_layer.shape
         # mask, normalise, divide the values by (number of real tokens) ** sigmoid(norm_const)  (:162-178)
         keep = _keep_from_additive_mask(attention_mask, b, s, query_layer.device)
         cnt = keep.sum(-1, keepdim=True).to(torch.float32).expand(b, s)
         dt = _autocast_target(query_layer)
-        q, k, v = PrepareInputs.apply(query_layer, key_layer, value_layer, keep, cnt, self.norm_const.sigmoid().reshape(h), dt)
+        q, k, v = PrepareInputs.apply(query_layer, key_layer, value_layer, keep, cnt, self.norm_const.sigmoid().reshape(h),
+                                      dt, None, None, True)
         context_layer = NonCausalAttention.apply(q, k, v)               # Q (K^T V)  (:249); (QK^T)V at :222 is the same product
         if not _autocast_on():
             context_layer = context_layer.to(hidden_states.dtype)
@@ -201,5 +218,5 @@ class BertCosAttention(nn.Module):
         context_layer = context_layer.view(context_layer.size()[:-2] + (self.all_head_size,))
         outputs = (context_layer, None) if output_attentions else (context_layer,)
         if self.is_decoder:
-            outputs = outputs + ((key_layer, value_layer),)
+            outputs = outputs + ((key_layer.permute(0, 2, 1, 3), value_layer.permute(0, 2, 1, 3)),)
         return outputs

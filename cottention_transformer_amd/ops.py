@@ -213,14 +213,43 @@ def _ptr(t):
     return t.data_ptr() if t is not None else None
 
 
-def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None):
+def _prep_shapes(q, k, v, bnhd):
+    """(b, h, n, dk, dv) of q, k, v given as (B,H,N,D), or as (B,N,H,D) when `bnhd`."""
+    if bnhd:
+        if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.shape != k.shape or q.shape[:3] != v.shape[:3]:
+            raise RuntimeError("Q, K and V must have shape (N, S, H, D) and agree in (N, S, H)")
+        b, n, h, dk = q.shape
+        return b, h, n, dk, v.size(3)
+    return _shapes(q, k, v)
+
+
+def _rotary_args(rotary, b, n, dk, device):
+    if rotary is None:
+        return None, None, 0, 0
+    table, pos = rotary
+    if table.dim() != 2 or table.size(1) % 4 != 0 or table.size(1) > dk:
+        raise RuntimeError("rotary table must be (positions, rotary_dim), rotary_dim a multiple of 4 and <= Dk")
+    if pos.shape != (b, n):
+        raise RuntimeError(f"position ids must have shape {(b, n)}")
+    if pos.numel() and (int(pos.max()) >= table.size(0) or int(pos.min()) < 0):
+        raise RuntimeError("position id outside the rotary table")
+    table = table.to(device=device, dtype=torch.float32).contiguous()
+    pos = pos.to(device=device, dtype=torch.int64).contiguous()
+    return table, pos, table.size(1), table.size(0)
+
+
+def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None, rotary=None, bnhd=False):
     """Fused input preparation of the cosine-attention module, one pass per tensor:
         q_out = keep * q / max(|q|, 1e-12),  k_out likewise,  v_out = keep * v / max(cnt ** sig[h], 1)
-    converted to `out_dtype` (default: the input dtype).  Replaces GPT_Trainer/GPTCosAttention.py:216-241
-    and BERT_Trainer/BertCosAttention.py:162-178.  keep: (B,N) bool/0-1, True = real token; cnt: (B,N) number of
-    kept keys each position attends to; sig: (H,) = sigmoid(norm_const)."""
+    converted to `out_dtype` (default: the input dtype) and returned as (B,H,N,D).  Replaces
+    GPT_Trainer/GPTCosAttention.py:216-241 and BERT_Trainer/BertCosAttention.py:162-178.
+    keep: (B,N) bool/0-1, True = real token; cnt: (B,N) number of kept keys each position attends to;
+    sig: (H,) = sigmoid(norm_const).
+    rotary=(table, position_ids): also applies the GPT-J rotary embedding to the first table.size(1) columns of
+    q and k (GPTCosAttention.py:453-472); bnhd=True: q, k, v are given as (B,N,H,D), the layout the projections
+    produce, and the head permute of :474-475 happens in the same pass."""
     _require_gpu(Q=q, K=k, V=v)
-    b, h, n, dk, dv = _shapes(q, k, v)
+    b, h, n, dk, dv = _prep_shapes(q, k, v, bnhd)
     if not (q.dtype == k.dtype == v.dtype):
         raise RuntimeError("Q, K and V must have the same dtype")
     code = _dtype_code(q)
@@ -228,34 +257,41 @@ def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None):
     if out_dtype not in _DTYPES:
         raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
     keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
+    table, pos, rdim, rows = _rotary_args(rotary, b, n, dk, q.device)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    qo, ko, vo = (torch.empty(t.shape, dtype=out_dtype, device=t.device) for t in (q, k, v))
+    qo, ko = (torch.empty((b, h, n, dk), dtype=out_dtype, device=q.device) for _ in range(2))
+    vo = torch.empty((b, h, n, dv), dtype=out_dtype, device=q.device)
     L = _loader.lib()
     with torch.cuda.device(q.device):
-        rc = L.cott_prep_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), qo.data_ptr(), ko.data_ptr(), vo.data_ptr(),
-                             _ptr(keep), _ptr(cnt), _ptr(sig), b, h, n, dk, dv, code, _DTYPES[out_dtype], _stream())
-    _check(rc, "cott_prep_fwd")
+        rc = L.cott_prep_ex_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), qo.data_ptr(), ko.data_ptr(), vo.data_ptr(),
+                                _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), _ptr(pos), rdim, rows, int(bool(bnhd)),
+                                b, h, n, dk, dv, code, _DTYPES[out_dtype], _stream())
+    _check(rc, "cott_prep_ex_fwd")
     return qo, ko, vo
 
 
-def prepare_inputs_backward(q, k, v, gq, gk, gv, keep=None, cnt=None, sig=None, want_dsig=False):
-    """Gradients of `prepare_inputs` with respect to q, k, v (in their dtype) and, if asked, to sig (H,)."""
+def prepare_inputs_backward(q, k, v, gq, gk, gv, keep=None, cnt=None, sig=None, want_dsig=False, rotary=None,
+                            bnhd=False):
+    """Gradients of `prepare_inputs` with respect to q, k, v (their dtype and layout) and, if asked, to sig (H,).
+    gq, gk, gv: gradients with respect to the outputs, (B,H,N,D)."""
     _require_gpu(Q=q, K=k, V=v, gq=gq, gk=gk, gv=gv)
-    b, h, n, dk, dv = _shapes(q, k, v)
-    if gq.shape != q.shape or gk.shape != k.shape or gv.shape != v.shape:
-        raise RuntimeError("gradient shapes must match q, k, v")
+    b, h, n, dk, dv = _prep_shapes(q, k, v, bnhd)
+    if gq.shape != (b, h, n, dk) or gk.shape != (b, h, n, dk) or gv.shape != (b, h, n, dv):
+        raise RuntimeError("gradient shapes must be (B,H,N,D)")
     if not (q.dtype == k.dtype == v.dtype) or not (gq.dtype == gk.dtype == gv.dtype):
         raise RuntimeError("q, k, v share one dtype and their gradients share one dtype")
     code, gcode = _dtype_code(q), _dtype_code(gq)
     keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
+    table, pos, rdim, rows = _rotary_args(rotary, b, n, dk, q.device)
     q, k, v, gq, gk, gv = (t.contiguous() for t in (q, k, v, gq, gk, gv))
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    rows = torch.empty((b, h, n), dtype=torch.float32, device=q.device) if (want_dsig and sig is not None) else None
+    drows = torch.empty((b, h, n), dtype=torch.float32, device=q.device) if (want_dsig and sig is not None) else None
     L = _loader.lib()
     with torch.cuda.device(q.device):
-        rc = L.cott_prep_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
-                             dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), _ptr(rows), _ptr(keep), _ptr(cnt), _ptr(sig),
-                             b, h, n, dk, dv, code, gcode, _stream())
-    _check(rc, "cott_prep_bwd")
-    dsig = rows.sum(dim=(0, 2)) if rows is not None else None
+        rc = L.cott_prep_ex_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
+                                dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), _ptr(drows), _ptr(keep), _ptr(cnt),
+                                _ptr(sig), _ptr(table), _ptr(pos), rdim, rows, int(bool(bnhd)), b, h, n, dk, dv, code,
+                                gcode, _stream())
+    _check(rc, "cott_prep_ex_bwd")
+    dsig = drows.sum(dim=(0, 2)) if drows is not None else None
     return dq, dk_, dv_, dsig

@@ -126,6 +126,23 @@ COTT_API int cott_prep_bwd(const void *q, const void *k, const void *v,
                   float *dsig_rows, const unsigned char *keep, const float *cnt, const float *sig,
                   int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream);
 
+/* The same with the two steps that surround it in the GPT block folded in (GPTCosAttention.py:434-476):
+ * in_bnhd != 0: q, k, v (and, backward, dq, dk, dv) are laid out (B,N,H,D), as the projections produce them
+ * (the outputs / incoming gradients stay (B,H,N,D)), which removes the permute + contiguous copies of :474-475 and
+ * Custom_Kernel.py:11-13;  rot_table != NULL: the GPT-J rotary embedding (apply_rotary_pos_emb, :463-472) is
+ * applied to the first rotary_dim columns of q and k before normalisation.  rot_table: (table_rows, rotary_dim)
+ * fp32, row p = [sin(p f_i) | cos(p f_i)]; pos: (B,N) int64 row index per position (must be < table_rows; not
+ * checked on the device). */
+COTT_API int cott_prep_ex_fwd(const void *q, const void *k, const void *v, void *q_out, void *k_out, void *v_out,
+                     const unsigned char *keep, const float *cnt, const float *sig,
+                     const float *rot_table, const long long *pos, int rotary_dim, int table_rows, int in_bnhd,
+                     int B, int H, int N, int Dk, int Dv, int in_dtype, int out_dtype, void *stream);
+COTT_API int cott_prep_ex_bwd(const void *q, const void *k, const void *v,
+                     const void *gq, const void *gk, const void *gv, void *dq, void *dk, void *dv,
+                     float *dsig_rows, const unsigned char *keep, const float *cnt, const float *sig,
+                     const float *rot_table, const long long *pos, int rotary_dim, int table_rows, int in_bnhd,
+                     int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream);
+
 /* ---- per-kernel timing -----------------------------------------------------------------------
  * While enabled, every kernel launch made by the entry points above is bracketed by a pair of HIP
  * events on the launch stream (this is the one place the library creates HIP objects).

@@ -384,3 +384,45 @@ def test_prepare_inputs_autograd_function_feeds_attention(ct, oracle):
     for got, ref in zip((qd.grad, kd.grad, vd.grad, cd.grad), ref_grads):
         assert got.dtype == torch.float32
         assert rel_l2(got, ref.numpy()) <= 2e-2
+
+
+@pytest.mark.parametrize("case", [(2, 3, 150, 64, 64, F32, BF, 32), (2, 2, 97, 48, 80, BF, BF, 48), (1, 2, 63, 128, 128, F64, F64, 64),
+                                  (1, 4, 130, 256, 64, HF, F32, 64), (2, 2, 40, 512, 512, F32, F32, 256)],
+                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1] + "-rot" + str(c[7]))
+def test_input_preparation_with_rotary_and_projection_layout(ct, case):
+    # GPTCosAttention.py:434-476: split heads (B,S,H,D), rotary on the first R columns of q and k, permute to
+    # (B,H,S,D), then the preparation steps -- against the same sequence written with the CPU forms.
+    from oracle import torch_forms as tf
+    b, h, n, dk, dv, dt_in, dt_out, rdim = case
+    say("prep+rotary", case)
+    g = torch.Generator().manual_seed(n + rdim)
+    q, k = (torch.randn(b, n, h, dk, generator=g).to(dt_in) for _ in range(2))
+    v = torch.randn(b, n, h, dv, generator=g).to(dt_in)
+    keep = torch.rand(b, n, generator=g) > 0.2
+    sig = torch.sigmoid(torch.randn(h, generator=g)).double()
+    table = tf.gptj_sinusoid_table(300, rdim)
+    pos = torch.randint(0, 300, (b, n), generator=g)
+    q64, k64, v64 = (t.clone().double().requires_grad_(True) for t in (q, k, v))
+    sig64 = sig.clone().requires_grad_(True)
+    sin, cos = torch.split(table.double()[pos], rdim // 2, dim=-1)
+    qr = torch.cat([tf.gptj_rotate(q64[..., :rdim], sin, cos), q64[..., rdim:]], -1).permute(0, 2, 1, 3)
+    kr = torch.cat([tf.gptj_rotate(k64[..., :rdim], sin, cos), k64[..., rdim:]], -1).permute(0, 2, 1, 3)
+    rq, rk, rv, cnt = tf.input_prep_gpt(qr, kr, v64.permute(0, 2, 1, 3), keep, sig64)
+    args = dict(keep=keep.to(DEV), cnt=cnt.float().to(DEV), sig=sig.float().to(DEV), rotary=(table.to(DEV), pos.to(DEV)),
+                bnhd=True)
+    oq, ok, ov = ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), out_dtype=dt_out, **args)
+    assert oq.shape == (b, h, n, dk) and ov.shape == (b, h, n, dv) and oq.is_contiguous()
+    for got, ref in ((oq, rq), (ok, rk), (ov, rv)):
+        assert rel_l2(got, ref.detach().numpy()) <= TOL[dt_out]
+    gq, gk = (torch.randn(b, h, n, dk, generator=g).to(dt_out) for _ in range(2))
+    gv = torch.randn(b, h, n, dv, generator=g).to(dt_out)
+    grads = torch.autograd.grad([rq, rk, rv], [q64, k64, v64, sig64], [gq.double(), gk.double(), gv.double()])
+    dq, dk_, dv_, dsig = ct.prepare_inputs_backward(q.to(DEV), k.to(DEV), v.to(DEV), gq.to(DEV), gk.to(DEV), gv.to(DEV),
+                                                    want_dsig=True, **args)
+    assert dq.shape == q.shape and dq.dtype == dt_in
+    tol = max(TOL[dt_in], TOL[dt_out])
+    for got, ref in ((dq, grads[0]), (dk_, grads[1]), (dv_, grads[2])):
+        assert rel_l2(got, ref.numpy()) <= tol
+    assert rel_l2(dsig, grads[3].numpy()) <= max(tol, 1e-4)
+    with pytest.raises(RuntimeError):
+        ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), rotary=(table.to(DEV), (pos + 300).to(DEV)), bnhd=True)
