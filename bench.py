@@ -17,6 +17,7 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+SPINUP_S = 0.3               # untimed GPU spin-up before the warm-up steps
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 # HBM-side bytes per launch at the headline shape, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
@@ -108,6 +109,13 @@ def main():
         grads = ct.causal_backward(q, k, v, do)
         return o, grads
 
+    # untimed spin-up so that the clocks have settled before the W warm-up steps (a cold process measures ~8 % low)
+    t_end = time.perf_counter() + SPINUP_S
+    while time.perf_counter() < t_end:
+        for _ in range(50):
+            step()
+        torch.cuda.synchronize()
+
     sec = time_region(torch, step, args.steps, args.warmup)
     tokens_per_s = B * N / sec
 
@@ -146,6 +154,7 @@ def main():
 
     extras = {"fwd_us": sec_f * 1e6, "bwd_us": sec_b * 1e6, "kernels": kern}
     if not args.no_extras:
+        extras["cold_cache_headline"] = cold_cache_kernel_times(torch, ct, dev, q, k, v, do)
         extras.update(run_extras(torch, ct, dev))
 
     out = {
@@ -154,12 +163,40 @@ def main():
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[2]: GPT-300M-shape causal cosine attention fwd+bwd (dQ,dK,dV), "
-                               "B=8 H=16 N=2048 D=64 bf16, fp32 state carry", "B": B, "H": H, "N": N, "D": D},
+                               "B=8 H=16 N=2048 D=64 bf16, fp32 state carry", "B": B, "H": H, "N": N, "D": D,
+                   "spinup_s": SPINUP_S},
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(torch),
         "extras": extras,
     }
     print(json.dumps(out))
+
+
+def cold_cache_kernel_times(torch, ct, dev, q, k, v, do):
+    """Kernel durations at the headline shape when nothing is left in L2 or the 256 MB last-level cache from the
+    previous call (a 1 GiB device copy runs before every launch), which is how a training step meets these kernels.
+    The step loop above re-uses its 256 MiB of tensors every iteration and so is served partly from that cache."""
+    from cottention_transformer_amd import _loader
+    big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    big2 = torch.empty_like(big)
+    state = ct.causal_prefill(q, k, v)[1]
+
+    def run(fn, kernel):
+        fn()
+        torch.cuda.synchronize()
+        _loader.profile_enable(True)
+        for _ in range(20):
+            big2.copy_(big)
+            fn()
+        torch.cuda.synchronize()
+        _loader.profile_enable(False)
+        ms, n = _loader.profile_read(kernel)
+        return 1e3 * ms / n
+    out = {"fwd_kernel_us": run(lambda: ct.causal_dot_product(q, k, v), "scan"),
+           "bwd_kernel_us": run(lambda: ct.causal_backward(q, k, v, do), "scan_grad"),
+           "bwd_kernel_with_forward_state_us": run(lambda: ct.causal_backward(q, k, v, do, total_state=state), "scan_grad")}
+    del big, big2
+    return out
 
 
 def run_extras(torch, ct, dev):
