@@ -100,8 +100,6 @@ struct Op {
     int di, dj, reversed;
     const void *sin = nullptr;  // (BH,di,dj) state to start from / to receive the final state (causal only)
     void *sout = nullptr;
-    const float *total = nullptr;  // complement form, see cott::OpDesc
-    int tot_si = 0, tot_sj = 0, tot_head = 0;
 };
 
 // How a set of `nops` ops with the same padded head dims is laid on the chip.
@@ -234,10 +232,6 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
                 d.sin = o.sin ? static_cast<const char *>(o.sin) + (size_t)h * djh * ssz : nullptr;
                 d.sout = o.sout ? static_cast<char *>(o.sout) + (size_t)h * djh * ssz : nullptr;
                 d.lds = o.dj;
-                d.total = o.total ? o.total + (size_t)h * djh * o.tot_sj : nullptr;
-                d.tot_si = o.tot_si;
-                d.tot_sj = o.tot_sj;
-                d.tot_head = o.tot_head;
             }
         }
         a.ws = p.ws_bytes ? reinterpret_cast<float *>(ws_cursor) : nullptr;
@@ -381,35 +375,6 @@ int cott_causal_bwd(const void *q, const void *k, const void *v, const void *d_o
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
     Op ops[3];
     grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
-    return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
-}
-
-int cott_causal_bwd_state(const void *q, const void *k, const void *v, const void *d_o, const void *state_total, void *dq,
-                          void *dk, void *dv, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace,
-                          size_t workspace_bytes, void *stream) {
-    const char *fn = "cott_causal_bwd_state";
-    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
-    if (int rc = check_common(fn, B, H, N, Dv, Dk, dtype)) return rc;
-    if ((long)B * H * N == 0) return COTT_OK;
-    if (!q || !k || !v || !d_o || !dq || !dk || !dv) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
-        !aligned16(dv) || !aligned16(state_total))
-        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
-    Op ops[3];
-    grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
-    // dQ[s] = dO[s] (sum_{s'<=s} V^T K) = dO[s] (total^T - sum_{s'>s} V^T K): with the whole-sequence state of the
-    // forward pass dQ can walk the sequence backwards like dK and dV, so the three problems of a head read the same
-    // rows of q, k, v, dO at the same time.  16-bit MFMA kernels only: the difference total - suffix is formed in
-    // fp32, good for the 16-bit tolerance, not for the fp32 one on long sequences.
-    bool mfma16 = (dtype == COTT_F16 || dtype == COTT_BF16) && state_total != nullptr;
-    for (int i = 0; i < 3; ++i) mfma16 = mfma16 && use_mfma(dtype, ops[i].di, ops[i].dj, N);
-    if (mfma16) {
-        ops[0].reversed = 1;
-        ops[0].total = static_cast<const float *>(state_total);  // (Dk,Dv) per head; the dQ problem needs [dv][dk]
-        ops[0].tot_si = 1;
-        ops[0].tot_sj = Dv;
-        ops[0].tot_head = Dk * Dv;
-    }
     return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 

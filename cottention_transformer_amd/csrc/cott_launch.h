@@ -16,10 +16,6 @@ struct OpDesc {
     const void *sin = nullptr;  // start from this state instead of zero
     void *sout = nullptr;       // receives the state after the last position
     int lds = 0;
-    // Complement form (16-bit MFMA path, reversed ops only): fp32 whole-sequence sum of B^T C per head, element
-    // [i][j] at total[i*tot_si + j*tot_sj], heads tot_head elements apart; see ProblemT in cott_mfma.h.
-    const void *total = nullptr;
-    int tot_si = 0, tot_sj = 0, tot_head = 0;
 };
 
 // A set of ops launched together over the same (BH, N); MFMA path: all share padded head dims.

@@ -36,12 +36,6 @@ struct ProblemT {
     const float *sin;
     float *sout;
     int di, dj, ldc, reversed, lds;
-    // Complement form (16-bit scan kernel only): `total`, if not null, is the head's sum of B^T C over the WHOLE
-    // sequence, element [i][j] at total[i*tot_si + j*tot_sj].  The problem must be `reversed`; the kernel then
-    // returns  A (total - sum over positions AFTER s) = the forward-direction result, while walking the sequence
-    // backwards like its neighbours in the set.
-    const float *total;
-    int tot_si, tot_sj, tot_head;  // tot_head: elements per head
 };
 
 template <class E>
@@ -325,34 +319,13 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
                     if (i0 + r < di && j < dj) S[u][r] += si[(size_t)(i0 + r) * pr.lds + j];
             }
         }
-        // complement form: T = the whole-sequence sum; the published state is S - T (the output wavefronts
-        // flip the sign of their result)
-        f32x4 T[TL::TPW];
-#pragma unroll
-        for (int u = 0; u < TL::TPW; ++u) T[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (pr.total != nullptr) {
-            const float *tt = pr.total + (size_t)wi.bh * pr.tot_head;
-#pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) {
-                const int t = w * TL::TPW + u;
-                const int i0 = 16 * (t / TL::NJT) + 4 * g, j = 16 * (t % TL::NJT) + m;
-                if (pr.tot_si == 1) {  // the four i of this lane are contiguous: one 16-byte load (di is a multiple of 16)
-                    if (i0 < di && j < dj) T[u] = *reinterpret_cast<const f32x4 *>(tt + (size_t)j * pr.tot_sj + i0);
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (i0 + r < di && j < dj) T[u][r] = tt[(size_t)(i0 + r) * pr.tot_si + (size_t)j * pr.tot_sj];
-                }
-            }
-        }
         // 16-bit copy of the state, transposed to [j][i] for the A_blk S product
         auto put_state = [&](u16 *dst) {
 #pragma unroll
             for (int u = 0; u < TL::TPW; ++u) {
                 const int t = w * TL::TPW + u;
                 const int it = t / TL::NJT, jt = t % TL::NJT;
-                u32x2 pk = {TR::pack2(S[u][0] - T[u][0], S[u][1] - T[u][1]),
-                            TR::pack2(S[u][2] - T[u][2], S[u][3] - T[u][3])};
+                u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
                 *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
             }
         };
@@ -380,9 +353,6 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
         const int w = wv;  // 0..OW-1
         const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
         const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
-        // complement form: only keys strictly after the position count, and the result changes sign
-        const int strict = pr.total != nullptr ? 1 : 0;
-        const uint32_t flip = pr.total != nullptr ? 0x80008000u : 0u;
         u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
         auto load_q = [&](int s, int p) {
             const int pc = min(p, p1 - 1);
@@ -432,7 +402,7 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
                             const int d0 = 16 * (jt - (IB * w + ib)) + 4 * g - m;  // key pos - query pos at r = 0
 #pragma unroll
                             for (int r = 0; r < 4; ++r) {
-                                const bool keep = reversed ? (d0 + r >= strict) : (d0 + r <= 0);
+                                const bool keep = reversed ? (d0 + r >= 0) : (d0 + r <= 0);
                                 acc[r] = keep ? acc[r] : 0.f;
                             }
                             pk[ib][jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
@@ -471,7 +441,7 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
                             const int col = 16 * jt + 4 * g;
                             const uint32_t off =
                                 (col < dj) ? (uint32_t)((orow + 16 * ib) * ldc + col) * 2u : kOobOffset;
-                            buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]) ^ flip, TR::pack2(o[2], o[3]) ^ flip});
+                            buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
                         }
                 }
                 __syncthreads();

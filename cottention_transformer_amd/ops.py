@@ -105,10 +105,8 @@ def causal_prefill(q, k, v, state=None, return_state=True):
     return o, s_out
 
 
-def causal_backward(q, k, v, grad_out, total_state=None):
-    """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out.
-    total_state: the state `causal_prefill(q, k, v)` returned for the same q, k, v (zero initial state); with it the
-    16-bit kernels compute dQ walking the sequence in the direction of dK and dV, which saves HBM reads."""
+def causal_backward(q, k, v, grad_out):
+    """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out."""
     _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)
     b, h, n, dk, dv = _shapes(q, k, v)
     if grad_out.shape != v.shape:
@@ -121,17 +119,9 @@ def causal_backward(q, k, v, grad_out, total_state=None):
     L = _loader.lib()
     with torch.cuda.device(q.device):
         ws, ws_ptr = _workspace(L.cott_causal_bwd_workspace_bytes(b, h, n, dk, dv, code), q.device)
-        if total_state is not None:
-            if (total_state.shape != (b, h, dk, dv) or total_state.dtype != torch.float32 or not total_state.is_contiguous()
-                    or total_state.device != q.device):
-                raise RuntimeError(f"total_state must be a contiguous fp32 tensor of shape {(b, h, dk, dv)} on {q.device}")
-            rc = L.cott_causal_bwd_state(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), total_state.data_ptr(),
-                                         dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr,
-                                         ws.numel() if ws is not None else 0, _stream())
-        else:
-            rc = L.cott_causal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(), dk_.data_ptr(),
-                                   dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0,
-                                   _stream())
+        rc = L.cott_causal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(), dk_.data_ptr(),
+                               dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0,
+                               _stream())
     _check(rc, "cott_causal_bwd")
     return dq, dk_, dv_
 

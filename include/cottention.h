@@ -83,18 +83,6 @@ COTT_API int cott_causal_bwd(const void *q, const void *k, const void *v, const 
                     int B, int H, int N, int Dk, int Dv, int dtype,
                     void *workspace, size_t workspace_bytes, void *stream);
 
-/* The same gradients, given the whole-sequence state that cott_causal_fwd_state returned for these q, k, v with
- * a zero (NULL) initial state: state_total[b,h] = sum over all positions of k v^T, (B,H,Dk,Dv) fp32.  For fp16 /
- * bf16 on the MFMA kernels dQ is then computed as dO (total - suffix sums), walking the sequence in the same
- * direction as dK and dV, so the three gradient problems of a head share their reads of q, k, v, dO in cache
- * (HBM fetch drops from 6.8 to about 4 tensor passes).  Other dtypes, and state_total == NULL, behave exactly
- * like cott_causal_bwd.  No counterpart in the reference (its three launches of Custom_Kernel.py:106-108 are
- * independent).  Workspace: cott_causal_bwd_workspace_bytes(). */
-COTT_API int cott_causal_bwd_state(const void *q, const void *k, const void *v, const void *d_o,
-                          const void *state_total, void *dq, void *dk, void *dv,
-                          int B, int H, int N, int Dk, int Dv, int dtype,
-                          void *workspace, size_t workspace_bytes, void *stream);
-
 /* ---- non-causal form ------------------------------------------------------------------------
  *   o = q (k^T v)   per (batch, head)
  * Replaces the two einsums of BERT_Trainer/BertCosAttention.py:249 (the (QK^T)V branch at :222

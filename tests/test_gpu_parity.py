@@ -80,25 +80,6 @@ def test_causal_backward(ct, oracle, case):
         assert rel_l2(got, ref) <= TOL[dt], name
 
 
-@pytest.mark.parametrize("case", [c for c in CAUSAL_CASES if c[5] in (BF, HF) and c[4] % 16 == 0],
-                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
-def test_causal_backward_with_forward_state(ct, oracle, case):
-    # dQ from the whole-sequence state of the forward pass (complement form): same gradients as the plain call
-    b, h, n, dk, dv, dt = case
-    say("causal bwd + state", case)
-    q, k, v, do = inputs(b, h, n, dk, dv, dt, seed=n + 1)
-    refs = oracle.causal_bwd(q, k, v, do)
-    qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
-    o, state = ct.causal_prefill(qd, kd, vd)
-    assert rel_l2(o, oracle.causal(q, k, v)) <= TOL[dt]
-    outs = ct.causal_backward(qd, kd, vd, dod, total_state=state)
-    for name, got, ref in zip(("dQ", "dK", "dV"), outs, refs):
-        assert rel_l2(got, ref) <= TOL[dt], name
-    # first and last positions separately: the complement form subtracts almost the whole total at the start
-    assert rel_l2(outs[0][:, :, :8], refs[0][:, :, :8]) <= TOL[dt]
-    assert rel_l2(outs[0][:, :, -8:], refs[0][:, :, -8:]) <= TOL[dt]
-
-
 def test_golden_fixtures(ct):
     for name in ("causal_cfg1_1x2x128x64.npz", "causal_odd_1x2x63x32_dv48.npz"):
         say("golden", name)
