@@ -207,7 +207,12 @@ def run_extras(torch, ct, dev):
     byts = 4 * b * h * n * d * 2
     ex["noncausal_fwd_B32_H12_N512_D64"] = {"us": s * 1e6, "tokens_per_s": b * n / s, "GBps": byts / s / 1e9,
                                             "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS}
-    del q, k, v
+    do = torch.randn_like(v)
+    s = time_region(torch, lambda: ct.noncausal_backward(q, k, v, do), 100, 10)
+    byts = 7 * b * h * n * d * 2
+    ex["noncausal_bwd_B32_H12_N512_D64"] = {"us": s * 1e6, "tokens_per_s": b * n / s, "GBps": byts / s / 1e9,
+                                            "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS}
+    del q, k, v, do
     # recurrent decode, state (256,16,128,128) fp32, 512 consecutive steps with fresh q,k,v per step
     b, h, d, steps = 256, 16, 128, 512
     g = torch.Generator(device=dev).manual_seed(0)

@@ -426,3 +426,67 @@ def test_input_preparation_with_rotary_and_projection_layout(ct, case):
     assert rel_l2(dsig, grads[3].numpy()) <= max(tol, 1e-4)
     with pytest.raises(RuntimeError):
         ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), rotary=(table.to(DEV), (pos + 300).to(DEV)), bnhd=True)
+
+
+def test_calls_can_be_captured_in_a_hip_graph_and_replayed(ct, oracle):
+    # The library allocates nothing and never synchronises, so its launches can be recorded into a graph: a decode
+    # step (state updated in place by every replay) and a forward+backward pair with fixed buffers.  Replays are
+    # interleaved with eager work and synchronisation, and every replay is checked against the eager result.
+    from cottention_transformer_amd import _loader
+    L = _loader.lib()
+    b, h, d = 4, 4, 64
+    g = torch.Generator().manual_seed(21)
+    steps = 5
+    qs = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g), dim=-1).to(BF).to(DEV)
+    ks = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g), dim=-1).to(BF).to(DEV)
+    vs = torch.randn(steps, b, h, d, generator=g).to(BF).to(DEV)
+    q1, k1, v1 = (torch.empty(b, h, d, dtype=BF, device=DEV) for _ in range(3))
+    out = torch.empty(b, h, d, dtype=BF, device=DEV)
+    state = torch.zeros(b, h, d, d, device=DEV)
+    eager_state = torch.zeros(b, h, d, d, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                         # warm-up on the capture stream
+        q1.copy_(qs[0]); k1.copy_(ks[0]); v1.copy_(vs[0])
+        ct.decode_step(torch.zeros_like(state), q1, k1, v1, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        rc = L.cott_decode_step(state.data_ptr(), q1.data_ptr(), k1.data_ptr(), v1.data_ptr(), out.data_ptr(), b, h, d, d,
+                                _loader.BF16, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+    for t in range(steps):
+        q1.copy_(qs[t]); k1.copy_(ks[t]); v1.copy_(vs[t])
+        graph.replay()
+        want = ct.decode_step(eager_state, qs[t], ks[t], vs[t])          # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {t}"
+    assert torch.equal(state, eager_state)
+
+    # forward + backward of a multi-group shape (workspace in use) in one graph
+    bb, hh, n = 1, 2, 1023
+    q, k, v, do = (x.to(DEV) for x in inputs(bb, hh, n, 64, 64, BF, seed=33))
+    o = torch.empty_like(v); dq = torch.empty_like(q); dk = torch.empty_like(k); dv = torch.empty_like(v)
+    nf = L.cott_causal_workspace_bytes(bb, hh, n, 64, 64, _loader.BF16)
+    nb = L.cott_causal_bwd_workspace_bytes(bb, hh, n, 64, 64, _loader.BF16)
+    assert nf > 0 and nb > 0
+    wsf = torch.empty(nf, dtype=torch.uint8, device=DEV); wsb = torch.empty(nb, dtype=torch.uint8, device=DEV)
+    graph2 = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph2, stream=side):
+        st = torch.cuda.current_stream().cuda_stream
+        assert L.cott_causal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), bb, hh, n, 64, 64, _loader.BF16, 0,
+                                 wsf.data_ptr(), nf, st) == 0
+        assert L.cott_causal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                 dv.data_ptr(), bb, hh, n, 64, 64, _loader.BF16, wsb.data_ptr(), nb, st) == 0
+    for rep in range(3):
+        new = [x.to(DEV) for x in inputs(bb, hh, n, 64, 64, BF, seed=40 + rep)]
+        for dst, src in zip((q, k, v, do), new):
+            dst.copy_(src)
+        graph2.replay()
+        want_o = ct.causal_dot_product(*new[:3])
+        want_g = ct.causal_backward(*new)
+        torch.cuda.synchronize()
+        assert torch.equal(o, want_o), f"replay {rep}"
+        for got, want in zip((dq, dk, dv), want_g):
+            assert torch.equal(got, want), f"replay {rep}"
