@@ -49,7 +49,7 @@ def decode_case(name, b, h, dk, dv, steps, seed):
 
 
 if __name__ == "__main__":
-    causal_case("causal_cfg1_1x2x128x64.npz", (1, 2, 128, 64), 64, seed=0)    # BASELINE configs[0]
+    causal_case("causal_cfg1_1x2x128x64.npz", (1, 2, 128, 64), 64, seed=0)    # the reference CPU-runnable benchmark case: fp32 (1,2,128,64)
     causal_case("causal_odd_1x2x63x32_dv48.npz", (1, 2, 63, 32), 48, seed=1)   # odd S (Custom_Kernel.py:157), Dk != Dv
     noncausal_case("noncausal_2x2x50x32.npz", (2, 2, 50, 32), 32, seed=2)
     decode_case("decode_2x2x32x48_4steps.npz", 2, 2, 32, 48, 4, seed=3)

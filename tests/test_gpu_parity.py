@@ -1,5 +1,5 @@
 """GPU parity: the HIP path, called through the C ABI (ctypes) from the host layer, against the CPU
-oracle on identical seeded inputs.  Tolerances are BASELINE's: rel-L2 <= 1e-4 for fp32 inputs,
+oracle on identical seeded inputs.  Tolerances of the benchmark definition: rel-L2 <= 1e-4 for fp32 inputs,
 <= 2e-2 for bf16/fp16 inputs (oracle evaluated in fp64 on the same rounded inputs); fp64 <= 1e-12."""
 import os
 import sys
@@ -33,7 +33,7 @@ BF, HF, F32, F64 = torch.bfloat16, torch.float16, torch.float32, torch.float64
 
 CAUSAL_CASES = [
     # b, h, n, dk, dv, dtype                      what it exercises
-    (1, 2, 128, 64, 64, F32),     # BASELINE configs[0]
+    (1, 2, 128, 64, 64, F32),     # the reference CPU-runnable benchmark case: fp32 (1,2,128,64)
     (1, 2, 128, 64, 64, BF),      # two chunks -> two groups
     (1, 2, 63, 128, 128, F64),    # the reference's gradcheck shape (Custom_Kernel.py:157)
     (1, 2, 63, 64, 64, BF),       # odd S, single partial chunk
@@ -279,7 +279,7 @@ def test_gradcheck_fp64(ct):
 
 
 def test_headline_shape_properties(ct, oracle):
-    """Full BASELINE size (B8 H16 N2048 D64 bf16): oracle on a head subset plus size-independent
+    """Full headline benchmark size (B8 H16 N2048 D64 bf16): oracle on a head subset plus size-independent
     properties -- linearity in V, `reversed` == flip(forward(flip)), last causal row == non-causal row."""
     b, h, n, d = 8, 16, 2048, 64
     say("headline shape")

@@ -6,7 +6,7 @@ import torch
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
-# BASELINE tolerances: rel-L2 <= 1e-4 for fp32 inputs, <= 2e-2 for bf16/fp16 inputs against the
+# Tolerances of the benchmark definition: rel-L2 <= 1e-4 for fp32 inputs, <= 2e-2 for bf16/fp16 inputs against the
 # fp32/fp64 oracle evaluated on the same rounded inputs; fp64 is held to 1e-12.
 TOL = {torch.float32: 1e-4, torch.float64: 1e-12, torch.float16: 2e-2, torch.bfloat16: 2e-2}
 
