@@ -109,11 +109,30 @@ struct SetPlan {
     size_t ws_bytes;      // group-state slots
 };
 
-SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtype) {
+// COTT_PAIR=0 switches the paired dK/dV workgroups off (experiments).
+bool pair_enabled() {
+    static const bool v = env_int("COTT_PAIR", 1) != 0;
+    return v;
+}
+
+// The last two of three causal ops form a pair when they are X = G(A,B,C), Y = G(A2,C,B), same direction, 16-bit
+// storage, and all three ops share square padded head dims of at most 64 (dK and dV of a backward pass).
+bool pair_eligible(const Op *ops, int n, int dtype, bool causal) {
+    if (!pair_enabled() || !causal || n != 3 || !(dtype == COTT_F16 || dtype == COTT_BF16)) return false;
+    const Op &x = ops[1], &y = ops[2];
+    if (!(x.B == y.C && x.C == y.B && x.reversed == y.reversed && x.di == y.dj && x.dj == y.di)) return false;
+    const int pd = cott::mfma_pad(ops[0].di);
+    if (pd > 64) return false;
+    for (int i = 0; i < 3; ++i)
+        if (cott::mfma_pad(ops[i].di) != pd || cott::mfma_pad(ops[i].dj) != pd || ops[i].sin || ops[i].sout) return false;
+    return true;
+}
+
+SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtype, bool no_split = false) {
     SetPlan p;
     // the fp32 kernels are MFMA-bound with four wavefronts per workgroup: two workgroups per CU overlap well
     const long tgt = target_workgroups() * (dtype == COTT_F32 ? 2 : 1);
-    const bool can_split = dtype != COTT_F32 && dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
+    const bool can_split = !no_split && dtype != COTT_F32 && dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
     const int pol = split_policy();
     p.nchunks = (N + 63) / 64;
     // Choose (column halves, sequence groups) to fill the target without exceeding it: halves cost
@@ -157,6 +176,7 @@ size_t ops_workspace(const Op *ops, int n, long BH, int N, int dtype, bool causa
     if (BH <= 0 || N <= 0) return 0;
     for (int i = 0; i < n; ++i)
         if (!use_mfma(dtype, ops[i].di, ops[i].dj, N)) return 0;
+    if (pair_eligible(ops, n, dtype, causal)) return plan_set(BH, N, 2, ops[0].di, ops[0].dj, causal, dtype, true).ws_bytes;
     size_t total = 0;
     bool done[8] = {false};
     for (int i = 0; i < n; ++i) {
@@ -214,7 +234,10 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         int members[8], cnt = 0;
         for (int j = i; j < n; ++j)
             if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; members[cnt++] = j; }
-        const SetPlan p = plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal, dtype);
+        const bool pair = pair_eligible(ops, n, dtype, causal);  // then all three ops are in this set
+        const SetPlan p = pair ? plan_set(BH, N, 2, ops[i].di, ops[i].dj, causal, dtype, true)
+                               : plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal, dtype);
+        a.pair = pair ? 1 : 0;
         for (int c = 0; c < cnt; ++c) {
             const Op &o = ops[members[c]];
             const int djh = o.dj / p.halves;

@@ -26,6 +26,10 @@ struct SetArgs {
     int BH, N;
     int nchunks, cpg, G;  // chunks of 64, chunks per group, groups per head
     int scan_prof_id;     // K_SCAN for a forward launch, K_SCAN_GRAD for the three-gradient launch
+    // pair > 0: op[pair] and op[pair + 1] are X = G(A,B,C) and Y = G(A2,C,B) with the same direction and square
+    // padded head dims; one workgroup serves both (scan_pair_kernel).  The launch then has count - 1 problems
+    // per head and the workspace count - 1 state slots per group.  pair must be count - 2.
+    int pair = 0;
     hipStream_t stream;
 };
 

@@ -36,6 +36,9 @@ struct ProblemT {
     const float *sin;
     float *sout;
     int di, dj, ldc, reversed, lds;
+    // scan_pair_kernel only: a second problem G(A2, C, B) -> O2 served by the same workgroup (null = none)
+    const E *A2;
+    E *O2;
 };
 
 template <class E>
@@ -228,19 +231,238 @@ __global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSetT<E> s
     if (mode == 1) p[0] = run;
 }
 
-// The chunk recurrence for one group of one head of one problem.
+// ---- the chunk recurrence --------------------------------------------------------------------------
 //
-// Wavefronts in three roles that share the SIMDs, so that each role's LDS / VALU / memory latencies
-// are covered by the other roles' work and no role's per-chunk dependency chain carries the others':
-//   * OW "output" wavefronts (first in the workgroup), each owning 64/OW output positions of the
-//     chunk as IB = 4/OW blocks of 16.  A block's scores are formed transposed, P^T = B_c A_blk^T,
-//     tile by tile, so the accumulator layout IS the operand layout of the next product and the
-//     masked scores never leave registers; then out_blk^T = C_c^T P^T + S^T A_blk^T, stored as 8-byte
-//     row segments.  Score tiles above the diagonal are computed and zeroed.
+// A workgroup handles one group of chunks of one head with wavefronts in three roles that share the
+// SIMDs, so that each role's LDS / VALU / memory latencies are covered by the other roles' work and
+// no role's per-chunk dependency chain carries the others':
+//   * "output" wavefronts, each owning IB blocks of 16 output positions of the chunk.  A block's
+//     scores are formed transposed, P^T = B_c A_blk^T, tile by tile, so the accumulator layout IS the
+//     operand layout of the next product and the masked scores never leave registers; then
+//     out_blk^T = C_c^T P^T + S^T A_blk^T, stored as 8-byte row segments.  Score tiles above the
+//     diagonal are computed and zeroed.
 //   * four "state" wavefronts carry the fp32 state S += B_c^T C_c in their accumulators and publish
 //     its 16-bit copy for the next chunk.
-//   * LW "loader" wavefronts move the B and C tiles global -> registers -> LDS, PF chunks ahead.
-// One barrier per chunk joins the roles; LDS tiles and the 16-bit state are double-buffered.
+//   * "loader" wavefronts move the B and C tiles global -> registers -> LDS, PF chunks ahead.
+// One barrier per chunk joins the roles (every role function below executes 1 + (p1 - p0) barriers);
+// LDS tiles and the 16-bit state are double-buffered.
+
+// Position of a workgroup in the scan: chunks [p0, p1) in scan order of `nchunks`.
+struct ScanRange {
+    int N, nchunks, p0, p1, reversed;
+};
+
+// Loader role: LT threads stage the B tile (rows of di) and the C tile (dj columns of rows of ldc).
+template <int DI, int DJ, int PF, int LT>
+__device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head, int di, int dj, int ldc,
+                                            const ScanRange &r, int tid, u16 *sB, u16 *sC) {
+    using TL = Tiling<DI, DJ>;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS;
+    const rsrc_t rB = make_rsrc(B_head, (uint32_t)r.N * di * 2u);
+    const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
+    u32x4 rb[PF][8 * DI / LT], rc[PF][8 * DJ / LT];
+    auto load_chunk = [&](int s, int p) {
+        const int pc = min(p, r.p1 - 1);
+        const int row0 = (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
+        load_tile<DI, LT>(rb[s], rB, row0, di, tid);
+        load_tile<DJ, LT>(rc[s], rC, row0, ldc, tid);
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_chunk(s, r.p0 + s);
+    store_tile<DI, TL::BS, LT>(sB, rb[0], di, tid);
+    store_tile<DJ, TL::CS, LT>(sC, rc[0], dj, tid);
+    load_chunk(0, r.p0 + PF);
+    __syncthreads();
+    for (int pb = r.p0;; pb += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int p = pb + s;
+            if (p >= r.p1) return;  // uniform over the workgroup
+            const int s1 = (s + 1) % PF;
+            const int buf = (p - r.p0) & 1;
+            // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
+            store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+            store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+            load_chunk(s1, p + 1 + PF);
+            __syncthreads();
+        }
+    }
+}
+
+// State role (wavefront w of 4).  seed: register-native group prefix or null; sin / sout: row-major
+// fp32 hand-over states or null (sout only written when `last_group`).  sS: 16-bit copy transposed to
+// [j][i] for the A_blk S product.  TWIN: also publish the copy of the TRANSPOSED state (which is
+// [i][j] of this one) in sS2, for a second problem whose B and C are this problem's C and B.
+template <class TR, int DI, int DJ, bool TWIN>
+__device__ __forceinline__ void state_role(const float *seed, const float *sin, float *sout, int lds, bool last_group,
+                                           int di, int dj, const ScanRange &r, int w, int l, const u16 *sB,
+                                           const u16 *sC, u16 *sS, u16 *sS2) {
+    using TL = Tiling<DI, DJ>;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
+    const int g = l >> 4, m = l & 15;
+    f32x4 S[TL::TPW];
+#pragma unroll
+    for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (seed != nullptr) {
+        const f32x4 *gs = reinterpret_cast<const f32x4 *>(seed);
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
+    }
+    // accumulator element r of tile (it, jt) is S[16it + 4g + r][16jt + m]
+    if (sin != nullptr) {
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) {
+            const int t = w * TL::TPW + u;
+            const int i0 = 16 * (t / TL::NJT) + 4 * g, j = 16 * (t % TL::NJT) + m;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (i0 + q < di && j < dj) S[u][q] += sin[(size_t)(i0 + q) * lds + j];
+        }
+    }
+    auto put_state = [&](u16 *dst, u16 *dst2) {
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) {
+            const int t = w * TL::TPW + u;
+            const int it = t / TL::NJT, jt = t % TL::NJT;
+            u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
+            *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
+            if (TWIN) {
+                dst2[(16 * it + 4 * g + 0) * TL::SS + 16 * jt + m] = (u16)(pk.x & 0xffffu);
+                dst2[(16 * it + 4 * g + 1) * TL::SS + 16 * jt + m] = (u16)(pk.x >> 16);
+                dst2[(16 * it + 4 * g + 2) * TL::SS + 16 * jt + m] = (u16)(pk.y & 0xffffu);
+                dst2[(16 * it + 4 * g + 3) * TL::SS + 16 * jt + m] = (u16)(pk.y >> 16);
+            }
+        }
+    };
+    put_state(sS, sS2);
+    __syncthreads();
+    for (int p = r.p0; p < r.p1; ++p) {
+        const int buf = (p - r.p0) & 1;
+        state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+        put_state(sS + (buf ^ 1) * SSZ, sS2 + (buf ^ 1) * SSZ);
+        __syncthreads();
+    }
+    if (sout != nullptr && last_group) {
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) {
+            const int t = w * TL::TPW + u;
+            const int i0 = 16 * (t / TL::NJT) + 4 * g, j = 16 * (t % TL::NJT) + m;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (i0 + q < di && j < dj) sout[(size_t)(i0 + q) * lds + j] = S[u][q];
+        }
+    }
+}
+
+// Output role: one wavefront, IB blocks of 16 positions starting at block `blk0` of each chunk.
+// cB: tile read by rows (the B operand of this problem), cC: tile read by columns (its C operand),
+// cS: its 16-bit state; all three double-buffered with the strides of Tiling<DI, DJ>.
+template <class TR, int DI, int DJ, int PF, int IB>
+__device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int ldc, const ScanRange &r,
+                                            int blk0, int l, const u16 *sB, const u16 *sC, const u16 *sS) {
+    using TL = Tiling<DI, DJ>;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
+    const int g = l >> 4, m = l & 15;
+    const rsrc_t rA = make_rsrc(A_head, (uint32_t)r.N * di * 2u);
+    const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
+    const int reversed = r.reversed;
+    u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
+    auto load_q = [&](int s, int p) {
+        const int pc = min(p, r.p1 - 1);
+        const int row = (reversed ? r.nchunks - 1 - pc : pc) * kChunk + 16 * blk0 + m;
+#pragma unroll
+        for (int ib = 0; ib < IB; ++ib)
+#pragma unroll
+            for (int ks = 0; ks < TL::KS; ++ks)
+                qn[s][ib][ks] = buf_load16(rA, (uint32_t)((row + 16 * ib) * di + 32 * ks + 8 * g) * 2u);
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_q(s, r.p0 + s);
+    __syncthreads();
+    for (int pb = r.p0;; pb += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int p = pb + s;
+            if (p >= r.p1) return;
+            const int buf = (p - r.p0) & 1;
+            const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
+            const int row0 = (reversed ? r.nchunks - 1 - p : p) * kChunk;
+#pragma unroll
+            for (int ib = 0; ib < IB; ++ib)
+#pragma unroll
+                for (int ks = 0; ks < TL::KS; ++ks)
+                    qc[ib][ks] = (32 * ks + 8 * g < di) ? qn[s][ib][ks] : u32x4{0u, 0u, 0u, 0u};
+            load_q(s, p + PF);
+
+            // masked scores, transposed: pk[ib][jt] = P^T[16jt+4g .. +3][16(blk0+ib)+m]; fragment
+            // reads first, MFMAs after, so the LDS latency is paid once per batch
+            u32x2 pk[IB][4];
+            {
+                u32x4 kf[4][TL::KS];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        kf[jt][ks] = *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
+#pragma unroll
+                for (int ib = 0; ib < IB; ++ib)
+#pragma unroll
+                    for (int jt = 0; jt < 4; ++jt) {
+                        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ib][ks], acc);
+                        const int d0 = 16 * (jt - (blk0 + ib)) + 4 * g - m;  // key pos - query pos at element 0
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const bool keep = reversed ? (d0 + q >= 0) : (d0 + q <= 0);
+                            acc[q] = keep ? acc[q] : 0.f;
+                        }
+                        pk[ib][jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
+                    }
+            }
+
+            const int orow = row0 + 16 * blk0 + m;
+#ifndef COTT_JB2
+#define COTT_JB2 4
+#endif
+            constexpr int JBmax = (IB == 1) ? 8 : COTT_JB2;
+            constexpr int JB = (JBmax / TL::KS < 1) ? 1 : ((JBmax / TL::KS < TL::NJT) ? (JBmax / TL::KS) : TL::NJT);
+#pragma unroll
+            for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
+                u32x4 vf[JB][2], sf[JB][TL::KS];
+#pragma unroll
+                for (int jj = 0; jj < JB; ++jj) {
+                    const int jt = j0 + jj;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+                        vf[jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
+                                         lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        sf[jj][ks] = *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
+                }
+#pragma unroll
+                for (int ib = 0; ib < IB; ++ib)
+#pragma unroll
+                    for (int jj = 0; jj < JB; ++jj) {
+                        const int jt = j0 + jj;
+                        f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int kb = 0; kb < 2; ++kb)
+                            o = TR::mfma(vf[jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
+#pragma unroll
+                        for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ib][ks], o);
+                        const int col = 16 * jt + 4 * g;
+                        const uint32_t off = (col < dj) ? (uint32_t)((orow + 16 * ib) * ldc + col) * 2u : kOobOffset;
+                        buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
+                    }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// One problem per workgroup: OW output wavefronts (IB = 4/OW blocks each), 4 state, LW loader.
 template <class TR, int DI, int DJ, int PF, int OW, int LW>
 __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set, int BH, int N, int nchunks,
                                                                   int cpg, int G) {
@@ -254,199 +476,91 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
     __shared__ __attribute__((aligned(16))) u16 sS[2 * SSZ];
-    const int l = threadIdx.x & 63, g = l >> 4, m = l & 15;
+    const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const WorkItem wi = decode_workgroup(set.count, G);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
-    const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
-    const int p0 = wi.grp * cpg;
-    const int p1 = min(p0 + cpg, nchunks);
-
+    const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
+    ScanRange r;
+    r.N = N;
+    r.nchunks = nchunks;
+    r.p0 = wi.grp * cpg;
+    r.p1 = min(r.p0 + cpg, nchunks);
+    r.reversed = pr.reversed;
     if (wv >= OW + 4) {
-        // ---------------------------------------------------------------- loader wavefronts
-        const int tid = (int)threadIdx.x - 64 * (OW + 4);  // 0..LT-1
-        const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-        const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
-        u32x4 rb[PF][8 * DI / LT], rc[PF][8 * DJ / LT];
-        auto load_chunk = [&](int s, int p) {
-            const int pc = min(p, p1 - 1);
-            const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
-            load_tile<DI, LT>(rb[s], rB, row0, di, tid);
-            load_tile<DJ, LT>(rc[s], rC, row0, ldc, tid);
-        };
-#pragma unroll
-        for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
-        store_tile<DI, TL::BS, LT>(sB, rb[0], di, tid);
-        store_tile<DJ, TL::CS, LT>(sC, rc[0], dj, tid);
-        load_chunk(0, p0 + PF);
-        __syncthreads();
-        for (int pb = p0;; pb += PF) {
-#pragma unroll
-            for (int s = 0; s < PF; ++s) {
-                const int p = pb + s;
-                if (p >= p1) return;  // uniform over the workgroup; nothing follows the loop
-                const int s1 = (s + 1) % PF;
-                const int buf = (p - p0) & 1;
-                // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
-                store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-                store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
-                load_chunk(s1, p + 1 + PF);
-                __syncthreads();
-            }
-        }
+        loader_role<DI, DJ, PF, LT>(pr.B + (size_t)wi.bh * N * di, pr.C + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
+                                    (int)threadIdx.x - 64 * (OW + 4), sB, sC);
     } else if (wv >= OW) {
-        // ---------------------------------------------------------------- state wavefronts
-        const int w = wv - OW;  // 0..3
-        f32x4 S[TL::TPW];
-#pragma unroll
-        for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (pr.gstate != nullptr) {
-            const f32x4 *gs =
-                reinterpret_cast<const f32x4 *>(pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS);
-#pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
-        }
-        // accumulator element r of tile (it, jt) is S[16it + 4g + r][16jt + m]
-        if (pr.sin != nullptr) {
-            const float *si = pr.sin + (size_t)wi.bh * di * pr.lds;
-#pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) {
-                const int t = w * TL::TPW + u;
-                const int i0 = 16 * (t / TL::NJT) + 4 * g, j = 16 * (t % TL::NJT) + m;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (i0 + r < di && j < dj) S[u][r] += si[(size_t)(i0 + r) * pr.lds + j];
-            }
-        }
-        // 16-bit copy of the state, transposed to [j][i] for the A_blk S product
-        auto put_state = [&](u16 *dst) {
-#pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) {
-                const int t = w * TL::TPW + u;
-                const int it = t / TL::NJT, jt = t % TL::NJT;
-                u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
-                *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
-            }
-        };
-        put_state(sS);
-        __syncthreads();
-        for (int p = p0; p < p1; ++p) {
-            const int buf = (p - p0) & 1;
-            state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
-            put_state(sS + (buf ^ 1) * SSZ);
-            __syncthreads();
-        }
-        if (pr.sout != nullptr && wi.grp == G - 1) {
-            float *so = pr.sout + (size_t)wi.bh * di * pr.lds;
-#pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) {
-                const int t = w * TL::TPW + u;
-                const int i0 = 16 * (t / TL::NJT) + 4 * g, j = 16 * (t % TL::NJT) + m;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (i0 + r < di && j < dj) so[(size_t)(i0 + r) * pr.lds + j] = S[u][r];
-            }
-        }
+        state_role<TR, DI, DJ, false>(
+            pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr,
+            pr.sin ? pr.sin + (size_t)wi.bh * di * pr.lds : nullptr, pr.sout ? pr.sout + (size_t)wi.bh * di * pr.lds : nullptr,
+            pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS, nullptr);
     } else {
-        // ---------------------------------------------------------------- output wavefronts
-        const int w = wv;  // 0..OW-1
-        const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-        const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
-        u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
-        auto load_q = [&](int s, int p) {
-            const int pc = min(p, p1 - 1);
-            const int row = (reversed ? nchunks - 1 - pc : pc) * kChunk + 16 * IB * w + m;
-#pragma unroll
-            for (int ib = 0; ib < IB; ++ib)
-#pragma unroll
-                for (int ks = 0; ks < TL::KS; ++ks)
-                    qn[s][ib][ks] = buf_load16(rA, (uint32_t)((row + 16 * ib) * di + 32 * ks + 8 * g) * 2u);
-        };
-#pragma unroll
-        for (int s = 0; s < PF; ++s) load_q(s, p0 + s);
-        __syncthreads();
-        for (int pb = p0;; pb += PF) {
-#pragma unroll
-            for (int s = 0; s < PF; ++s) {
-                const int p = pb + s;
-                if (p >= p1) return;
-                const int buf = (p - p0) & 1;
-                const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
-                const int row0 = (reversed ? nchunks - 1 - p : p) * kChunk;
-#pragma unroll
-                for (int ib = 0; ib < IB; ++ib)
-#pragma unroll
-                    for (int ks = 0; ks < TL::KS; ++ks)
-                        qc[ib][ks] = (32 * ks + 8 * g < di) ? qn[s][ib][ks] : u32x4{0u, 0u, 0u, 0u};
-                load_q(s, p + PF);
+        output_role<TR, DI, DJ, PF, IB>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
+                                        IB * wv, l, sB, sC, sS);
+    }
+}
 
-                // masked scores, transposed: pk[ib][jt] = P^T[16jt+4g .. +3][16(IB*w+ib)+m]; fragment
-                // reads first, MFMAs after, so the LDS latency is paid once per batch
-                u32x2 pk[IB][4];
-                {
-                    u32x4 kf[4][TL::KS];
-#pragma unroll
-                    for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-                        for (int ks = 0; ks < TL::KS; ++ks)
-                            kf[jt][ks] =
-                                *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
-#pragma unroll
-                    for (int ib = 0; ib < IB; ++ib)
-#pragma unroll
-                        for (int jt = 0; jt < 4; ++jt) {
-                            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                            for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ib][ks], acc);
-                            const int d0 = 16 * (jt - (IB * w + ib)) + 4 * g - m;  // key pos - query pos at r = 0
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) {
-                                const bool keep = reversed ? (d0 + r >= 0) : (d0 + r <= 0);
-                                acc[r] = keep ? acc[r] : 0.f;
-                            }
-                            pk[ib][jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
-                        }
-                }
-
-                const int orow = row0 + 16 * IB * w + m;
-                constexpr int JBmax = (IB == 1) ? 8 : 4;
-                constexpr int JB = (JBmax / TL::KS < 1) ? 1 : ((JBmax / TL::KS < TL::NJT) ? (JBmax / TL::KS) : TL::NJT);
-#pragma unroll
-                for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
-                    u32x4 vf[JB][2], sf[JB][TL::KS];
-#pragma unroll
-                    for (int jj = 0; jj < JB; ++jj) {
-                        const int jt = j0 + jj;
-#pragma unroll
-                        for (int kb = 0; kb < 2; ++kb)
-                            vf[jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
-                                             lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
-#pragma unroll
-                        for (int ks = 0; ks < TL::KS; ++ks)
-                            sf[jj][ks] =
-                                *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
-                    }
-#pragma unroll
-                    for (int ib = 0; ib < IB; ++ib)
-#pragma unroll
-                        for (int jj = 0; jj < JB; ++jj) {
-                            const int jt = j0 + jj;
-                            f32x4 o = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                            for (int kb = 0; kb < 2; ++kb)
-                                o = TR::mfma(vf[jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
-#pragma unroll
-                            for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ib][ks], o);
-                            const int col = 16 * jt + 4 * g;
-                            const uint32_t off =
-                                (col < dj) ? (uint32_t)((orow + 16 * ib) * ldc + col) * 2u : kOobOffset;
-                            buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
-                        }
-                }
-                __syncthreads();
-            }
+// Gradient launch for square head dims: two kinds of workgroup in one grid of 4 + 4 + LW wavefronts.
+//   * a plain problem (dQ): four output wavefronts of one block each, as in scan_kernel;
+//   * a PAIR of problems X = G(A, B, C) and Y = G(A2, C, B) that scan the same way (dK = G(V, dO, Q) and
+//     dV = G(K, Q, dO)): their tiles are the same two tiles with the roles swapped and their states are
+//     transposes of each other, so one workgroup stages the tiles once, carries the state once (publishing
+//     both orientations) and gives two output wavefronts of two blocks to each problem.
+// This puts the three gradients of a head on two workgroups instead of three, i.e. 2*BH workgroups:
+// one per CU at the headline shape instead of one and a half.
+// OWP = output wavefronts per problem of a pair (2 of two blocks, or 4 of one block); a plain problem
+// always uses four of one block and leaves the other OWP*2 - 4 output wavefronts idle at the barriers.
+template <class TR, int D, int PF, int LW, int OWP>
+__global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(ProblemSet set, int BH, int N, int nchunks,
+                                                                            int cpg, int G) {
+    using TL = Tiling<D, D>;
+    static_assert(TL::BS == TL::CS, "the two tiles are read both ways");
+    static_assert(OWP == 2 || OWP == 4, "two or four output wavefronts per problem");
+    constexpr int NOUT = 2 * OWP, IBP = 4 / OWP;
+    constexpr int LT = 64 * LW;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = D * TL::SS;
+    __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
+    __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
+    __shared__ __attribute__((aligned(16))) u16 sS[2 * SSZ];
+    __shared__ __attribute__((aligned(16))) u16 sS2[2 * SSZ];
+    const int l = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const WorkItem wi = decode_workgroup(set.count, G);
+    if (wi.bh >= BH) return;
+    const Problem &pr = set.p[wi.prob];
+    const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
+    const bool pair = pr.A2 != nullptr;
+    ScanRange r;
+    r.N = N;
+    r.nchunks = nchunks;
+    r.p0 = wi.grp * cpg;
+    r.p1 = min(r.p0 + cpg, nchunks);
+    r.reversed = pr.reversed;
+    const float *seed = pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr;
+    if (wv >= NOUT + 4) {
+        loader_role<D, D, PF, LT>(pr.B + (size_t)wi.bh * N * di, pr.C + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
+                                  (int)threadIdx.x - 64 * (NOUT + 4), sB, sC);
+    } else if (wv >= NOUT) {
+        if (pair)
+            state_role<TR, D, D, true>(seed, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, sS2);
+        else
+            state_role<TR, D, D, false>(seed, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, nullptr);
+    } else if (!pair) {
+        if (wv < 4) {
+            output_role<TR, D, D, PF, 1>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
+                                         wv, l, sB, sC, sS);
+        } else {
+            for (int p = r.p0 - 1; p < r.p1; ++p) __syncthreads();  // idle: keep the barrier count
         }
+    } else if (wv < OWP) {
+        output_role<TR, D, D, PF, IBP>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
+                                       IBP * wv, l, sB, sC, sS);
+    } else {
+        // Y: contracted dim dj of X, output dim di of X; its row-read tile is X's C tile and vice versa
+        output_role<TR, D, D, PF, IBP>(pr.A2 + (size_t)wi.bh * N * dj, pr.O2 + (size_t)wi.bh * N * di, dj, di, di, r,
+                                       IBP * (wv - OWP), l, sC, sB, sS2);
     }
 }
 
