@@ -422,10 +422,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
             }
 
             const int orow = row0 + 16 * blk0 + m;
-#ifndef COTT_JB2
-#define COTT_JB2 4
-#endif
-            constexpr int JBmax = (IB == 1) ? 8 : COTT_JB2;
+            constexpr int JBmax = (IB == 1) ? 8 : 4;
             constexpr int JB = (JBmax / TL::KS < 1) ? 1 : ((JBmax / TL::KS < TL::NJT) ? (JBmax / TL::KS) : TL::NJT);
 #pragma unroll
             for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
