@@ -64,6 +64,7 @@ struct Tiling {
     static constexpr int TPW = NIT * NJT / 4;    // fp32 state tiles owned by one wavefront
     static constexpr int KS = DI / 32;           // MFMA k-steps over i
     static constexpr int STATE_FLOATS = DI * DJ;
+    static constexpr int OS = DJ + 8;            // ... of a staged output tile [64][DJ] (8-byte writes, 16-byte reads)
 };
 
 // Workgroup -> (head, problem, group).  Linear id i runs on XCD i % 8; per XCD the ids are ordered
@@ -253,13 +254,41 @@ struct ScanRange {
 };
 
 // Loader role: LT threads stage the B tile (rows of di) and the C tile (dj columns of rows of ldc).
+// Output tiles staged in LDS by the output wavefronts (see output_role) and written to memory by the loader
+// wavefronts one chunk later: up to two tiles per chunk (the problems of a pair), each [64][DJ] with row
+// stride Tiling::OS, double-buffered; O[i] null = no such tile.
+struct StagedOut {
+    u16 *O[2];      // head base of each output tensor
+    int dj[2], ld[2];
+    const u16 *sO;  // [2 buffers][2 tiles][64 * OS]
+};
+
 template <int DI, int DJ, int PF, int LT>
 __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head, int di, int dj, int ldc,
-                                            const ScanRange &r, int tid, u16 *sB, u16 *sC) {
+                                            const ScanRange &r, int tid, u16 *sB, u16 *sC,
+                                            const StagedOut *so = nullptr) {
     using TL = Tiling<DI, DJ>;
-    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SO = kChunk * TL::OS;
     const rsrc_t rB = make_rsrc(B_head, (uint32_t)r.N * di * 2u);
     const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
+    // the staged tile(s) of chunk p (scan order): 16-byte row segments, rows past N dropped by the range check
+    auto write_out = [&](int p) {
+        const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (so->O[t] == nullptr) continue;
+            const rsrc_t rO = make_rsrc(so->O[t], ((uint32_t)(r.N - 1) * so->ld[t] + so->dj[t]) * 2u);
+            const u16 *tile = so->sO + (((p - r.p0) & 1) * 2 + t) * SO;
+#pragma unroll
+            for (int u = 0; u < 8 * DJ / LT; ++u) {
+                const int v = tid + LT * u;
+                const int row = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+                const u32x4 val = *reinterpret_cast<const u32x4 *>(tile + row * TL::OS + col);
+                const uint32_t off = (col < so->dj[t]) ? (uint32_t)((row0 + row) * so->ld[t] + col) * 2u : kOobOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(val, rO, (int)off, 0, 0);
+            }
+        }
+    };
     u32x4 rb[PF][8 * DI / LT], rc[PF][8 * DJ / LT];
     auto load_chunk = [&](int s, int p) {
         const int pc = min(p, r.p1 - 1);
@@ -277,13 +306,17 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
 #pragma unroll
         for (int s = 0; s < PF; ++s) {
             const int p = pb + s;
-            if (p >= r.p1) return;  // uniform over the workgroup
+            if (p >= r.p1) {  // uniform over the workgroup
+                if (so != nullptr && r.p1 > r.p0) write_out(r.p1 - 1);
+                return;
+            }
             const int s1 = (s + 1) % PF;
             const int buf = (p - r.p0) & 1;
             // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
             store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
             store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
             load_chunk(s1, p + 1 + PF);
+            if (so != nullptr && p > r.p0) write_out(p - 1);
             __syncthreads();
         }
     }
@@ -357,9 +390,13 @@ __device__ __forceinline__ void state_role(const float *seed, const float *sin, 
 // Output role: one wavefront, IB blocks of 16 positions starting at block `blk0` of each chunk.
 // cB: tile read by rows (the B operand of this problem), cC: tile read by columns (its C operand),
 // cS: its 16-bit state; all three double-buffered with the strides of Tiling<DI, DJ>.
+// sOt: null = store the outputs to memory from here; else the [2 buffers] of this problem's staged output tile
+// (buffer stride 2 * 64 * OS), written with 8-byte LDS stores and sent to memory by the loader wavefronts, so that
+// this wavefront's chain of LDS reads and MFMAs never waits for the vector-memory pipeline to take a store.
 template <class TR, int DI, int DJ, int PF, int IB>
 __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int ldc, const ScanRange &r,
-                                            int blk0, int l, const u16 *sB, const u16 *sC, const u16 *sS) {
+                                            int blk0, int l, const u16 *sB, const u16 *sC, const u16 *sS,
+                                            u16 *sOt = nullptr) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
@@ -450,8 +487,14 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 #pragma unroll
                         for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ib][ks], o);
                         const int col = 16 * jt + 4 * g;
-                        const uint32_t off = (col < dj) ? (uint32_t)((orow + 16 * ib) * ldc + col) * 2u : kOobOffset;
-                        buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
+                        const u32x2 val = {TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
+                        if (sOt != nullptr) {
+                            *reinterpret_cast<u32x2 *>(sOt + buf * (2 * kChunk * TL::OS) +
+                                                       (16 * (blk0 + ib) + m) * TL::OS + col) = val;
+                        } else {
+                            const uint32_t off = (col < dj) ? (uint32_t)((orow + 16 * ib) * ldc + col) * 2u : kOobOffset;
+                            buf_store8(rO, off, val);
+                        }
                     }
             }
             __syncthreads();
@@ -522,6 +565,7 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
     __shared__ __attribute__((aligned(16))) u16 sS[2 * SSZ];
     __shared__ __attribute__((aligned(16))) u16 sS2[2 * SSZ];
+    __shared__ __attribute__((aligned(16))) u16 sO[2 * 2 * kChunk * TL::OS];
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const WorkItem wi = decode_workgroup(set.count, G);
@@ -529,6 +573,7 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
     const bool pair = pr.A2 != nullptr;
+    constexpr int SO = kChunk * TL::OS;
     ScanRange r;
     r.N = N;
     r.nchunks = nchunks;
@@ -537,8 +582,16 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     r.reversed = pr.reversed;
     const float *seed = pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr;
     if (wv >= NOUT + 4) {
+        StagedOut so;
+        so.O[0] = pr.O + (size_t)wi.bh * N * ldc;
+        so.dj[0] = dj;
+        so.ld[0] = ldc;
+        so.O[1] = pair ? pr.O2 + (size_t)wi.bh * N * di : nullptr;
+        so.dj[1] = di;
+        so.ld[1] = di;
+        so.sO = sO;
         loader_role<D, D, PF, LT>(pr.B + (size_t)wi.bh * N * di, pr.C + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
-                                  (int)threadIdx.x - 64 * (NOUT + 4), sB, sC);
+                                  (int)threadIdx.x - 64 * (NOUT + 4), sB, sC, &so);
     } else if (wv >= NOUT) {
         if (pair)
             state_role<TR, D, D, true>(seed, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, sS2);
@@ -547,17 +600,17 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     } else if (!pair) {
         if (wv < 4) {
             output_role<TR, D, D, PF, 1>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
-                                         wv, l, sB, sC, sS);
+                                         wv, l, sB, sC, sS, sO);
         } else {
             for (int p = r.p0 - 1; p < r.p1; ++p) __syncthreads();  // idle: keep the barrier count
         }
     } else if (wv < OWP) {
         output_role<TR, D, D, PF, IBP>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
-                                       IBP * wv, l, sB, sC, sS);
+                                       IBP * wv, l, sB, sC, sS, sO);
     } else {
         // Y: contracted dim dj of X, output dim di of X; its row-read tile is X's C tile and vice versa
         output_role<TR, D, D, PF, IBP>(pr.A2 + (size_t)wi.bh * N * dj, pr.O2 + (size_t)wi.bh * N * di, dj, di, di, r,
-                                       IBP * (wv - OWP), l, sC, sB, sS2);
+                                       IBP * (wv - OWP), l, sC, sB, sS2, sO + SO);
     }
 }
 
