@@ -431,6 +431,27 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                     qc[ib][ks] = (32 * ks + 8 * g < di) ? qn[s][ib][ks] : u32x4{0u, 0u, 0u, 0u};
             load_q(s, p + PF);
 
+            // Operand fragments of the output products come in batches of JB column tiles; the reads of a batch are
+            // issued one batch ahead (the first before the score products), so their LDS latency runs under MFMAs.
+            constexpr int JBmax = (IB == 1) ? 8 : 4;
+            constexpr int JB = (JBmax / TL::KS < 1) ? 1 : ((JBmax / TL::KS < TL::NJT) ? (JBmax / TL::KS) : TL::NJT);
+            constexpr int NBATCH = TL::NJT / JB;
+            u32x4 vf[2][JB][2], sf[2][JB][TL::KS];
+            auto read_batch = [&](int slot, int j0) {
+#pragma unroll
+                for (int jj = 0; jj < JB; ++jj) {
+                    const int jt = j0 + jj;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+                        vf[slot][jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
+                                               lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        sf[slot][jj][ks] =
+                            *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
+                }
+            };
+
             // masked scores, transposed: pk[ib][jt] = P^T[16jt+4g .. +3][16(blk0+ib)+m]; fragment
             // reads first, MFMAs after, so the LDS latency is paid once per batch
             u32x2 pk[IB][4];
@@ -441,6 +462,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 #pragma unroll
                     for (int ks = 0; ks < TL::KS; ++ks)
                         kf[jt][ks] = *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
+                read_batch(0, 0);
 #pragma unroll
                 for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
@@ -459,22 +481,10 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
             }
 
             const int orow = row0 + 16 * blk0 + m;
-            constexpr int JBmax = (IB == 1) ? 8 : 4;
-            constexpr int JB = (JBmax / TL::KS < 1) ? 1 : ((JBmax / TL::KS < TL::NJT) ? (JBmax / TL::KS) : TL::NJT);
 #pragma unroll
-            for (int j0 = 0; j0 < TL::NJT; j0 += JB) {
-                u32x4 vf[JB][2], sf[JB][TL::KS];
-#pragma unroll
-                for (int jj = 0; jj < JB; ++jj) {
-                    const int jt = j0 + jj;
-#pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
-                        vf[jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
-                                         lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
-#pragma unroll
-                    for (int ks = 0; ks < TL::KS; ++ks)
-                        sf[jj][ks] = *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
-                }
+            for (int bt = 0; bt < NBATCH; ++bt) {
+                const int j0 = bt * JB, slot = bt & 1;
+                if (bt + 1 < NBATCH) read_batch(slot ^ 1, j0 + JB);
 #pragma unroll
                 for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
@@ -483,9 +493,9 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                         f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int kb = 0; kb < 2; ++kb)
-                            o = TR::mfma(vf[jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
+                            o = TR::mfma(vf[slot][jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
 #pragma unroll
-                        for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jj][ks], qc[ib][ks], o);
+                        for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[slot][jj][ks], qc[ib][ks], o);
                         const int col = 16 * jt + 4 * g;
                         const u32x2 val = {TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
                         if (sOt != nullptr) {
