@@ -74,7 +74,8 @@ class PrepareInputs(torch.autograd.Function):
         ctx.save_for_backward(q, k, v, keep, cnt, sig, rot_table, position_ids)
         ctx.bnhd = bool(bnhd)
         rotary = (rot_table, position_ids) if rot_table is not None else None
-        return ops.prepare_inputs(q, k, v, keep, cnt, sig, out_dtype, rotary=rotary, bnhd=bnhd)
+        # positions are not read back here (that would stall the launch queue): the kernel clamps them to the table
+        return ops.prepare_inputs(q, k, v, keep, cnt, sig, out_dtype, rotary=rotary, bnhd=bnhd, check_positions=False)
 
     @staticmethod
     def backward(ctx, gq, gk, gv):
@@ -82,7 +83,8 @@ class PrepareInputs(torch.autograd.Function):
         want = sig is not None and ctx.needs_input_grad[5]
         rotary = (rot_table, position_ids) if rot_table is not None else None
         dq, dk, dv, dsig = ops.prepare_inputs_backward(q, k, v, gq.contiguous(), gk.contiguous(), gv.contiguous(), keep,
-                                                       cnt, sig, want_dsig=want, rotary=rotary, bnhd=ctx.bnhd)
+                                                       cnt, sig, want_dsig=want, rotary=rotary, bnhd=ctx.bnhd,
+                                                       check_positions=False)
         if dsig is not None:
             dsig = dsig.to(sig.dtype)
         return dq, dk, dv, None, None, dsig, None, None, None, None

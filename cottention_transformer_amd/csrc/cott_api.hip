@@ -491,7 +491,7 @@ int cott_prep_ex_fwd(const void *q, const void *k, const void *v, void *q_out, v
     void *y[3] = {q_out, k_out, v_out};
     hipError_t e = cott::launch_prep(false, x, nullptr, y, keep, cnt, sig, nullptr, B, H, N, Dk, Dv, in_dtype, out_dtype,
                                      out_dtype, 1e-12f, in_bnhd ? 1 : 0, rot_table, pos, rot_table ? rotary_dim : 0,
-                                     static_cast<hipStream_t>(stream));
+                                     table_rows, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
     return COTT_OK;
 }
@@ -514,7 +514,7 @@ int cott_prep_ex_bwd(const void *q, const void *k, const void *v, const void *gq
     void *y[3] = {dq, dk, dv};
     hipError_t e = cott::launch_prep(true, x, g, y, keep, cnt, sig, dsig_rows, B, H, N, Dk, Dv, in_dtype, in_dtype,
                                      grad_dtype, 1e-12f, in_bnhd ? 1 : 0, rot_table, pos, rot_table ? rotary_dim : 0,
-                                     static_cast<hipStream_t>(stream));
+                                     table_rows, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
     return COTT_OK;
 }

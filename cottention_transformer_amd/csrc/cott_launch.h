@@ -74,7 +74,7 @@ bool generic_fits(int dtype, int di);
 hipError_t launch_prep(bool backward, const void *const x[3], const void *const g[3], void *const y[3],
                        const unsigned char *keep, const float *cnt, const float *sig, float *dsig_rows, int B, int H, int N,
                        int dk, int dv, int x_dtype, int y_dtype, int g_dtype, float eps, int x_bnhd, const float *rot,
-                       const long long *pos, int R, hipStream_t stream);
+                       const long long *pos, int R, int table_rows, hipStream_t stream);
 
 hipError_t launch_decode(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH,
                          int dk, int dv, hipStream_t stream);

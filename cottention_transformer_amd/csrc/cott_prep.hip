@@ -106,8 +106,8 @@ struct PrepArgs {
     // (B,H,N,D), and the GPT-J rotary embedding applied to the first R columns of q and k.
     int x_bnhd;           // 1: x (and, backward, y) are (B,N,H,D); g (backward) / y (forward) stay (B,H,N,D)
     const float *rot;     // (P,R) table, row p = [sin(p f_0..f_{R/2-1}) | cos(...)], or null
-    const long long *pos; // (B,N) row of the table per position
-    int R;
+    const long long *pos; // (B,N) row of the table per position (clamped to the table)
+    int R, table_rows;
 };
 
 // Rotates the pairs (v[0],v[1]) and (v[2],v[3]) by +angle (inverse = false) or -angle.
@@ -175,7 +175,9 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
         const long b = bh / a.H;
         const ACC keep = (a.keep == nullptr || a.keep[b * a.N + s] != 0) ? (ACC)1 : (ACC)0;
         const bool rotary = t < 2 && a.rot != nullptr;
-        const float *sc = rotary ? a.rot + (size_t)a.pos[b * a.N + s] * a.R : nullptr;
+        long long tp = rotary ? a.pos[b * a.N + s] : 0;
+        tp = tp < 0 ? 0 : (tp >= a.table_rows ? a.table_rows - 1 : tp);  // never read outside the table
+        const float *sc = rotary ? a.rot + (size_t)tp * a.R : nullptr;
         // y = keep R x / |R x| with R the block rotation built from the table (orthogonal only up to the table's
         // rounding, so the norm is taken after the rotation).  Backward: dx = R^T J^T g with J the Jacobian of
         // the normalisation at x' = R x: the usual combination of g and x', rotated back at the end.
@@ -256,8 +258,9 @@ int lanes_per_row(int d) {
 hipError_t launch_prep(bool backward, const void *const x[3], const void *const g[3], void *const y[3],
                        const uint8_t *keep, const float *cnt, const float *sig, float *dsig_rows, int B, int H, int N,
                        int dk, int dv, int x_dtype, int y_dtype, int g_dtype, float eps, int x_bnhd, const float *rot,
-                       const long long *pos, int R, hipStream_t stream) {
+                       const long long *pos, int R, int table_rows, hipStream_t stream) {
     PrepArgs a;
+    a.table_rows = table_rows > 0 ? table_rows : 1;
     a.x_bnhd = x_bnhd;
     a.rot = rot;
     a.pos = pos;

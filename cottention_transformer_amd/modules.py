@@ -120,7 +120,8 @@ class GPTCosAttention(nn.Module):
             # value scaling by absolute position (:223), then the recurrence (:253-272) from the stored state
             cnt = (self.cur_s + torch.arange(s, device=query.device, dtype=torch.float32)).expand(b, s)
             dt = query.dtype
-            q, k, v = ops.prepare_inputs(query, key, value, keep, cnt, sig, out_dtype=dt, rotary=rotary, bnhd=bnhd)
+            q, k, v = ops.prepare_inputs(query, key, value, keep, cnt, sig, out_dtype=dt, rotary=rotary, bnhd=bnhd,
+                                         check_positions=False)
             if self.state is None:
                 self.state = torch.zeros(b, h, q.shape[-1], v.shape[-1], device=q.device,
                                          dtype=torch.float64 if dt == torch.float64 else torch.float32)

@@ -223,7 +223,7 @@ def _prep_shapes(q, k, v, bnhd):
     return _shapes(q, k, v)
 
 
-def _rotary_args(rotary, b, n, dk, device):
+def _rotary_args(rotary, b, n, dk, device, check=True):
     if rotary is None:
         return None, None, 0, 0
     table, pos = rotary
@@ -231,14 +231,17 @@ def _rotary_args(rotary, b, n, dk, device):
         raise RuntimeError("rotary table must be (positions, rotary_dim), rotary_dim a multiple of 4 and <= Dk")
     if pos.shape != (b, n):
         raise RuntimeError(f"position ids must have shape {(b, n)}")
-    if pos.numel() and (int(pos.max()) >= table.size(0) or int(pos.min()) < 0):
+    # (this check reads the positions back and so waits for the device; callers in a hot loop pass check=False,
+    # the kernel then clamps stray positions to the table)
+    if check and pos.numel() and (int(pos.max()) >= table.size(0) or int(pos.min()) < 0):
         raise RuntimeError("position id outside the rotary table")
     table = table.to(device=device, dtype=torch.float32).contiguous()
     pos = pos.to(device=device, dtype=torch.int64).contiguous()
     return table, pos, table.size(1), table.size(0)
 
 
-def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None, rotary=None, bnhd=False):
+def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None, rotary=None, bnhd=False,
+                   check_positions=True):
     """Fused input preparation of the cosine-attention module, one pass per tensor:
         q_out = keep * q / max(|q|, 1e-12),  k_out likewise,  v_out = keep * v / max(cnt ** sig[h], 1)
     converted to `out_dtype` (default: the input dtype) and returned as (B,H,N,D).  Replaces
@@ -257,7 +260,7 @@ def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None, rotar
     if out_dtype not in _DTYPES:
         raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
     keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
-    table, pos, rdim, rows = _rotary_args(rotary, b, n, dk, q.device)
+    table, pos, rdim, rows = _rotary_args(rotary, b, n, dk, q.device, check_positions)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     qo, ko = (torch.empty((b, h, n, dk), dtype=out_dtype, device=q.device) for _ in range(2))
     vo = torch.empty((b, h, n, dv), dtype=out_dtype, device=q.device)
@@ -271,7 +274,7 @@ def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None, rotar
 
 
 def prepare_inputs_backward(q, k, v, gq, gk, gv, keep=None, cnt=None, sig=None, want_dsig=False, rotary=None,
-                            bnhd=False):
+                            bnhd=False, check_positions=True):
     """Gradients of `prepare_inputs` with respect to q, k, v (their dtype and layout) and, if asked, to sig (H,).
     gq, gk, gv: gradients with respect to the outputs, (B,H,N,D)."""
     _require_gpu(Q=q, K=k, V=v, gq=gq, gk=gk, gv=gv)
@@ -282,7 +285,7 @@ def prepare_inputs_backward(q, k, v, gq, gk, gv, keep=None, cnt=None, sig=None, 
         raise RuntimeError("q, k, v share one dtype and their gradients share one dtype")
     code, gcode = _dtype_code(q), _dtype_code(gq)
     keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
-    table, pos, rdim, rows = _rotary_args(rotary, b, n, dk, q.device)
+    table, pos, rdim, rows = _rotary_args(rotary, b, n, dk, q.device, check_positions)
     q, k, v, gq, gk, gv = (t.contiguous() for t in (q, k, v, gq, gk, gv))
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     drows = torch.empty((b, h, n), dtype=torch.float32, device=q.device) if (want_dsig and sig is not None) else None

@@ -131,8 +131,8 @@ COTT_API int cott_prep_bwd(const void *q, const void *k, const void *v,
  * (the outputs / incoming gradients stay (B,H,N,D)), which removes the permute + contiguous copies of :474-475 and
  * Custom_Kernel.py:11-13;  rot_table != NULL: the GPT-J rotary embedding (apply_rotary_pos_emb, :463-472) is
  * applied to the first rotary_dim columns of q and k before normalisation.  rot_table: (table_rows, rotary_dim)
- * fp32, row p = [sin(p f_i) | cos(p f_i)]; pos: (B,N) int64 row index per position (must be < table_rows; not
- * checked on the device). */
+ * fp32, row p = [sin(p f_i) | cos(p f_i)]; pos: (B,N) int64 row index per position; an index outside [0, table_rows) is clamped
+ * to the table on the device, nothing reports it. */
 COTT_API int cott_prep_ex_fwd(const void *q, const void *k, const void *v, void *q_out, void *k_out, void *v_out,
                      const unsigned char *keep, const float *cnt, const float *sig,
                      const float *rot_table, const long long *pos, int rotary_dim, int table_rows, int in_bnhd,

@@ -426,6 +426,12 @@ def test_input_preparation_with_rotary_and_projection_layout(ct, case):
     assert rel_l2(dsig, grads[3].numpy()) <= max(tol, 1e-4)
     with pytest.raises(RuntimeError):
         ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), rotary=(table.to(DEV), (pos + 300).to(DEV)), bnhd=True)
+    # without the host-side check a stray position is clamped to the table by the kernel, never read out of bounds
+    far = pos.clone(); far[0, 0] = 10 ** 9; far[0, 1] = -5
+    clamped = far.clamp(0, 299)
+    a1 = ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), rotary=(table.to(DEV), far.to(DEV)), bnhd=True, check_positions=False)
+    a2 = ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), rotary=(table.to(DEV), clamped.to(DEV)), bnhd=True)
+    assert all(torch.equal(x, y) for x, y in zip(a1, a2))
 
 
 def test_calls_can_be_captured_in_a_hip_graph_and_replayed(ct, oracle):
