@@ -110,12 +110,16 @@ struct PrepArgs {
     int R, table_rows;
 };
 
-// Rotates the pairs (v[0],v[1]) and (v[2],v[3]) by +angle (inverse = false) or -angle.
+// Rotates the pairs (v[0],v[1]) and (v[2],v[3]) by +angle (inverse = false) or -angle.  sc points at the sine of
+// the first pair; the two sines and, `half` floats further, the two cosines are each one 8-byte load (the column
+// of a lane's group is a multiple of 4, so both are 8-byte aligned).
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 template <class ACC>
 __device__ __forceinline__ void rotate4(Vec4<ACC> &v, const float *sc, int half, bool inverse) {
+    const f32x2 sn = *reinterpret_cast<const f32x2 *>(sc), cs = *reinterpret_cast<const f32x2 *>(sc + half);
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-        const ACC s = inverse ? -(ACC)sc[p] : (ACC)sc[p], c = (ACC)sc[half + p];
+        const ACC s = inverse ? -(ACC)sn[p] : (ACC)sn[p], c = (ACC)cs[p];
         const ACC e = v.x[2 * p], o = v.x[2 * p + 1];
         v.x[2 * p] = e * c - o * s;
         v.x[2 * p + 1] = o * c + e * s;
