@@ -110,13 +110,11 @@ struct PrepArgs {
     int R, table_rows;
 };
 
-// Rotates the pairs (v[0],v[1]) and (v[2],v[3]) by +angle (inverse = false) or -angle.  sc points at the sine of
-// the first pair; the two sines and, `half` floats further, the two cosines are each one 8-byte load (the column
-// of a lane's group is a multiple of 4, so both are 8-byte aligned).
+// Rotates the pairs (v[0],v[1]) and (v[2],v[3]) by +angle (inverse = false) or -angle; sn and cs hold the sines
+// and cosines of the two pairs.
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 template <class ACC>
-__device__ __forceinline__ void rotate4(Vec4<ACC> &v, const float *sc, int half, bool inverse) {
-    const f32x2 sn = *reinterpret_cast<const f32x2 *>(sc), cs = *reinterpret_cast<const f32x2 *>(sc + half);
+__device__ __forceinline__ void rotate4(Vec4<ACC> &v, f32x2 sn, f32x2 cs, bool inverse) {
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
         const ACC s = inverse ? -(ACC)sn[p] : (ACC)sn[p], c = (ACC)cs[p];
@@ -126,13 +124,33 @@ __device__ __forceinline__ void rotate4(Vec4<ACC> &v, const float *sc, int half,
     }
 }
 
-__device__ __forceinline__ float pow_pos(float c, float s) { return c > 0.f ? expf(s * logf(c)) : 0.f; }
+// (hardware exp2 / log2: about 1e-6 relative, far inside the fp32 tolerance of the op)
+__device__ __forceinline__ float pow_pos(float c, float s) { return c > 0.f ? __expf(s * __logf(c)) : 0.f; }
 __device__ __forceinline__ double pow_pos(double c, double s) { return c > 0.0 ? exp(s * log(c)) : 0.0; }
+
+// row = (b*H + h)*N + s.  Row counts below 2^32 (every realistic shape) take 32-bit divisions, which cost a
+// fraction of the 64-bit ones.
+__device__ __forceinline__ void split_row(long row, const PrepArgs &a, int &s, int &h, int &b) {
+    if (a.rows <= 0xffffffffL) {
+        const uint32_t r = (uint32_t)row, bh = r / (uint32_t)a.N;
+        s = (int)(r - bh * (uint32_t)a.N);
+        b = (int)(bh / (uint32_t)a.H);
+        h = (int)(bh - (uint32_t)b * (uint32_t)a.H);
+    } else {
+        const long bh = row / a.N;
+        s = (int)(row % a.N);
+        h = (int)(bh % a.H);
+        b = (int)(bh / a.H);
+    }
+}
 
 // blockIdx.y selects the tensor (0 q, 1 k, 2 v).  A row of D elements lives in lpr consecutive
 // lanes, 4 elements per lane and group; groups c = 0..NV-1 cover D up to 4*64*NV.  Each lane group
 // handles R rows (row, row + stride, ...) whose loads are all issued before the first use, so that
-// enough bytes are in flight per wavefront to cover the memory latency.
+// enough bytes are in flight per wavefront to cover the memory latency.  For head-sized rows the kernel is
+// limited by instruction issue, not by bytes: the per-row work (index split, norm, division) is repeated by
+// every lane of the row, so two groups per lane (half as many wavefronts) are faster than one, while more
+// rows or groups per lane only cost registers.
 template <class ACC, bool BACKWARD, int NV, int R>
 __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
     const int t = blockIdx.y;
@@ -146,15 +164,29 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
     long rr[R];
     size_t xoff[R];
     bool act[R];
+    const bool rotary = t < 2 && a.rot != nullptr;
+    const bool side = t == 2 && a.cnt != nullptr && a.sig != nullptr;
+    // Three rounds of loads, all issued before the first use: the per-row side inputs, the rows themselves, then
+    // the table entries (which need the positions of the first round, back long before the rows are).
+    uint8_t keep_in[R];
+    long long pos_in[R];
+    float cnt_in[R], sig_in[R];
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const long row = row0 + (long)u * rpb;
         act[u] = row < a.rows;
         rr[u] = act[u] ? row : 0;
-        {
-            const long bh_ = rr[u] / a.N, s_ = rr[u] % a.N;
-            xoff[u] = a.x_bnhd ? (size_t)(((bh_ / a.H) * a.N + s_) * a.H + bh_ % a.H) * D : (size_t)rr[u] * D;
-        }
+        int sq, hq, bq;  // position, head, batch element of the row
+        split_row(rr[u], a, sq, hq, bq);
+        xoff[u] = a.x_bnhd ? (size_t)(((long)bq * a.N + sq) * a.H + hq) * D : (size_t)rr[u] * D;
+        const long tok = (long)bq * a.N + sq;
+        keep_in[u] = a.keep != nullptr ? a.keep[tok] : (uint8_t)1;
+        pos_in[u] = rotary ? a.pos[tok] : 0;
+        cnt_in[u] = side ? a.cnt[tok] : 0.f;
+        sig_in[u] = side ? a.sig[hq] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
 #pragma unroll
         for (int c = 0; c < NV; ++c) {
             const int col = 4 * (lane + c * lpr);
@@ -170,18 +202,28 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
             }
         }
     }
+    // sines and cosines of a lane's pairs: two 8-byte loads per group (its column is a multiple of 4)
+    f32x2 sn[R][NV], cs[R][NV];
+    if (rotary) {
+#pragma unroll
+        for (int u = 0; u < R; ++u) {
+            long long tp = pos_in[u];
+            tp = tp < 0 ? 0 : (tp >= a.table_rows ? a.table_rows - 1 : tp);  // never read outside the table
+            const float *sc = a.rot + (size_t)tp * a.R;
+#pragma unroll
+            for (int c = 0; c < NV; ++c) {
+                const int col = 4 * (lane + c * lpr);
+                if (col < a.R) {
+                    sn[u][c] = *reinterpret_cast<const f32x2 *>(sc + col / 2);
+                    cs[u][c] = *reinterpret_cast<const f32x2 *>(sc + col / 2 + a.R / 2);
+                }
+            }
+        }
+    }
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const long r = rr[u];
-        const int s = (int)(r % a.N);
-        const long bh = r / a.N;
-        const int h = (int)(bh % a.H);
-        const long b = bh / a.H;
-        const ACC keep = (a.keep == nullptr || a.keep[b * a.N + s] != 0) ? (ACC)1 : (ACC)0;
-        const bool rotary = t < 2 && a.rot != nullptr;
-        long long tp = rotary ? a.pos[b * a.N + s] : 0;
-        tp = tp < 0 ? 0 : (tp >= a.table_rows ? a.table_rows - 1 : tp);  // never read outside the table
-        const float *sc = rotary ? a.rot + (size_t)tp * a.R : nullptr;
+        const ACC keep = keep_in[u] != 0 ? (ACC)1 : (ACC)0;
         // y = keep R x / |R x| with R the block rotation built from the table (orthogonal only up to the table's
         // rounding, so the norm is taken after the rotation).  Backward: dx = R^T J^T g with J the Jacobian of
         // the normalisation at x' = R x: the usual combination of g and x', rotated back at the end.
@@ -189,7 +231,7 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
 #pragma unroll
             for (int c = 0; c < NV; ++c) {
                 const int col = 4 * (lane + c * lpr);
-                if (col < a.R) rotate4(x[u][c], sc + col / 2, a.R / 2, false);
+                if (col < a.R) rotate4(x[u][c], sn[u][c], cs[u][c], false);
             }
         }
         ACC ss = 0, dot = 0;
@@ -218,8 +260,8 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
             bool scaled = false;
             ACC c = 0;
             if (a.cnt != nullptr && a.sig != nullptr) {
-                c = (ACC)a.cnt[b * a.N + s];
-                const ACC p = pow_pos(c, (ACC)a.sig[h]);
+                c = (ACC)cnt_in[u];
+                const ACC p = pow_pos(c, (ACC)sig_in[u]);
                 if (p > (ACC)1) {
                     scale = (ACC)1 / p;
                     scaled = true;
@@ -244,16 +286,16 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     y.x[i] = BACKWARD ? mul_g * g[u][c].x[i] + mul_x * x[u][c].x[i] : mul_x * x[u][c].x[i];
-                if (BACKWARD && rotary && col < a.R) rotate4(y, sc + col / 2, a.R / 2, true);
+                if (BACKWARD && rotary && col < a.R) rotate4(y, sn[u][c], cs[u][c], true);
                 store4<ACC>(a.y[t], BACKWARD ? a.x_dtype : a.y_dtype, (BACKWARD ? xoff[u] : (size_t)r * D) + col, y);
             }
         }
     }
 }
 
-int lanes_per_row(int d) {
+int lanes_per_row(int d, int nv) {
     int l = 1;
-    while (4 * l < d && l < 64) l <<= 1;
+    while (4 * nv * l < d && l < 64) l <<= 1;
     return l;
 }
 
@@ -286,13 +328,14 @@ hipError_t launch_prep(bool backward, const void *const x[3], const void *const 
     a.x_dtype = x_dtype;
     a.y_dtype = y_dtype;
     a.g_dtype = g_dtype;
-    a.lpr[0] = a.lpr[1] = lanes_per_row(dk);
-    a.lpr[2] = lanes_per_row(dv);
     a.eps = eps;
     // one grid for the three tensors; rows per block differ per tensor, size x for the largest need
     const int big = dk > dv ? dk : dv;
-    const bool wide = big > 256;              // more than one element group per lane
-    const int rows_per_group = wide ? 1 : 4;
+    const bool wide = big > 256;              // four element groups per lane and one row instead of two and two
+    const int rows_per_group = wide ? 1 : 2;
+    const int nv = wide ? kMaxVec : (big > 4 ? 2 : 1);
+    a.lpr[0] = a.lpr[1] = lanes_per_row(dk, nv);
+    a.lpr[2] = lanes_per_row(dv, nv);
     const int min_rows = rows_per_group * kPrepThreads / (a.lpr[0] > a.lpr[2] ? a.lpr[0] : a.lpr[2]);
     const long blocks = (a.rows + min_rows - 1) / min_rows;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
@@ -302,7 +345,8 @@ hipError_t launch_prep(bool backward, const void *const x[3], const void *const 
 #define COTT_PREP(ACC, BWD) \
     do { \
         if (wide) prep_kernel<ACC, BWD, kMaxVec, 1><<<grid, blk, 0, stream>>>(a); \
-        else prep_kernel<ACC, BWD, 1, 4><<<grid, blk, 0, stream>>>(a); \
+        else if (nv == 2) prep_kernel<ACC, BWD, 2, 2><<<grid, blk, 0, stream>>>(a); \
+        else prep_kernel<ACC, BWD, 1, 2><<<grid, blk, 0, stream>>>(a); \
     } while (0)
     if (backward) {
         if (f64) COTT_PREP(double, true);
