@@ -148,6 +148,47 @@ __device__ __forceinline__ void state_update(f32x4 *S, const u16 *sB, const u16 
 // and store in the loop is unconditional (prefetch past the end of the group re-reads its last
 // chunk), which lets the compiler wait on exactly the stage it needs.
 
+// Runs step(s, p) for p = p0 .. p1-1 with s = (p - p0) % PF a constant after unrolling (s indexes register
+// stages that are reloaded PF chunks ahead).  The control flow is chosen for the wait counts the compiler derives
+// from it, which are the most conservative over all paths into a point, whether they ever run or not:
+//   * whole rounds of PF chunks run in a loop with a single exit and the remainder as straight-line code after
+//     it: an exit test inside the round adds a path from the middle of a round back to its start, on which the
+//     loads issued last look like the ones about to be used;
+//   * the first round runs before the loop, so that the loop is only ever entered with the same loads and stores
+//     in flight as on its back edge (after the prologue alone fewer are, and the oldest look younger).
+// With either path present, a round waits for loads issued one chunk ago instead of PF chunks ago.
+template <int PF, bool EXIT_INSIDE = false, class F>
+__device__ __forceinline__ void run_rounds(int p0, int p1, F &&step) {
+    int pb = p0;
+    if (EXIT_INSIDE) {  // the plain form, for the callers that measured faster with it
+        for (;; pb += PF) {
+#pragma unroll
+            for (int s = 0; s < PF; ++s) {
+                if (pb + s >= p1) return;
+                step(s, pb + s);
+            }
+        }
+    }
+    if (pb + PF <= p1) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) step(s, pb + s);
+        for (pb += PF; pb + PF <= p1; pb += PF) {
+#pragma unroll
+            for (int s = 0; s < PF; ++s) step(s, pb + s);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < PF - 1; ++s)
+        if (pb + s < p1) step(s, pb + s);  // uniform over the workgroup
+}
+
+// The per-chunk barrier; also a fence for the instruction scheduler, which otherwise moves the next chunk's
+// register work (and with it the waits for that chunk's loads) above the barrier.
+__device__ __forceinline__ void chunk_barrier() {
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // Sum of B^T C over each group of chunks, written in register-native order:
 // float4 index (w*TPW + u)*64 + lane of slot (bh*G + grp).  `ngroups` of the G groups are launched
 // (the causal scan never needs the last group's sum).
@@ -191,23 +232,16 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
     load_chunk(0, p0 + PF);
     __syncthreads();
-    for (int pb = p0;; pb += PF) {
-#pragma unroll
-        for (int s = 0; s < PF; ++s) {
-            const int p = pb + s;
-            if (p >= p1) {
-                finish();
-                return;
-            }
-            const int s1 = (s + 1) % PF;
-            const int buf = (p - p0) & 1;
-            store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-            store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
-            load_chunk(s1, p + 1 + PF);
-            state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
-            __syncthreads();
-        }
-    }
+    run_rounds<PF>(p0, p1, [&](int s, int p) {
+        const int s1 = (s + 1) % PF;
+        const int buf = (p - p0) & 1;
+        store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+        store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+        load_chunk(s1, p + 1 + PF);
+        state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+        chunk_barrier();
+    });
+    finish();
 }
 
 // Over the G slots of one head, element-wise: mode 0 -> exclusive prefix in place (slot g gets the
@@ -302,24 +336,17 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
     store_tile<DJ, TL::CS, LT>(sC, rc[0], dj, tid);
     load_chunk(0, r.p0 + PF);
     __syncthreads();
-    for (int pb = r.p0;; pb += PF) {
-#pragma unroll
-        for (int s = 0; s < PF; ++s) {
-            const int p = pb + s;
-            if (p >= r.p1) {  // uniform over the workgroup
-                if (so != nullptr && r.p1 > r.p0) write_out(r.p1 - 1);
-                return;
-            }
-            const int s1 = (s + 1) % PF;
-            const int buf = (p - r.p0) & 1;
-            // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
-            store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-            store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
-            load_chunk(s1, p + 1 + PF);
-            if (so != nullptr && p > r.p0) write_out(p - 1);
-            __syncthreads();
-        }
-    }
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+        const int s1 = (s + 1) % PF;
+        const int buf = (p - r.p0) & 1;
+        // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
+        store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+        store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+        load_chunk(s1, p + 1 + PF);
+        if (so != nullptr && p > r.p0) write_out(p - 1);
+        chunk_barrier();
+    });
+    if (so != nullptr && r.p1 > r.p0) write_out(r.p1 - 1);
 }
 
 // State role (wavefront w of 4).  seed: register-native group prefix or null; sin / sout: row-major
@@ -416,11 +443,10 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_q(s, r.p0 + s);
     __syncthreads();
-    for (int pb = r.p0;; pb += PF) {
-#pragma unroll
-        for (int s = 0; s < PF; ++s) {
-            const int p = pb + s;
-            if (p >= r.p1) return;
+    // (the large tiles keep the exit test inside the round: with 8 column tiles and 4 contraction steps per block
+    // the single-exit form measured 8 % slower there, at D = 128 on long sequences)
+    run_rounds<PF, (DI * DJ > 64 * 64)>(r.p0, r.p1, [&](int s, int p) {
+        {
             const int buf = (p - r.p0) & 1;
             const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
             const int row0 = (reversed ? r.nchunks - 1 - p : p) * kChunk;
@@ -507,9 +533,9 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                         }
                     }
             }
-            __syncthreads();
+            chunk_barrier();
         }
-    }
+    });
 }
 
 // One problem per workgroup: OW output wavefronts (IB = 4/OW blocks each), 4 state, LW loader.
@@ -666,11 +692,8 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
 #pragma unroll
         for (int ks = 0; ks < TL::KS; ++ks)
             sf[jt][ks] = *reinterpret_cast<const u32x4 *>(sS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
-    for (int pb = p0;; pb += PF) {
-#pragma unroll
-        for (int s = 0; s < PF; ++s) {
-            const int p = pb + s;
-            if (p >= p1) return;
+    run_rounds<PF>(p0, p1, [&](int s, int p) {
+        {
             u32x4 qc[TL::KS];
 #pragma unroll
             for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
@@ -685,8 +708,9 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
                 const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
                 buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
             }
+            __builtin_amdgcn_sched_barrier(0);  // keep the next chunk's waits out of this one
         }
-    }
+    });
 }
 
 // Non-causal form for a head that one workgroup handles alone (no sequence groups): pass 1 sums
@@ -734,24 +758,15 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
         store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
         load_chunk(0, PF);
         __syncthreads();
-        bool more = true;
-        for (int pb = 0; more; pb += PF) {
-#pragma unroll
-            for (int s = 0; s < PF; ++s) {
-                const int p = pb + s;
-                if (p >= nchunks) {
-                    more = false;
-                } else {
-                    const int s1 = (s + 1) % PF;
-                    const int buf = p & 1;
-                    store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-                    store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
-                    load_chunk(s1, p + 1 + PF);
-                    state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
-                    __syncthreads();
-                }
-            }
-        }
+        run_rounds<PF>(0, nchunks, [&](int s, int p) {
+            const int s1 = (s + 1) % PF;
+            const int buf = p & 1;
+            store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
+            store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+            load_chunk(s1, p + 1 + PF);
+            state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+            chunk_barrier();
+        });
     }
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_q(s, s);  // in flight while the state is converted
@@ -773,11 +788,8 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
             sf[jt][ks] = *reinterpret_cast<const u32x4 *>(sS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
 
     // ---- pass 2: out_c = A_c S
-    for (int pb = 0;; pb += PF) {
-#pragma unroll
-        for (int s = 0; s < PF; ++s) {
-            const int p = pb + s;
-            if (p >= nchunks) return;
+    run_rounds<PF>(0, nchunks, [&](int s, int p) {
+        {
             u32x4 qc[TL::KS];
 #pragma unroll
             for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
@@ -792,8 +804,9 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
                 const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
                 buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
             }
+            __builtin_amdgcn_sched_barrier(0);  // keep the next chunk's waits out of this one
         }
-    }
+    });
 }
 
 }  // namespace cott
