@@ -27,12 +27,15 @@ def _dtype_code(t):
 
 
 def _require_gpu(**tensors):
+    dev = None
     for name, t in tensors.items():
         if not t.is_cuda:
             raise RuntimeError(f"{name} must be a CUDA tensor")  # wording of combined_kernel_general.cu:355-357
-    devs = {t.device for t in tensors.values()}
-    if len(devs) != 1:
-        raise RuntimeError(f"all tensors must be on the same device, got {sorted(map(str, devs))}")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            devs = sorted({str(x.device) for x in tensors.values()})
+            raise RuntimeError(f"all tensors must be on the same device, got {devs}")
 
 
 def _shapes(q, k, v):
@@ -53,8 +56,43 @@ def _workspace(nbytes, device):
     return ws, ws.data_ptr()
 
 
-def _stream():
-    return torch.cuda.current_stream().cuda_stream
+# The host side of a call costs about as much as the kernels of a small problem run, so the fixed parts are kept
+# short: workspace sizes are remembered per shape, the device is only switched when it is not the current one, and
+# the stream handle comes from torch's raw accessor.
+_ws_bytes_cache = {}
+
+
+def _ws_bytes(query, *key):
+    k = (query, key)
+    n = _ws_bytes_cache.get(k)
+    if n is None:
+        n = _ws_bytes_cache[k] = getattr(_loader.lib(), query)(*key)
+    return n
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on(device):
+    """Context that makes `device` current for the launch (a no-op when it already is)."""
+    return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream(device=None):
+    if _raw_stream is not None and device is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def causal_dot_product(q, k, v, reversed=False):
@@ -67,10 +105,10 @@ def causal_dot_product(q, k, v, reversed=False):
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
     L = _loader.lib()
-    with torch.cuda.device(q.device):
-        ws, ws_ptr = _workspace(L.cott_causal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+    with _on(q.device):
+        ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
         rc = L.cott_causal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,
-                               int(bool(reversed)), ws_ptr, ws.numel() if ws is not None else 0, _stream())
+                               int(bool(reversed)), ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
     _check(rc, "cott_causal_fwd")
     return o
 
@@ -95,12 +133,12 @@ def causal_prefill(q, k, v, state=None, return_state=True):
     o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
     s_out = torch.empty((b, h, dk, dv), dtype=sdt, device=q.device) if return_state else None
     L = _loader.lib()
-    with torch.cuda.device(q.device):
-        ws, ws_ptr = _workspace(L.cott_causal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+    with _on(q.device):
+        ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
         rc = L.cott_causal_fwd_state(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                      state.data_ptr() if state is not None else None,
                                      s_out.data_ptr() if s_out is not None else None, b, h, n, dk, dv, code, ws_ptr,
-                                     ws.numel() if ws is not None else 0, _stream())
+                                     ws.numel() if ws is not None else 0, _stream(q.device))
     _check(rc, "cott_causal_fwd_state")
     return o, s_out
 
@@ -117,11 +155,11 @@ def causal_backward(q, k, v, grad_out):
     q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), grad_out.contiguous()
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     L = _loader.lib()
-    with torch.cuda.device(q.device):
-        ws, ws_ptr = _workspace(L.cott_causal_bwd_workspace_bytes(b, h, n, dk, dv, code), q.device)
+    with _on(q.device):
+        ws, ws_ptr = _workspace(_ws_bytes("cott_causal_bwd_workspace_bytes", b, h, n, dk, dv, code), q.device)
         rc = L.cott_causal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(), dk_.data_ptr(),
                                dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0,
-                               _stream())
+                               _stream(q.device))
     _check(rc, "cott_causal_bwd")
     return dq, dk_, dv_
 
@@ -136,10 +174,10 @@ def noncausal_dot_product(q, k, v):
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
     L = _loader.lib()
-    with torch.cuda.device(q.device):
-        ws, ws_ptr = _workspace(L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+    with _on(q.device):
+        ws, ws_ptr = _workspace(_ws_bytes("cott_noncausal_workspace_bytes", b, h, n, dk, dv, code), q.device)
         rc = L.cott_noncausal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,
-                                  ws_ptr, ws.numel() if ws is not None else 0, _stream())
+                                  ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
     _check(rc, "cott_noncausal_fwd")
     return o
 
@@ -156,11 +194,11 @@ def noncausal_backward(q, k, v, grad_out):
     q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), grad_out.contiguous()
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     L = _loader.lib()
-    with torch.cuda.device(q.device):
-        ws, ws_ptr = _workspace(L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, code), q.device)
+    with _on(q.device):
+        ws, ws_ptr = _workspace(_ws_bytes("cott_noncausal_workspace_bytes", b, h, n, dk, dv, code), q.device)
         rc = L.cott_noncausal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(),
                                   dk_.data_ptr(), dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr,
-                                  ws.numel() if ws is not None else 0, _stream())
+                                  ws.numel() if ws is not None else 0, _stream(q.device))
     _check(rc, "cott_noncausal_bwd")
     return dq, dk_, dv_
 
@@ -187,9 +225,9 @@ def decode_step(state, q, k, v, out=None):
     elif out.shape != (b, h, dv) or out.dtype != q.dtype or not out.is_contiguous() or out.device != q.device:
         raise RuntimeError("decode_step: bad `out` tensor")
     L = _loader.lib()
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = L.cott_decode_step(state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b, h, dk,
-                                dv, code, _stream())
+                                dv, code, _stream(q.device))
     _check(rc, "cott_decode_step")
     return out
 
@@ -265,10 +303,10 @@ def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None, rotar
     qo, ko = (torch.empty((b, h, n, dk), dtype=out_dtype, device=q.device) for _ in range(2))
     vo = torch.empty((b, h, n, dv), dtype=out_dtype, device=q.device)
     L = _loader.lib()
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = L.cott_prep_ex_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), qo.data_ptr(), ko.data_ptr(), vo.data_ptr(),
                                 _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), _ptr(pos), rdim, rows, int(bool(bnhd)),
-                                b, h, n, dk, dv, code, _DTYPES[out_dtype], _stream())
+                                b, h, n, dk, dv, code, _DTYPES[out_dtype], _stream(q.device))
     _check(rc, "cott_prep_ex_fwd")
     return qo, ko, vo
 
@@ -290,11 +328,11 @@ def prepare_inputs_backward(q, k, v, gq, gk, gv, keep=None, cnt=None, sig=None, 
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     drows = torch.empty((b, h, n), dtype=torch.float32, device=q.device) if (want_dsig and sig is not None) else None
     L = _loader.lib()
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         rc = L.cott_prep_ex_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
                                 dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), _ptr(drows), _ptr(keep), _ptr(cnt),
                                 _ptr(sig), _ptr(table), _ptr(pos), rdim, rows, int(bool(bnhd)), b, h, n, dk, dv, code,
-                                gcode, _stream())
+                                gcode, _stream(q.device))
     _check(rc, "cott_prep_ex_bwd")
     dsig = drows.sum(dim=(0, 2)) if drows is not None else None
     return dq, dk_, dv_, dsig
