@@ -516,12 +516,26 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 #pragma unroll
                     for (int jj = 0; jj < JB; ++jj) {
                         const int jt = j0 + jj;
+                        // With four contraction steps (DI = 128) a tile's 2 + 4 products run as three chains of two: a
+                        // dependent MFMA waits for the whole latency of the one before and such a batch has only
+                        // IB tiles to interleave (5 % faster there; at DI <= 64 the extra accumulators only cost
+                        // registers, spilling in the pair kernel).
                         f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int kb = 0; kb < 2; ++kb)
                             o = TR::mfma(vf[slot][jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
+                        if constexpr (TL::KS >= 4) {
+                            f32x4 o2 = {0.f, 0.f, 0.f, 0.f}, o3 = o2;
 #pragma unroll
-                        for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[slot][jj][ks], qc[ib][ks], o);
+                            for (int ks = 0; ks < TL::KS; ks += 2) {
+                                o2 = TR::mfma(sf[slot][jj][ks], qc[ib][ks], o2);
+                                o3 = TR::mfma(sf[slot][jj][ks + 1], qc[ib][ks + 1], o3);
+                            }
+                            o += o2 + o3;
+                        } else {
+#pragma unroll
+                            for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[slot][jj][ks], qc[ib][ks], o);
+                        }
                         const int col = 16 * jt + 4 * g;
                         const u32x2 val = {TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
                         if (sOt != nullptr) {
