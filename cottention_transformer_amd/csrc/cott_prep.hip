@@ -124,6 +124,14 @@ __device__ __forceinline__ void rotate4(Vec4<ACC> &v, f32x2 sn, f32x2 cs, bool i
     }
 }
 
+// Per-row scalars in fp32 use the hardware reciprocal and square root (1 ulp, no denormal fix-up sequences: the
+// operands are clamped away from the denormal range); every lane of a row repeats them, and for head-sized
+// rows the kernel is bound by instruction issue.
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ double fast_rcp(double x) { return 1.0 / x; }
+__device__ __forceinline__ float fast_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+__device__ __forceinline__ double fast_sqrt(double x) { return sqrt(x); }
+
 // (hardware exp2 / log2: about 1e-6 relative, far inside the fp32 tolerance of the op)
 __device__ __forceinline__ float pow_pos(float c, float s) { return c > 0.f ? __expf(s * __logf(c)) : 0.f; }
 __device__ __forceinline__ double pow_pos(double c, double s) { return c > 0.0 ? exp(s * log(c)) : 0.0; }
@@ -245,15 +253,16 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
         ACC mul_x = 0, mul_g = 0;  // y = mul_x * x (forward);  dx = mul_g * g + mul_x * x (backward)
         if (t < 2) {
             ss = row_sum(ss, lpr);
-            const ACC nrm = sqrt(ss);
+            const ACC nrm = fast_sqrt(ss);
             const ACC den = nrm > (ACC)a.eps ? nrm : (ACC)a.eps;
+            const ACC rden = fast_rcp(den);
             if (!BACKWARD) {
-                mul_x = keep / den;
+                mul_x = keep * rden;
             } else {
                 dot = row_sum(dot, lpr);
-                mul_g = keep / den;
+                mul_g = keep * rden;
                 // d/dx of x / max(|x|, eps): the norm term only exists where the norm is not clamped
-                mul_x = nrm > (ACC)a.eps ? -keep * dot / (nrm * nrm * nrm) : (ACC)0;
+                mul_x = nrm > (ACC)a.eps ? -keep * dot * (rden * rden * rden) : (ACC)0;
             }
         } else {
             ACC scale = 1;
@@ -263,7 +272,7 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
                 c = (ACC)cnt_in[u];
                 const ACC p = pow_pos(c, (ACC)sig_in[u]);
                 if (p > (ACC)1) {
-                    scale = (ACC)1 / p;
+                    scale = fast_rcp(p);
                     scaled = true;
                 }
             }
