@@ -5,15 +5,16 @@ include/cottention.h; this package is the torch-facing host side.  `Cuda_Kernel/
 named like the reference's extension (`FastAttention2.kernel`, `FastAttention.forward/backward`,
 `Custom_Kernel.CustomAttention`) so its callers import them unchanged.
 """
-from .ops import (causal_backward, causal_dot_product, causal_prefill, decode_step, noncausal_backward,  # noqa: F401
-                  noncausal_dot_product, prepare_inputs, prepare_inputs_backward)
+from .ops import (causal_backward, causal_dot_product, causal_prefill, decode_step, merged_heads_supported,  # noqa: F401
+                  noncausal_backward, noncausal_dot_product, prepare_inputs, prepare_inputs_backward)
 
-__all__ = ["causal_dot_product", "causal_prefill", "causal_backward", "noncausal_dot_product", "noncausal_backward", "decode_step",
-           "prepare_inputs", "prepare_inputs_backward", "CustomAttention", "NonCausalAttention", "PrepareInputs"]
+__all__ = ["causal_dot_product", "causal_prefill", "causal_backward", "merged_heads_supported", "noncausal_dot_product",
+           "noncausal_backward", "decode_step",
+           "prepare_inputs", "prepare_inputs_backward", "CustomAttention", "CustomAttentionMergedHeads", "NonCausalAttention", "PrepareInputs"]
 
 
 def __getattr__(name):
-    if name in ("CustomAttention", "NonCausalAttention", "PrepareInputs"):
+    if name in ("CustomAttention", "CustomAttentionMergedHeads", "NonCausalAttention", "PrepareInputs"):
         from . import autograd
         return getattr(autograd, name)
     raise AttributeError(name)

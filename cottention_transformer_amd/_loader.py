@@ -25,6 +25,8 @@ SIGNATURES = {
     "cott_prep_ex_bwd": (_i, [_vp] * 15 + [_i] * 10 + [_vp]),
     "cott_causal_bwd_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_causal_fwd_bnhd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_causal_bwd_bnhd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_workspace_bytes": (_sz, [_i] * 6),
     "cott_noncausal_fwd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),

@@ -43,6 +43,27 @@ class CustomAttention(torch.autograd.Function):
         return ops.causal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g)
 
 
+class CustomAttentionMergedHeads(torch.autograd.Function):
+    """CustomAttention with the head merge folded in: apply(Q, K, V) -> O of shape (N, S, H, Dv), i.e. the rows
+    of the (N, S, H*Dv) input of the output projection (GPT_Trainer/GPTCosAttention.py:479,500), and a backward
+    that reads the gradient in that layout.  Only where ops.merged_heads_supported() holds for the dtype the
+    forward computes in; callers fall back to CustomAttention + permute otherwise."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V):
+        if Q.dtype not in _SUPPORTED:
+            raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
+        dt = _autocast_target(Q, half_entry=(Q.dtype == torch.float16))
+        Q, K, V = Q.contiguous().to(dt), K.contiguous().to(dt), V.contiguous().to(dt)
+        ctx.save_for_backward(Q, K, V)  # in the computed (16-bit) type: the backward reads the merged layout too
+        return ops.causal_dot_product(Q, K, V, False, merged_heads=True)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        Q, K, V = ctx.saved_tensors
+        return ops.causal_backward(Q, K, V, grad_output.contiguous().to(Q.dtype), merged_heads=True)
+
+
 class NonCausalAttention(torch.autograd.Function):
     """O = Q (K^T V): the BERT form (BERT_Trainer/BertCosAttention.py:249) as one fused operator."""
 

@@ -100,6 +100,8 @@ struct Op {
     int di, dj, reversed;
     const void *sin = nullptr;  // (BH,di,dj) state to start from / to receive the final state (causal only)
     void *sout = nullptr;
+    unsigned char lay[4] = {0, 0, 0, 0};  // A, B, C, O given as (B,N,H,width) instead of (BH,N,width)
+    int H = 1;
 };
 
 // How a set of `nops` ops with the same padded head dims is laid on the chip.
@@ -230,6 +232,10 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
     bool mfma = true;
     for (int i = 0; i < n; ++i) mfma = mfma && use_mfma(dtype, ops[i].di, ops[i].dj, N);
     const size_t esz = elem_size(dtype);
+    bool interleaved = false;
+    for (int i = 0; i < n; ++i) interleaved = interleaved || ops[i].lay[0] || ops[i].lay[1] || ops[i].lay[2] || ops[i].lay[3];
+    if (interleaved && !(mfma && causal && (dtype == COTT_BF16 || dtype == COTT_F16)))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: (B,N,H,D) operands need bf16 / fp16 and head dims 32..128 in steps of 16", fn);
     if (!mfma) {
         for (int i = 0; i < n; ++i) {
             if (!cott::generic_fits(dtype, ops[i].di))
@@ -276,6 +282,8 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
                 d.sin = o.sin ? static_cast<const char *>(o.sin) + (size_t)h * djh * ssz : nullptr;
                 d.sout = o.sout ? static_cast<char *>(o.sout) + (size_t)h * djh * ssz : nullptr;
                 d.lds = o.dj;
+                for (int x = 0; x < 4; ++x) d.lay[x] = o.lay[x];
+                d.H = o.H;
             }
         }
         a.ws = p.ws_bytes ? reinterpret_cast<float *>(ws_cursor) : nullptr;
@@ -419,6 +427,56 @@ int cott_causal_bwd(const void *q, const void *k, const void *v, const void *d_o
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
     Op ops[3];
     grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
+    return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+// (B,N,H,D) operands are addressed with 32-bit byte offsets inside one batch element
+int check_interleaved(const char *fn, int H, int N, int Dk, int Dv, int dtype) {
+    if (dtype != COTT_BF16 && dtype != COTT_F16)
+        return fail(COTT_ERR_UNSUPPORTED, "%s: (B,N,H,D) operands need bf16 / fp16 tensors", fn);
+    if (!use_mfma(dtype, Dk, Dv, N) || !use_mfma(dtype, Dv, Dk, N))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: (B,N,H,D) operands need head dims 32..128 in steps of 16", fn);
+    const long dmax = Dk > Dv ? Dk : Dv;
+    if ((long)N * H * dmax > (1L << 30))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: N*H*D = %ld exceeds 2^30", fn, (long)N * H * dmax);
+    return COTT_OK;
+}
+}  // namespace
+
+int cott_causal_fwd_bnhd(const void *q, const void *k, const void *v, void *o, int B, int H, int N, int Dk, int Dv,
+                         int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+    const char *fn = "cott_causal_fwd_bnhd";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (int rc = check_interleaved(fn, H, N, Dk, Dv, dtype)) return rc;
+    if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op op{q, k, v, o, Dk, Dv, 0};
+    op.lay[3] = 1;
+    op.H = H;
+    return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int cott_causal_bwd_bnhd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
+                         int B, int H, int N, int Dk, int Dv, int dtype, void *workspace, size_t workspace_bytes,
+                         void *stream) {
+    const char *fn = "cott_causal_bwd_bnhd";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if (int rc = check_common(fn, B, H, N, Dv, Dk, dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (int rc = check_interleaved(fn, H, N, Dk, Dv, dtype)) return rc;
+    if (!q || !k || !v || !d_o || !dq || !dk || !dv) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
+        !aligned16(dv))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op ops[3];
+    grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
+    ops[0].lay[0] = 1;  // dq = G(d_o, v, k):      d_o is A
+    ops[1].lay[1] = 1;  // dk = G(v, d_o, q, rev): d_o is B
+    ops[2].lay[2] = 1;  // dv = G(k, q, d_o, rev): d_o is C
+    for (int i = 0; i < 3; ++i) ops[i].H = H;
     return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 

@@ -16,6 +16,10 @@ struct OpDesc {
     const void *sin = nullptr;  // start from this state instead of zero
     void *sout = nullptr;       // receives the state after the last position
     int lds = 0;
+    // Layout of A, B, C, O (16-bit causal MFMA kernels only): 0 = (BH,N,width), 1 = (B,N,H,width) with the heads
+    // of a position next to each other, as the projections of a transformer block produce and consume them.
+    unsigned char lay[4] = {0, 0, 0, 0};
+    int H = 1;  // heads per batch element; needed when any layout flag is set
 };
 
 // A set of ops launched together over the same (BH, N); MFMA path: all share padded head dims.

@@ -36,6 +36,12 @@ struct ProblemT {
     const float *sin;
     float *sout;
     int di, dj, ldc, reversed, lds;
+    // Causal kernels only.  Row strides of A, B and O in elements (C's is ldc) and, for each operand, where a head
+    // starts: head bh is at (bh / H) * bs + (bh % H) * hs elements.  (BH,N,w) tensors have ld = w, hs = N * w,
+    // bs = H * hs; (B,N,H,w) tensors, whose heads are interleaved inside a position, ld = H * w, hs = w,
+    // bs = N * H * w.
+    int lda, ldb, ldo, H;
+    long hsA, bsA, hsB, bsB, hsC, bsC, hsO, bsO;
     // scan_pair_kernel only: a second problem G(A2, C, B) -> O2 served by the same workgroup (null = none)
     const E *A2;
     E *O2;
@@ -48,6 +54,10 @@ struct ProblemSetT {
 };
 typedef ProblemT<u16> Problem;  // 16-bit storage (bf16 / fp16)
 typedef ProblemSetT<u16> ProblemSet;
+
+__device__ __forceinline__ size_t head_base(long bs, long hs, int H, int bh) {
+    return (size_t)(bh / H) * (size_t)bs + (size_t)(bh % H) * (size_t)hs;
+}
 
 template <int DI, int DJ>
 struct Tiling {
@@ -204,9 +214,9 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     const WorkItem wi = decode_workgroup(set.count, ngroups);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
-    const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
-    const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-    const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const int di = pr.di, dj = pr.dj, ldb = pr.ldb, ldc = pr.ldc, reversed = pr.reversed;
+    const rsrc_t rB = make_rsrc(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), ((uint32_t)(N - 1) * ldb + di) * 2u);
+    const rsrc_t rC = make_rsrc(pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), ((uint32_t)(N - 1) * ldc + dj) * 2u);
     const int p0 = wi.grp * cpg;
     const int p1 = min(p0 + cpg, nchunks);
 
@@ -218,7 +228,7 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     auto load_chunk = [&](int s, int p) {
         const int pc = min(p, p1 - 1);
         const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
-        load_tile<DI>(rb[s], rB, row0, di, tid);
+        load_tile<DI>(rb[s], rB, row0, ldb, tid);
         load_tile<DJ>(rc[s], rC, row0, ldc, tid);
     };
     auto finish = [&]() {
@@ -298,12 +308,12 @@ struct StagedOut {
 };
 
 template <int DI, int DJ, int PF, int LT>
-__device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head, int di, int dj, int ldc,
+__device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head, int di, int dj, int ldb, int ldc,
                                             const ScanRange &r, int tid, u16 *sB, u16 *sC,
                                             const StagedOut *so = nullptr) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SO = kChunk * TL::OS;
-    const rsrc_t rB = make_rsrc(B_head, (uint32_t)r.N * di * 2u);
+    const rsrc_t rB = make_rsrc(B_head, ((uint32_t)(r.N - 1) * ldb + di) * 2u);
     const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     // the staged tile(s) of chunk p (scan order): 16-byte row segments, rows past N dropped by the range check
     auto write_out = [&](int p) {
@@ -327,7 +337,7 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
     auto load_chunk = [&](int s, int p) {
         const int pc = min(p, r.p1 - 1);
         const int row0 = (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
-        load_tile<DI, LT>(rb[s], rB, row0, di, tid);
+        load_tile<DI, LT>(rb[s], rB, row0, ldb, tid);
         load_tile<DJ, LT>(rc[s], rC, row0, ldc, tid);
     };
 #pragma unroll
@@ -415,19 +425,20 @@ __device__ __forceinline__ void state_role(const float *seed, const float *sin, 
 }
 
 // Output role: one wavefront, IB blocks of 16 positions starting at block `blk0` of each chunk.
+// lda, ldc: row strides of A and of O.
 // cB: tile read by rows (the B operand of this problem), cC: tile read by columns (its C operand),
 // cS: its 16-bit state; all three double-buffered with the strides of Tiling<DI, DJ>.
 // sOt: null = store the outputs to memory from here; else the [2 buffers] of this problem's staged output tile
 // (buffer stride 2 * 64 * OS), written with 8-byte LDS stores and sent to memory by the loader wavefronts, so that
 // this wavefront's chain of LDS reads and MFMAs never waits for the vector-memory pipeline to take a store.
 template <class TR, int DI, int DJ, int PF, int IB>
-__device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int ldc, const ScanRange &r,
-                                            int blk0, int l, const u16 *sB, const u16 *sC, const u16 *sS,
-                                            u16 *sOt = nullptr) {
+__device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int lda, int ldc,
+                                            const ScanRange &r, int blk0, int l, const u16 *sB, const u16 *sC,
+                                            const u16 *sS, u16 *sOt = nullptr) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
-    const rsrc_t rA = make_rsrc(A_head, (uint32_t)r.N * di * 2u);
+    const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
     const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     const int reversed = r.reversed;
     u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
@@ -438,7 +449,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
         for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
             for (int ks = 0; ks < TL::KS; ++ks)
-                qn[s][ib][ks] = buf_load16(rA, (uint32_t)((row + 16 * ib) * di + 32 * ks + 8 * g) * 2u);
+                qn[s][ib][ks] = buf_load16(rA, (uint32_t)((row + 16 * ib) * lda + 32 * ks + 8 * g) * 2u);
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_q(s, r.p0 + s);
@@ -579,16 +590,17 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     r.p1 = min(r.p0 + cpg, nchunks);
     r.reversed = pr.reversed;
     if (wv >= OW + 4) {
-        loader_role<DI, DJ, PF, LT>(pr.B + (size_t)wi.bh * N * di, pr.C + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
-                                    (int)threadIdx.x - 64 * (OW + 4), sB, sC);
+        loader_role<DI, DJ, PF, LT>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
+                                    di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC);
     } else if (wv >= OW) {
         state_role<TR, DI, DJ, false>(
             pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr,
             pr.sin ? pr.sin + (size_t)wi.bh * di * pr.lds : nullptr, pr.sout ? pr.sout + (size_t)wi.bh * di * pr.lds : nullptr,
             pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS, nullptr);
     } else {
-        output_role<TR, DI, DJ, PF, IB>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
-                                        IB * wv, l, sB, sC, sS);
+        output_role<TR, DI, DJ, PF, IB>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
+                                        pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r, IB * wv, l,
+                                        sB, sC, sS);
     }
 }
 
@@ -633,15 +645,15 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     const float *seed = pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr;
     if (wv >= NOUT + 4) {
         StagedOut so;
-        so.O[0] = pr.O + (size_t)wi.bh * N * ldc;
+        so.O[0] = pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh);
         so.dj[0] = dj;
-        so.ld[0] = ldc;
+        so.ld[0] = pr.ldo;
         so.O[1] = pair ? pr.O2 + (size_t)wi.bh * N * di : nullptr;
         so.dj[1] = di;
         so.ld[1] = di;
         so.sO = sO;
-        loader_role<D, D, PF, LT>(pr.B + (size_t)wi.bh * N * di, pr.C + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
-                                  (int)threadIdx.x - 64 * (NOUT + 4), sB, sC, &so);
+        loader_role<D, D, PF, LT>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
+                                  di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (NOUT + 4), sB, sC, &so);
     } else if (wv >= NOUT) {
         if (pair)
             state_role<TR, D, D, true>(seed, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, sS2);
@@ -649,18 +661,19 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
             state_role<TR, D, D, false>(seed, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, nullptr);
     } else if (!pair) {
         if (wv < 4) {
-            output_role<TR, D, D, PF, 1>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
+            output_role<TR, D, D, PF, 1>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r,
                                          wv, l, sB, sC, sS, sO);
         } else {
             for (int p = r.p0 - 1; p < r.p1; ++p) __syncthreads();  // idle: keep the barrier count
         }
     } else if (wv < OWP) {
-        output_role<TR, D, D, PF, IBP>(pr.A + (size_t)wi.bh * N * di, pr.O + (size_t)wi.bh * N * ldc, di, dj, ldc, r,
+        output_role<TR, D, D, PF, IBP>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r,
                                        IBP * wv, l, sB, sC, sS, sO);
     } else {
         // Y: contracted dim dj of X, output dim di of X; its row-read tile is X's C tile and vice versa
-        output_role<TR, D, D, PF, IBP>(pr.A2 + (size_t)wi.bh * N * dj, pr.O2 + (size_t)wi.bh * N * di, dj, di, di, r,
-                                       IBP * (wv - OWP), l, sC, sB, sS2, sO + SO);
+        // the second problem's own operands (A2, O2) are plain (BH,N,w) tensors
+        output_role<TR, D, D, PF, IBP>(pr.A2 + (size_t)wi.bh * N * dj, nullptr, dj, di, dj, di, r, IBP * (wv - OWP), l, sC,
+                                       sB, sS2, sO + SO);
     }
 }
 

@@ -15,7 +15,8 @@ import torch
 from torch import nn
 
 from . import ops
-from .autograd import CustomAttention, NonCausalAttention, PrepareInputs, _autocast_target
+from .autograd import (CustomAttention, CustomAttentionMergedHeads, NonCausalAttention, PrepareInputs,
+                       _autocast_target)
 
 
 def _autocast_on():
@@ -104,10 +105,13 @@ class GPTCosAttention(nn.Module):
             key, query = apply_rotary(key, sin, cos), apply_rotary(query, sin, cos)
         return query, key
 
-    def _cos_attn(self, query, key, value, attention_mask=None, head_mask=None, rotary=None, bnhd=False):
+    def _cos_attn(self, query, key, value, attention_mask=None, head_mask=None, rotary=None, bnhd=False,
+                  merge_heads=False):
         """GPTCosAttention.py:200-282.  query, key, value: (B,H,S,D), already rotated -- or, with `bnhd`, (B,S,H,D)
         as the projections produce them, with rotary=(table, position_ids) still to be applied; in that case the
-        rotation, the head permute and the preparation steps are one fused pass."""
+        rotation, the head permute and the preparation steps are one fused pass.
+        merge_heads: the caller wants the output as (B,S,H,D) (:500); returned that way, with None in place of
+        the second value, when the training path can write it directly, else (B,H,S,D) as usual."""
         if bnhd:
             b, s, h, _ = query.shape
         else:
@@ -134,6 +138,8 @@ class GPTCosAttention(nn.Module):
         cnt = keep.to(torch.float32).cumsum(-1)                        # kept keys at positions <= s (:228)
         dt = _autocast_target(query)
         q, k, v = PrepareInputs.apply(query, key, value, keep, cnt, sig, dt, table, pos, bnhd)
+        if merge_heads and ops.merged_heads_supported(q.dtype, s, h, q.shape[-1], v.shape[-1]):
+            return CustomAttentionMergedHeads.apply(q, k, v), None
         out = CustomAttention.apply(q, k, v)
         return out, out
 
@@ -153,7 +159,8 @@ class GPTCosAttention(nn.Module):
                 table = self.embed_positions = table.to(hidden_states.device)
             present = None
             attn_output, attn_weights = self._cos_attn(query, key, value, attention_mask, head_mask,
-                                                       rotary=(table, position_ids), bnhd=True)
+                                                       rotary=(table, position_ids), bnhd=True,
+                                                       merge_heads=not output_attentions)
         else:
             query, key = self._rotate(query, key, position_ids)
             key, query, value = key.permute(0, 2, 1, 3), query.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3)
@@ -164,7 +171,8 @@ class GPTCosAttention(nn.Module):
             attn_output, attn_weights = self._cos_attn(query, key, value, attention_mask, head_mask)
         if not _autocast_on():
             attn_output = attn_output.to(hidden_states.dtype)
-        attn_output = attn_output.permute(0, 2, 1, 3).contiguous()
+        if attn_weights is not None:  # came back (B,H,S,D): merge the heads here (:500)
+            attn_output = attn_output.permute(0, 2, 1, 3).contiguous()
         attn_output = attn_output.view(attn_output.size()[:-2] + (self.embed_dim,))
         attn_output = self.resid_dropout(self.out_proj(attn_output))
         outputs = (attn_output, present)

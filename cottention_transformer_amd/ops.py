@@ -95,16 +95,36 @@ def _stream(device=None):
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def causal_dot_product(q, k, v, reversed=False):
-    """o[s,j] = sum_i q[s,i] sum_{s'<=s (>=s if reversed)} k[s',i] v[s',j]; all of one dtype."""
+def merged_heads_supported(dtype, n, h, dk, dv):
+    """Whether the causal ops can write o / read grad_out as (B,N,H,Dv) (see causal_dot_product)."""
+    ok = lambda d: 32 <= d <= 128 and d % 16 == 0
+    return dtype in (torch.bfloat16, torch.float16) and ok(dk) and ok(dv) and n * h * max(dk, dv) <= 1 << 30
+
+
+def causal_dot_product(q, k, v, reversed=False, merged_heads=False):
+    """o[s,j] = sum_i q[s,i] sum_{s'<=s (>=s if reversed)} k[s',i] v[s',j]; all of one dtype.
+
+    merged_heads: return o as (B,N,H,Dv), the rows of the (B,N,H*Dv) tensor an output projection reads, instead
+    of (B,H,N,Dv): the head merge of GPT_Trainer/GPTCosAttention.py:500 without its copy (bf16 / fp16 only, see
+    merged_heads_supported)."""
     _require_gpu(Q=q, K=k, V=v)
     b, h, n, dk, dv = _shapes(q, k, v)
     if not (q.dtype == k.dtype == v.dtype):
         raise RuntimeError("Q, K and V must have the same dtype")
     code = _dtype_code(q)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
     L = _loader.lib()
+    if merged_heads:
+        if reversed:
+            raise RuntimeError("merged_heads is only available for the forward direction")
+        o = torch.empty((b, n, h, dv), dtype=q.dtype, device=q.device)
+        with _on(q.device):
+            ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
+            rc = L.cott_causal_fwd_bnhd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,
+                                        ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
+        _check(rc, "cott_causal_fwd_bnhd")
+        return o
+    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
     with _on(q.device):
         ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
         rc = L.cott_causal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,
@@ -143,12 +163,13 @@ def causal_prefill(q, k, v, state=None, return_state=True):
     return o, s_out
 
 
-def causal_backward(q, k, v, grad_out):
-    """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out."""
+def causal_backward(q, k, v, grad_out, merged_heads=False):
+    """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out ((B,N,H,Dv) with merged_heads)."""
     _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)
     b, h, n, dk, dv = _shapes(q, k, v)
-    if grad_out.shape != v.shape:
-        raise RuntimeError(f"prev_grad must have V's shape {tuple(v.shape)}, got {tuple(grad_out.shape)}")
+    want = (b, n, h, dv) if merged_heads else tuple(v.shape)
+    if tuple(grad_out.shape) != want:
+        raise RuntimeError(f"prev_grad must have shape {want}, got {tuple(grad_out.shape)}")
     if not (q.dtype == k.dtype == v.dtype == grad_out.dtype):
         raise RuntimeError("Q, K, V and prev_grad must have the same dtype")
     code = _dtype_code(q)
@@ -157,10 +178,10 @@ def causal_backward(q, k, v, grad_out):
     L = _loader.lib()
     with _on(q.device):
         ws, ws_ptr = _workspace(_ws_bytes("cott_causal_bwd_workspace_bytes", b, h, n, dk, dv, code), q.device)
-        rc = L.cott_causal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(), dk_.data_ptr(),
-                               dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0,
-                               _stream(q.device))
-    _check(rc, "cott_causal_bwd")
+        fn = L.cott_causal_bwd_bnhd if merged_heads else L.cott_causal_bwd
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), b, h,
+                n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
+    _check(rc, "cott_causal_bwd_bnhd" if merged_heads else "cott_causal_bwd")
     return dq, dk_, dv_
 
 

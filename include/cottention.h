@@ -83,6 +83,22 @@ COTT_API int cott_causal_bwd(const void *q, const void *k, const void *v, const 
                     int B, int H, int N, int Dk, int Dv, int dtype,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- causal forward / backward with the head merge folded in --------------------------------
+ * The same two operations with the attention output o (forward) and its gradient d_o (backward) laid out
+ * (B,N,H,Dv), i.e. as the rows of the (B,N,H*Dv) tensor that the output projection reads and
+ * differentiates.  Replaces the permute + contiguous copy of the head merge around the op
+ * (GPT_Trainer/GPTCosAttention.py:500 `_merge_heads`, called at :479, and its backward).  q, k, v and
+ * dq, dk, dv stay (B,H,N,D) (cott_prep_ex_* already reads and writes the projection layout on that side).
+ * bf16 / fp16, head dims 32..128 in steps of 16, N*H*D <= 2^30; other cases return COTT_ERR_UNSUPPORTED
+ * and the caller permutes.  Workspace: cott_causal_workspace_bytes / cott_causal_bwd_workspace_bytes. */
+COTT_API int cott_causal_fwd_bnhd(const void *q, const void *k, const void *v, void *o,
+                         int B, int H, int N, int Dk, int Dv, int dtype,
+                         void *workspace, size_t workspace_bytes, void *stream);
+COTT_API int cott_causal_bwd_bnhd(const void *q, const void *k, const void *v, const void *d_o,
+                         void *dq, void *dk, void *dv,
+                         int B, int H, int N, int Dk, int Dv, int dtype,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- non-causal form ------------------------------------------------------------------------
  *   o = q (k^T v)   per (batch, head)
  * Replaces the two einsums of BERT_Trainer/BertCosAttention.py:249 (the (QK^T)V branch at :222

@@ -80,6 +80,48 @@ def test_causal_backward(ct, oracle, case):
         assert rel_l2(got, ref) <= TOL[dt], name
 
 
+MERGED_CASES = [
+    # b, h, n, dk, dv, dtype                   launch form the shape takes
+    (2, 16, 2048, 64, 64, BF),    # forward: two column halves per head; gradients: dQ + (dK, dV) pair workgroups
+    (2, 3, 1000, 64, 32, HF),     # Dk != Dv: three separate gradient problems, ragged tail
+    (1, 4, 8192, 128, 128, BF),   # sequence groups, 128-wide heads
+    (3, 5, 63, 32, 128, BF),      # a single partial chunk
+    (2, 12, 300, 48, 80, HF),     # head dims padded to 64 / 128
+]
+
+
+@pytest.mark.parametrize("case", MERGED_CASES, ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_merged_heads_layout(ct, oracle, case):
+    """o written as (B,N,H,Dv) and d_o read as (B,N,H,Dv) (cott_causal_fwd_bnhd / cott_causal_bwd_bnhd): the same
+    numbers as the (B,H,N,D) entry points, bit for bit, and within tolerance of the oracle."""
+    b, h, n, dk, dv, dt = case
+    say("merged heads", case)
+    q, k, v, do = inputs(b, h, n, dk, dv, dt, seed=n + 7)
+    qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
+    assert ct.merged_heads_supported(dt, n, h, dk, dv)
+    om = ct.causal_dot_product(qd, kd, vd, merged_heads=True)
+    assert om.shape == (b, n, h, dv) and om.is_contiguous()
+    assert torch.equal(om.permute(0, 2, 1, 3), ct.causal_dot_product(qd, kd, vd))
+    assert rel_l2(om.permute(0, 2, 1, 3), oracle.causal(q, k, v, False)) <= TOL[dt]
+    plain = ct.causal_backward(qd, kd, vd, dod)
+    merged = ct.causal_backward(qd, kd, vd, dod.permute(0, 2, 1, 3).contiguous(), merged_heads=True)
+    for name, got, want, ref in zip(("dQ", "dK", "dV"), merged, plain, oracle.causal_bwd(q, k, v, do)):
+        assert torch.equal(got, want), name
+        assert rel_l2(got, ref) <= TOL[dt], name
+
+
+def test_merged_heads_layout_is_refused_where_not_built(ct):
+    q, k, v, _ = inputs(1, 2, 64, 64, 64, F32, seed=3)
+    assert not ct.merged_heads_supported(F32, 64, 2, 64, 64)
+    with pytest.raises(RuntimeError, match="bf16 / fp16"):
+        ct.causal_dot_product(q.to(DEV), k.to(DEV), v.to(DEV), merged_heads=True)
+    q, k, v, _ = inputs(1, 2, 64, 256, 256, BF, seed=3)  # beyond the MFMA head dims
+    with pytest.raises(RuntimeError, match="head dims"):
+        ct.causal_dot_product(q.to(DEV), k.to(DEV), v.to(DEV), merged_heads=True)
+    with pytest.raises(RuntimeError, match="forward direction"):
+        ct.causal_dot_product(q.to(DEV), k.to(DEV), v.to(DEV), True, merged_heads=True)
+
+
 def test_golden_fixtures(ct):
     for name in ("causal_cfg1_1x2x128x64.npz", "causal_odd_1x2x63x32_dv48.npz"):
         say("golden", name)
