@@ -10,11 +10,12 @@ from .ops import (causal_backward, causal_dot_product, causal_prefill, decode_st
 
 __all__ = ["causal_dot_product", "causal_prefill", "causal_backward", "merged_heads_supported", "noncausal_dot_product",
            "noncausal_backward", "decode_step",
-           "prepare_inputs", "prepare_inputs_backward", "CustomAttention", "CustomAttentionMergedHeads", "NonCausalAttention", "PrepareInputs"]
+           "prepare_inputs", "prepare_inputs_backward", "CustomAttention", "CustomAttentionMergedHeads", "NonCausalAttention", "NonCausalAttentionMergedHeads",
+           "PrepareInputs"]
 
 
 def __getattr__(name):
-    if name in ("CustomAttention", "CustomAttentionMergedHeads", "NonCausalAttention", "PrepareInputs"):
+    if name in __all__ and name[0].isupper():
         from . import autograd
         return getattr(autograd, name)
     raise AttributeError(name)

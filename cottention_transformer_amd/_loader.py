@@ -30,6 +30,8 @@ SIGNATURES = {
     "cott_noncausal_workspace_bytes": (_sz, [_i] * 6),
     "cott_noncausal_fwd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_noncausal_fwd_bnhd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_noncausal_bwd_bnhd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_decode_step": (_i, [_vp] * 5 + [_i] * 5 + [_vp]),
     "cott_profile_enable": (_i, [_i]),
     "cott_profile_read": (_i, [_i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_long)]),

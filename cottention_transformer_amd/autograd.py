@@ -83,6 +83,25 @@ class NonCausalAttention(torch.autograd.Function):
         return ops.noncausal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g)
 
 
+class NonCausalAttentionMergedHeads(torch.autograd.Function):
+    """NonCausalAttention returning O as (N, S, H, Dv) and reading its gradient in that layout
+    (BERT_Trainer/BertCosAttention.py:251-252); same conditions as CustomAttentionMergedHeads."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V):
+        if Q.dtype not in _SUPPORTED:
+            raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
+        dt = _autocast_target(Q)
+        Q, K, V = Q.contiguous().to(dt), K.contiguous().to(dt), V.contiguous().to(dt)
+        ctx.save_for_backward(Q, K, V)
+        return ops.noncausal_dot_product(Q, K, V, merged_heads=True)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        Q, K, V = ctx.saved_tensors
+        return ops.noncausal_backward(Q, K, V, grad_output.contiguous().to(Q.dtype), merged_heads=True)
+
+
 class PrepareInputs(torch.autograd.Function):
     """(q, k, v, keep, cnt, sig, out_dtype[, rot_table, position_ids, bnhd]) -> (q_hat, k_hat, v_scaled), (B,H,N,D):
     the normalise / value-scale / mask steps in front of the attention op (GPT_Trainer/GPTCosAttention.py:216-241),

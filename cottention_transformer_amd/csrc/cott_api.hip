@@ -234,7 +234,7 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
     const size_t esz = elem_size(dtype);
     bool interleaved = false;
     for (int i = 0; i < n; ++i) interleaved = interleaved || ops[i].lay[0] || ops[i].lay[1] || ops[i].lay[2] || ops[i].lay[3];
-    if (interleaved && !(mfma && causal && (dtype == COTT_BF16 || dtype == COTT_F16)))
+    if (interleaved && !(mfma && (dtype == COTT_BF16 || dtype == COTT_F16)))
         return fail(COTT_ERR_UNSUPPORTED, "%s: (B,N,H,D) operands need bf16 / fp16 and head dims 32..128 in steps of 16", fn);
     if (!mfma) {
         for (int i = 0; i < n; ++i) {
@@ -478,6 +478,42 @@ int cott_causal_bwd_bnhd(const void *q, const void *k, const void *v, const void
     ops[2].lay[2] = 1;  // dv = G(k, q, d_o, rev): d_o is C
     for (int i = 0; i < 3; ++i) ops[i].H = H;
     return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int cott_noncausal_fwd_bnhd(const void *q, const void *k, const void *v, void *o, int B, int H, int N, int Dk, int Dv,
+                            int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+    const char *fn = "cott_noncausal_fwd_bnhd";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (int rc = check_interleaved(fn, H, N, Dk, Dv, dtype)) return rc;
+    if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op op{q, k, v, o, Dk, Dv, 0};
+    op.lay[3] = 1;
+    op.H = H;
+    return run_ops(fn, false, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int cott_noncausal_bwd_bnhd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
+                            int B, int H, int N, int Dk, int Dv, int dtype, void *workspace, size_t workspace_bytes,
+                            void *stream) {
+    const char *fn = "cott_noncausal_bwd_bnhd";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if (int rc = check_common(fn, B, H, N, Dv, Dk, dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (int rc = check_interleaved(fn, H, N, Dk, Dv, dtype)) return rc;
+    if (!q || !k || !v || !d_o || !dq || !dk || !dv) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
+        !aligned16(dv))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op ops[3];
+    grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, false);
+    ops[0].lay[0] = 1;
+    ops[1].lay[1] = 1;
+    ops[2].lay[2] = 1;
+    for (int i = 0; i < 3; ++i) ops[i].H = H;
+    return run_ops(fn, false, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 size_t cott_noncausal_workspace_bytes(int B, int H, int N, int Dk, int Dv, int dtype) {

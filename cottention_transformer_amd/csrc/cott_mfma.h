@@ -36,7 +36,7 @@ struct ProblemT {
     const float *sin;
     float *sout;
     int di, dj, ldc, reversed, lds;
-    // Causal kernels only.  Row strides of A, B and O in elements (C's is ldc) and, for each operand, where a head
+    // Row strides of A, B and O in elements (C's is ldc) and, for each operand, where a head
     // starts: head bh is at (bh / H) * bs + (bh % H) * hs elements.  (BH,N,w) tensors have ld = w, hs = N * w,
     // bs = H * hs; (B,N,H,w) tensors, whose heads are interleaved inside a position, ld = H * w, hs = w,
     // bs = N * H * w.
@@ -688,9 +688,9 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
     const WorkItem wi = decode_workgroup(set.count, G);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
-    const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
-    const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-    const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const int di = pr.di, dj = pr.dj, lda = pr.lda, ldo = pr.ldo;
+    const rsrc_t rA = make_rsrc(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), ((uint32_t)(N - 1) * lda + di) * 2u);
+    const rsrc_t rO = make_rsrc(pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), ((uint32_t)(N - 1) * ldo + dj) * 2u);
     const int p0 = wi.grp * cpg;
     const int p1 = min(p0 + cpg, nchunks);
     {
@@ -708,7 +708,7 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
     auto load_q = [&](int s, int p) {
         const int row = min(p, p1 - 1) * kChunk + 16 * w + m;
 #pragma unroll
-        for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + 32 * ks + 8 * g) * 2u);
+        for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * lda + 32 * ks + 8 * g) * 2u);
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_q(s, p0 + s);
@@ -732,7 +732,7 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
 #pragma unroll
                 for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jt][ks], qc[ks], o);
                 const int col = 16 * jt + 4 * g;
-                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
+                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldo + col) * 2u : kOobOffset;
                 buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the next chunk's waits out of this one
@@ -755,17 +755,17 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
     const WorkItem wi = decode_workgroup(set.count, 1);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
-    const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
-    const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-    const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 2u);
-    const rsrc_t rC = make_rsrc(pr.C + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
-    const rsrc_t rO = make_rsrc(pr.O + (size_t)wi.bh * N * ldc, ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const int di = pr.di, dj = pr.dj, lda = pr.lda, ldb = pr.ldb, ldc = pr.ldc, ldo = pr.ldo;
+    const rsrc_t rA = make_rsrc(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), ((uint32_t)(N - 1) * lda + di) * 2u);
+    const rsrc_t rB = make_rsrc(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), ((uint32_t)(N - 1) * ldb + di) * 2u);
+    const rsrc_t rC = make_rsrc(pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), ((uint32_t)(N - 1) * ldc + dj) * 2u);
+    const rsrc_t rO = make_rsrc(pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), ((uint32_t)(N - 1) * ldo + dj) * 2u);
 
     u32x4 qn[PF][TL::KS];
     auto load_q = [&](int s, int p) {
         const int row = min(p, nchunks - 1) * kChunk + 16 * w + m;
 #pragma unroll
-        for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * di + 32 * ks + 8 * g) * 2u);
+        for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * lda + 32 * ks + 8 * g) * 2u);
     };
 
     // ---- pass 1: S = sum over all chunks of B_c^T C_c
@@ -776,7 +776,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
         u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
         auto load_chunk = [&](int s, int p) {
             const int row0 = min(p, nchunks - 1) * kChunk;
-            load_tile<DI>(rb[s], rB, row0, di, tid);
+            load_tile<DI>(rb[s], rB, row0, ldb, tid);
             load_tile<DJ>(rc[s], rC, row0, ldc, tid);
         };
 #pragma unroll
@@ -828,7 +828,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
 #pragma unroll
                 for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jt][ks], qc[ks], o);
                 const int col = 16 * jt + 4 * g;
-                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldc + col) * 2u : kOobOffset;
+                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldo + col) * 2u : kOobOffset;
                 buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the next chunk's waits out of this one

@@ -15,8 +15,8 @@ import torch
 from torch import nn
 
 from . import ops
-from .autograd import (CustomAttention, CustomAttentionMergedHeads, NonCausalAttention, PrepareInputs,
-                       _autocast_target)
+from .autograd import (CustomAttention, CustomAttentionMergedHeads, NonCausalAttention,
+                       NonCausalAttentionMergedHeads, PrepareInputs, _autocast_target)
 
 
 def _autocast_on():
@@ -220,10 +220,16 @@ class BertCosAttention(nn.Module):
         dt = _autocast_target(query_layer)
         q, k, v = PrepareInputs.apply(query_layer, key_layer, value_layer, keep, cnt, self.norm_const.sigmoid().reshape(h),
                                       dt, None, None, True)
-        context_layer = NonCausalAttention.apply(q, k, v)               # Q (K^T V)  (:249); (QK^T)V at :222 is the same product
-        if not _autocast_on():
-            context_layer = context_layer.to(hidden_states.dtype)
-        context_layer = context_layer.permute(0, 2, 1, 3).contiguous()
+        # Q (K^T V)  (:249); (QK^T)V at :222 is the same product
+        if ops.merged_heads_supported(q.dtype, s, h, q.shape[-1], v.shape[-1]):
+            context_layer = NonCausalAttentionMergedHeads.apply(q, k, v)  # already (B,S,H,D) (:251)
+            if not _autocast_on():
+                context_layer = context_layer.to(hidden_states.dtype)
+        else:
+            context_layer = NonCausalAttention.apply(q, k, v)
+            if not _autocast_on():
+                context_layer = context_layer.to(hidden_states.dtype)
+            context_layer = context_layer.permute(0, 2, 1, 3).contiguous()
         context_layer = context_layer.view(context_layer.size()[:-2] + (self.all_head_size,))
         outputs = (context_layer, None) if output_attentions else (context_layer,)
         if self.is_decoder:

@@ -185,30 +185,33 @@ def causal_backward(q, k, v, grad_out, merged_heads=False):
     return dq, dk_, dv_
 
 
-def noncausal_dot_product(q, k, v):
-    """o = q (k^T v) per (batch, head): BERT_Trainer/BertCosAttention.py:249."""
+def noncausal_dot_product(q, k, v, merged_heads=False):
+    """o = q (k^T v) per (batch, head): BERT_Trainer/BertCosAttention.py:249.  merged_heads: o as (B,N,H,Dv)
+    (the context-layer permute of :251-252 without its copy; see merged_heads_supported)."""
     _require_gpu(Q=q, K=k, V=v)
     b, h, n, dk, dv = _shapes(q, k, v)
     if not (q.dtype == k.dtype == v.dtype):
         raise RuntimeError("Q, K and V must have the same dtype")
     code = _dtype_code(q)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
+    o = torch.empty((b, n, h, dv) if merged_heads else (b, h, n, dv), dtype=q.dtype, device=q.device)
     L = _loader.lib()
     with _on(q.device):
         ws, ws_ptr = _workspace(_ws_bytes("cott_noncausal_workspace_bytes", b, h, n, dk, dv, code), q.device)
-        rc = L.cott_noncausal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,
-                                  ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
-    _check(rc, "cott_noncausal_fwd")
+        fn = L.cott_noncausal_fwd_bnhd if merged_heads else L.cott_noncausal_fwd
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code, ws_ptr,
+                ws.numel() if ws is not None else 0, _stream(q.device))
+    _check(rc, "cott_noncausal_fwd_bnhd" if merged_heads else "cott_noncausal_fwd")
     return o
 
 
-def noncausal_backward(q, k, v, grad_out):
-    """(dQ, dK, dV) of noncausal_dot_product."""
+def noncausal_backward(q, k, v, grad_out, merged_heads=False):
+    """(dQ, dK, dV) of noncausal_dot_product (grad_out (B,N,H,Dv) with merged_heads)."""
     _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)
     b, h, n, dk, dv = _shapes(q, k, v)
-    if grad_out.shape != v.shape:
-        raise RuntimeError(f"prev_grad must have V's shape {tuple(v.shape)}, got {tuple(grad_out.shape)}")
+    want = (b, n, h, dv) if merged_heads else tuple(v.shape)
+    if tuple(grad_out.shape) != want:
+        raise RuntimeError(f"prev_grad must have shape {want}, got {tuple(grad_out.shape)}")
     if not (q.dtype == k.dtype == v.dtype == grad_out.dtype):
         raise RuntimeError("Q, K, V and prev_grad must have the same dtype")
     code = _dtype_code(q)
@@ -217,10 +220,10 @@ def noncausal_backward(q, k, v, grad_out):
     L = _loader.lib()
     with _on(q.device):
         ws, ws_ptr = _workspace(_ws_bytes("cott_noncausal_workspace_bytes", b, h, n, dk, dv, code), q.device)
-        rc = L.cott_noncausal_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(),
-                                  dk_.data_ptr(), dv_.data_ptr(), b, h, n, dk, dv, code, ws_ptr,
-                                  ws.numel() if ws is not None else 0, _stream(q.device))
-    _check(rc, "cott_noncausal_bwd")
+        fn = L.cott_noncausal_bwd_bnhd if merged_heads else L.cott_noncausal_bwd
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), b, h,
+                n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
+    _check(rc, "cott_noncausal_bwd_bnhd" if merged_heads else "cott_noncausal_bwd")
     return dq, dk_, dv_
 
 

@@ -113,6 +113,17 @@ COTT_API int cott_noncausal_bwd(const void *q, const void *k, const void *v, con
                        int B, int H, int N, int Dk, int Dv, int dtype,
                        void *workspace, size_t workspace_bytes, void *stream);
 
+/* Non-causal form with o / d_o laid out (B,N,H,Dv): the context-layer permute of
+ * BERT_Trainer/BertCosAttention.py:251-252 and its backward without the copy.  Same limits as
+ * cott_causal_fwd_bnhd; workspace: cott_noncausal_workspace_bytes. */
+COTT_API int cott_noncausal_fwd_bnhd(const void *q, const void *k, const void *v, void *o,
+                            int B, int H, int N, int Dk, int Dv, int dtype,
+                            void *workspace, size_t workspace_bytes, void *stream);
+COTT_API int cott_noncausal_bwd_bnhd(const void *q, const void *k, const void *v, const void *d_o,
+                            void *dq, void *dk, void *dv,
+                            int B, int H, int N, int Dk, int Dv, int dtype,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- recurrent decode step ------------------------------------------------------------------
  *   S[b,h,dk,dv] += k[b,h,dk] * v[b,h,dv] ;  o[b,h,dv] = sum_dk q[b,h,dk] * S[b,h,dk,dv]
  * Replaces the per-token body of GPT_Trainer/GPTCosAttention.py:262-269 (:264 update, :267 read;

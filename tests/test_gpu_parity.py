@@ -110,6 +110,25 @@ def test_merged_heads_layout(ct, oracle, case):
         assert rel_l2(got, ref) <= TOL[dt], name
 
 
+@pytest.mark.parametrize("case", [(2, 12, 512, 64, 64, BF), (1, 3, 63, 64, 32, HF), (1, 2, 9000, 128, 128, BF), (2, 5, 300, 48, 80, BF)],
+                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_merged_heads_layout_noncausal(ct, oracle, case):
+    """cott_noncausal_fwd_bnhd / cott_noncausal_bwd_bnhd against the (B,H,N,D) entry points (bit for bit) and the
+    oracle; the third shape is cut into sequence groups (group-state, prefix and apply kernels)."""
+    b, h, n, dk, dv, dt = case
+    say("merged heads, non-causal", case)
+    q, k, v, do = inputs(b, h, n, dk, dv, dt, seed=n + 11)
+    qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
+    om = ct.noncausal_dot_product(qd, kd, vd, merged_heads=True)
+    assert om.shape == (b, n, h, dv)
+    assert torch.equal(om.permute(0, 2, 1, 3), ct.noncausal_dot_product(qd, kd, vd))
+    assert rel_l2(om.permute(0, 2, 1, 3), oracle.noncausal(q, k, v)) <= TOL[dt]
+    plain = ct.noncausal_backward(qd, kd, vd, dod)
+    merged = ct.noncausal_backward(qd, kd, vd, dod.permute(0, 2, 1, 3).contiguous(), merged_heads=True)
+    for name, got, want in zip(("dQ", "dK", "dV"), merged, plain):
+        assert torch.equal(got, want), name
+
+
 def test_merged_heads_layout_is_refused_where_not_built(ct):
     q, k, v, _ = inputs(1, 2, 64, 64, 64, F32, seed=3)
     assert not ct.merged_heads_supported(F32, 64, 2, 64, 64)
