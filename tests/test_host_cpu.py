@@ -73,6 +73,11 @@ def test_workspace_queries_are_pure_host_functions():
     assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 4 * 128 * 64 * 64 * 4
     assert L.cott_causal_workspace_bytes(32, 16, 2048, 64, 64, _loader.F32) == 0
     assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F64) == 0
+    # Few heads, long sequence (groups needed with or without column halves): whole problems in 16 groups of 16
+    # chunks, 16 heads x 16 groups x 128 x 128 floats ...
+    assert L.cott_causal_workspace_bytes(1, 16, 16384, 128, 128, _loader.BF16) == 16 * 16 * 128 * 128 * 4
+    # ... but with only 4 chunks per group that way, two column halves in 8 groups of 8 chunks
+    assert L.cott_causal_workspace_bytes(1, 16, 4096, 128, 128, _loader.BF16) == 2 * 16 * 8 * 128 * 64 * 4
     # fp32 non-causal always stages K^T V through the workspace
     assert L.cott_noncausal_workspace_bytes(32, 12, 512, 64, 64, _loader.F32) > 0
     assert L.cott_causal_bwd_workspace_bytes(1, 2, 8192, 64, 64, _loader.BF16) > 0
