@@ -80,6 +80,28 @@ def test_causal_backward(ct, oracle, case):
         assert rel_l2(got, ref) <= TOL[dt], name
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes_all_forms(ct, oracle, seed):
+    """Shapes drawn at random (ragged lengths, unequal head dims, every launch form the planner can pick for small
+    problems): causal forward in both directions, causal and non-causal gradients, against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    b, h = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+    n = int(rng.choice([1, 17, 64, 65, 127, 200, 333, 640, 1000]))
+    dk = int(rng.choice([32, 48, 64, 80, 96, 128]))
+    dv = int(rng.choice([32, 48, 64, 80, 96, 128]))
+    dt = [BF, HF, F32][int(rng.integers(0, 3))]
+    say("random shape", seed, (b, h, n, dk, dv, dt))
+    q, k, v, do = inputs(b, h, n, dk, dv, dt, seed=seed)
+    qd, kd, vd, dod = q.to(DEV), k.to(DEV), v.to(DEV), do.to(DEV)
+    for rev in (False, True):
+        assert rel_l2(ct.causal_dot_product(qd, kd, vd, rev), oracle.causal(q, k, v, rev)) <= TOL[dt], ("causal", rev)
+    for name, got, ref in zip(("dQ", "dK", "dV"), ct.causal_backward(qd, kd, vd, dod), oracle.causal_bwd(q, k, v, do)):
+        assert rel_l2(got, ref) <= TOL[dt], name
+    assert rel_l2(ct.noncausal_dot_product(qd, kd, vd), oracle.noncausal(q, k, v)) <= TOL[dt]
+    for name, got, ref in zip(("dQ", "dK", "dV"), ct.noncausal_backward(qd, kd, vd, dod), oracle.noncausal_bwd(q, k, v, do)):
+        assert rel_l2(got, ref) <= TOL[dt], "non-causal " + name
+
+
 MERGED_CASES = [
     # b, h, n, dk, dv, dtype                   launch form the shape takes
     (2, 16, 2048, 64, 64, BF),    # forward: two column halves per head; gradients: dQ + (dK, dV) pair workgroups
