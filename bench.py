@@ -34,6 +34,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary configs (non-causal, decode, long)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--block-only", action="store_true",
+                    help="run only the GPT attention block fwd+bwd (a secondary figure) for --steps steps: for profiling")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -94,6 +96,12 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.block_only:
+        block_step = gpt_block_step(torch, dev)
+        s = time_region(torch, lambda: block_step(False), args.steps, args.warmup)
+        print(json.dumps({"gpt_block_fwd_bwd_B8_S2048_E1024_H16_autocast_bf16_us": s * 1e6, "steps": args.steps,
+                          "warmup": args.warmup}))
+        return
     B, H, N, D = 8, 16, 2048, 64
     q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
 
@@ -197,6 +205,24 @@ def cold_cache_kernel_times(torch, ct, dev, q, k, v, do):
     return out
 
 
+def gpt_block_step(torch, dev):
+    """step(use_cache): forward + backward of one GPT attention block (B8 S2048 E1024 H16) under bf16 autocast.
+    use_cache=True makes the module return the rotated keys, i.e. rotary and head permutes run as torch ops."""
+    from types import SimpleNamespace
+    from cottention_transformer_amd import modules
+    cfg = SimpleNamespace(max_position_embeddings=2048, attn_pdrop=0.0, resid_pdrop=0.0, hidden_size=1024,
+                          num_attention_heads=16, rotary_dim=64)
+    blk = modules.GPTCosAttention(cfg).to(dev)
+    hid = torch.randn(8, 2048, 1024, device=dev, requires_grad=True)
+    gout = torch.randn(8, 2048, 1024, device=dev, dtype=torch.bfloat16)
+
+    def step(use_cache):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = blk(hid, use_cache=use_cache)[0]
+        out.backward(gout)
+    return step
+
+
 def run_extras(torch, ct, dev):
     """Secondary configurations of the same path (not the headline value)."""
     ex = {}
@@ -281,24 +307,13 @@ def run_extras(torch, ct, dev):
     del keep, cnt, sig
     # whole GPT attention block (projections, rotary, preparation, attention, output projection), fwd+bwd under
     # bf16 autocast at the GPT-300M shape; second figure: same block with rotary / head permute as torch ops
-    from types import SimpleNamespace
-    from cottention_transformer_amd import modules
-    cfg = SimpleNamespace(max_position_embeddings=2048, attn_pdrop=0.0, resid_pdrop=0.0, hidden_size=1024,
-                          num_attention_heads=16, rotary_dim=64)
-    blk = modules.GPTCosAttention(cfg).to(dev)
-    hid = torch.randn(8, 2048, 1024, device=dev, requires_grad=True)
-    gout = torch.randn(8, 2048, 1024, device=dev, dtype=torch.bfloat16)
-
-    def block_step(use_cache):
-        with torch.autocast("cuda", dtype=torch.bfloat16):
-            out = blk(hid, use_cache=use_cache)[0]
-        out.backward(gout)
+    block_step = gpt_block_step(torch, dev)
     s_fused = time_region(torch, lambda: block_step(False), 20, 3)
     s_torch = time_region(torch, lambda: block_step(True), 20, 3)
     ex["gpt_block_fwd_bwd_B8_S2048_E1024_H16_autocast_bf16"] = {
         "us": s_fused * 1e6, "tokens_per_s": 8 * 2048 / s_fused,
         "us_with_rotary_and_permute_as_torch_ops": s_torch * 1e6}
-    del blk, hid, gout
+    del block_step
     ex["fp32_fwd_bwd_B8_H16_N2048_D64"] = {"us": s * 1e6, "tokens_per_s": 8 * 2048 / s, "GBps": byts / s / 1e9,
                                            "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS,
                                            "executed_tflops": flops / s / 1e12,
