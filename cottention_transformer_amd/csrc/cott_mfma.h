@@ -564,7 +564,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 }
 
 // One problem per workgroup: OW output wavefronts (IB = 4/OW blocks each), 4 state, LW loader.
-template <class TR, int DI, int DJ, int PF, int OW, int LW>
+template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false>
 __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set, int BH, int N, int nchunks,
                                                                   int cpg, int G) {
     using TL = Tiling<DI, DJ>;
@@ -577,6 +577,9 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
     __shared__ __attribute__((aligned(16))) u16 sS[2 * SSZ];
+    // STAGED: output tiles go through LDS and leave as 16-byte row segments from the loader wavefronts (StagedOut;
+    // the layout has room for two tiles per buffer, this kernel uses the first)
+    __shared__ __attribute__((aligned(16))) u16 sO[STAGED ? 2 * 2 * kChunk * TL::OS : 8];
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const WorkItem wi = decode_workgroup(set.count, G);
@@ -590,8 +593,16 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     r.p1 = min(r.p0 + cpg, nchunks);
     r.reversed = pr.reversed;
     if (wv >= OW + 4) {
+        StagedOut so;
+        so.O[0] = pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh);
+        so.dj[0] = dj;
+        so.ld[0] = pr.ldo;
+        so.O[1] = nullptr;
+        so.dj[1] = 0;
+        so.ld[1] = 0;
+        so.sO = sO;
         loader_role<DI, DJ, PF, LT>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
-                                    di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC);
+                                    di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC, STAGED ? &so : nullptr);
     } else if (wv >= OW) {
         state_role<TR, DI, DJ, false>(
             pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr,
@@ -600,7 +611,7 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     } else {
         output_role<TR, DI, DJ, PF, IB>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
                                         pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r, IB * wv, l,
-                                        sB, sC, sS);
+                                        sB, sC, sS, STAGED ? sO : nullptr);
     }
 }
 
