@@ -319,6 +319,15 @@ def run_extras(torch, ct, dev):
                                            "executed_tflops": flops / s / 1e12,
                                            "frac_mfma_fp32": flops / s / 1e12 / 157.3}
     del q, k, v, do
+    # For scale: what plain torch kernels stream on this GPU over 1 GiB buffers (far beyond the caches)
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    gb = src.numel() * 4 / 1e9
+    ex["torch_streaming_1GiB_GBps"] = {
+        "read_sum": gb / time_region(torch, lambda: src.sum(), 10, 2),
+        "write_fill": gb / time_region(torch, lambda: dst.fill_(1.0), 10, 2),
+        "copy_read_plus_write": 2 * gb / time_region(torch, lambda: dst.copy_(src), 10, 2)}
+    del src, dst
     return ex
 
 
