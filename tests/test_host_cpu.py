@@ -103,6 +103,16 @@ def test_c_abi_argument_errors_without_a_gpu():
     # empty problems are a no-op
     assert L.cott_causal_fwd(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, 0, None, 0, None) == _loader.OK
     assert L.cott_decode_step(16, 16, 16, 16, 16, 1, 1, 32, 30, _loader.F32, None) == _loader.ERR_UNSUPPORTED
+    # o / d_o in the projection layout (B,N,H,D): 16-bit MFMA shapes only, 32-bit offsets inside a batch element
+    assert L.cott_causal_fwd_bnhd(16, 16, 16, 16, 1, 2, 64, 64, 64, _loader.F32, None, 0, None) == _loader.ERR_UNSUPPORTED
+    assert "bf16 / fp16" in _loader.last_error()
+    assert L.cott_causal_bwd_bnhd(16, 16, 16, 16, 16, 16, 16, 1, 2, 64, 256, 256, _loader.BF16, None, 0,
+                                  None) == _loader.ERR_UNSUPPORTED
+    assert "head dims" in _loader.last_error()
+    assert L.cott_noncausal_fwd_bnhd(16, 16, 16, 16, 1, 4096, 8192, 64, 64, _loader.BF16, None, 0,
+                                     None) == _loader.ERR_UNSUPPORTED
+    assert "2^30" in _loader.last_error()
+    assert L.cott_causal_fwd_bnhd(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, None, 0, None) == _loader.OK
 
 
 # ---- host layer mirrors the reference's checks ----------------------------------------------------
