@@ -33,6 +33,7 @@ SIGNATURES = {
     "cott_noncausal_fwd_bnhd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_bwd_bnhd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_decode_step": (_i, [_vp] * 5 + [_i] * 5 + [_vp]),
+    "cott_decode_step_prep": (_i, [_vp] * 6 + [ctypes.c_float, _vp, ctypes.c_longlong] + [_i] * 7 + [_vp]),
     "cott_profile_enable": (_i, [_i]),
     "cott_profile_read": (_i, [_i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_long)]),
     "cott_kernel_name": (ctypes.c_char_p, [_i]),

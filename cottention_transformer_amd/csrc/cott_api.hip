@@ -571,6 +571,34 @@ int cott_decode_step(void *state, const void *q, const void *k, const void *v, v
     return COTT_OK;
 }
 
+int cott_decode_step_prep(void *state, const void *q, const void *k, const void *v, void *o, const float *sig, float cnt,
+                          const float *rot_table, long long position, int rotary_dim, int table_rows, int B, int H,
+                          int Dk, int Dv, int dtype, void *stream) {
+    const char *fn = "cott_decode_step_prep";
+    if (elem_size(dtype) == 0) return fail(COTT_ERR_INVALID, "%s: unknown dtype %d", fn, dtype);
+    if (B < 0 || H < 0 || Dk < 1 || Dv < 1) return fail(COTT_ERR_INVALID, "%s: bad size", fn);
+    const int nv = Dv / 4;
+    if (Dv % 4 != 0 || !(nv == 8 || nv == 16 || nv == 32 || nv == 64) || Dk > 256)
+        return fail(COTT_ERR_UNSUPPORTED, "%s: needs Dv in {32, 64, 128, 256} and Dk <= 256 (got Dk=%d Dv=%d)", fn, Dk, Dv);
+    const long BH = (long)B * H;
+    if (BH == 0) return COTT_OK;
+    if (BH >= (1L << 31)) return fail(COTT_ERR_UNSUPPORTED, "%s: B*H too large", fn);
+    if (!state || !q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null pointer", fn);
+    if (!aligned16(state) || (dtype == COTT_F64 && (reinterpret_cast<uintptr_t>(state) & 31u)))
+        return fail(COTT_ERR_INVALID, "%s: state must be 16-byte (fp64: 32-byte) aligned", fn);
+    long long pos = 0;
+    if (rot_table != nullptr) {
+        if (rotary_dim < 2 || rotary_dim % 2 != 0 || rotary_dim > Dk)
+            return fail(COTT_ERR_INVALID, "%s: rotary_dim must be even and in [2, Dk] (got %d)", fn, rotary_dim);
+        if (table_rows < 1) return fail(COTT_ERR_INVALID, "%s: empty rotary table", fn);
+        pos = position < 0 ? 0 : (position >= table_rows ? table_rows - 1 : position);  // clamped like the batched pass
+    }
+    hipError_t e = cott::launch_decode_prep(dtype, state, q, k, v, o, (int)BH, H, Dk, Dv, sig, cnt, rot_table, pos, rotary_dim,
+                                            1e-12f, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: HIP launch failed: %s", fn, hipGetErrorString(e));
+    return COTT_OK;
+}
+
 namespace {
 int check_prep(const char *fn, int B, int H, int N, int Dk, int Dv, int d0, int d1) {
     if (elem_size(d0) == 0 || elem_size(d1) == 0) return fail(COTT_ERR_INVALID, "%s: unknown dtype", fn);

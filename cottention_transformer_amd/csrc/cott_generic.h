@@ -216,11 +216,24 @@ __global__ __launch_bounds__(256) void decode_kernel(SF *__restrict__ S, const t
 // LDS slice while the first batch of state loads is in flight; the row groups are combined with
 // lane-xor shuffles.  Plain (cacheable) loads and stores: a state that fits the last-level cache is
 // then served from it on the next step.
+// Optional preparation of the raw projections of the ONE new token inside the decode step (on = 1): GPT-J
+// rotation of the first R columns of q and k by the table row `pos`, L2 normalisation of q and k, and
+// v / max(cnt^sig[h], 1) -- what GPT_Trainer/GPTCosAttention.py:216-241,453-475 do with separate kernels before
+// the recurrence of :264-267.  dk <= 256.
+struct DecodePrep {
+    const float *sig;  // (H) sigmoid(norm_const), or null: no value scaling
+    const float *rot;  // (rows, R) table [sin | cos], or null: no rotation
+    long long pos;     // table row, already clamped to the table
+    float cnt, eps;    // number of tokens so far including this one; norm clamp
+    int R, H, on;
+};
+
 template <class ST, class SF>
 __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, const typename ST::elem *__restrict__ q,
                                                           const typename ST::elem *__restrict__ k,
                                                           const typename ST::elem *__restrict__ v,
-                                                          typename ST::elem *__restrict__ o, int BH, int dk, int dv) {
+                                                          typename ST::elem *__restrict__ o, int BH, int dk, int dv,
+                                                          DecodePrep prep) {
     typedef SF __attribute__((ext_vector_type(4))) sf4;
     constexpr int U = 16;
     extern __shared__ __attribute__((aligned(32))) unsigned char smem_raw[];
@@ -250,14 +263,53 @@ __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, co
             if (r < dk) s[u] = col[(size_t)r * nv];
         }
         if (!staged) {
-            for (int i = lane; i < dk; i += 64) {
-                sq[i] = (SF)ST::load(q + i);
-                sk[i] = (SF)ST::load(k + i);
-            }
             vv.x = (SF)ST::load(v + 4 * mc);
             vv.y = (SF)ST::load(v + 4 * mc + 1);
             vv.z = (SF)ST::load(v + 4 * mc + 2);
             vv.w = (SF)ST::load(v + 4 * mc + 3);
+            if (prep.on) {
+                // element i = lane + 64 t of q and k lives in lane `lane`; the pair partner of the rotation (i ^ 1) in
+                // the neighbouring lane; every lane takes part in every shuffle
+                SF xq[4], xk[4], ssq = 0, ssk = 0;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int i = lane + 64 * t;
+                    xq[t] = i < dk ? (SF)ST::load(q + i) : (SF)0;
+                    xk[t] = i < dk ? (SF)ST::load(k + i) : (SF)0;
+                    const SF pq = __shfl_xor(xq[t], 1), pk = __shfl_xor(xk[t], 1);
+                    if (prep.rot != nullptr && i < prep.R) {
+                        const SF sn = (SF)prep.rot[prep.pos * prep.R + i / 2];
+                        const SF cs = (SF)prep.rot[prep.pos * prep.R + prep.R / 2 + i / 2];
+                        xq[t] = (i & 1) ? xq[t] * cs + pq * sn : xq[t] * cs - pq * sn;
+                        xk[t] = (i & 1) ? xk[t] * cs + pk * sn : xk[t] * cs - pk * sn;
+                    }
+                    ssq += xq[t] * xq[t];
+                    ssk += xk[t] * xk[t];
+                }
+                for (int off = 1; off < 64; off <<= 1) {
+                    ssq += __shfl_xor(ssq, off);
+                    ssk += __shfl_xor(ssk, off);
+                }
+                const SF nq = sqrt(ssq), nk = sqrt(ssk);
+                const SF rq = (SF)1 / (nq > (SF)prep.eps ? nq : (SF)prep.eps), rk = (SF)1 / (nk > (SF)prep.eps ? nk : (SF)prep.eps);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int i = lane + 64 * t;
+                    if (i < dk) {
+                        sq[i] = xq[t] * rq;
+                        sk[i] = xk[t] * rk;
+                    }
+                }
+                if (prep.sig != nullptr) {
+                    const SF p = prep.cnt > 0.f ? (SF)pow((SF)prep.cnt, (SF)prep.sig[bh % prep.H]) : (SF)0;
+                    if (p > (SF)1) vv = vv * ((SF)1 / p);
+                }
+            } else {
+                for (int i = lane; i < dk; i += 64) {
+                    sq[i] = (SF)ST::load(q + i);
+                    sk[i] = (SF)ST::load(k + i);
+                }
+            }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");

@@ -52,7 +52,7 @@ hipError_t run_generic(const OpDesc &a, int BH, int N, hipStream_t stream) {
 
 template <class ST, class SF>
 hipError_t run_decode(void *state, const void *q, const void *k, const void *v, void *o, int BH, int dk, int dv,
-                      hipStream_t stream) {
+                      const DecodePrep &prep, hipStream_t stream) {
     typedef typename ST::elem E;
     ProfScope ps(K_DECODE, stream);
     const int nv = dv / 4;
@@ -61,9 +61,10 @@ hipError_t run_decode(void *state, const void *q, const void *k, const void *v, 
         const size_t lds_w = (size_t)4 * 2 * dk * sizeof(SF);
         decode_wave_kernel<ST, SF><<<dim3((unsigned)((BH + 3) / 4)), dim3(256), lds_w, stream>>>(
             static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
-            static_cast<E *>(o), BH, dk, dv);
+            static_cast<E *>(o), BH, dk, dv, prep);
         return hipGetLastError();
     }
+    if (prep.on) return hipErrorInvalidValue;  // the fused preparation exists in the one-wavefront-per-head kernel only
     const size_t lds = (size_t)2 * dk * sizeof(SF) + 256 * 4 * sizeof(SF);
     decode_kernel<ST, SF><<<dim3((unsigned)BH), dim3(256), lds, stream>>>(
         static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
@@ -88,15 +89,38 @@ hipError_t launch_generic(int dtype, bool causal, const OpDesc &a, int BH, int N
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_decode(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH,
-                         int dk, int dv, hipStream_t stream) {
+namespace {
+hipError_t decode_any(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH, int dk, int dv,
+                      const DecodePrep &prep, hipStream_t stream) {
     switch (dtype) {
-        case COTT_F32: return run_decode<StF32, float>(state, q, k, v, o, BH, dk, dv, stream);
-        case COTT_F64: return run_decode<StF64, double>(state, q, k, v, o, BH, dk, dv, stream);
-        case COTT_F16: return run_decode<StFp16, float>(state, q, k, v, o, BH, dk, dv, stream);
-        case COTT_BF16: return run_decode<StBf16, float>(state, q, k, v, o, BH, dk, dv, stream);
+        case COTT_F32: return run_decode<StF32, float>(state, q, k, v, o, BH, dk, dv, prep, stream);
+        case COTT_F64: return run_decode<StF64, double>(state, q, k, v, o, BH, dk, dv, prep, stream);
+        case COTT_F16: return run_decode<StFp16, float>(state, q, k, v, o, BH, dk, dv, prep, stream);
+        case COTT_BF16: return run_decode<StBf16, float>(state, q, k, v, o, BH, dk, dv, prep, stream);
     }
     return hipErrorInvalidValue;
+}
+}  // namespace
+
+hipError_t launch_decode(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH,
+                         int dk, int dv, hipStream_t stream) {
+    DecodePrep none{};
+    return decode_any(dtype, state, q, k, v, o, BH, dk, dv, none, stream);
+}
+
+hipError_t launch_decode_prep(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH, int H,
+                              int dk, int dv, const float *sig, float cnt, const float *rot, long long pos, int R,
+                              float eps, hipStream_t stream) {
+    DecodePrep p{};
+    p.sig = sig;
+    p.rot = rot;
+    p.pos = pos;
+    p.cnt = cnt;
+    p.eps = eps;
+    p.R = R;
+    p.H = H;
+    p.on = 1;
+    return decode_any(dtype, state, q, k, v, o, BH, dk, dv, p, stream);
 }
 
 }  // namespace cott

@@ -82,5 +82,11 @@ hipError_t launch_prep(bool backward, const void *const x[3], const void *const 
 
 hipError_t launch_decode(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH,
                          int dk, int dv, hipStream_t stream);
+// The same step on the raw projections of the new token: rotation by table row `pos` (rot null = none), L2
+// normalisation of q and k, v / max(cnt^sig[h], 1) (sig null = none) happen inside the kernel.  dv / 4 in
+// {8,16,32,64} and dk <= 256, else hipErrorInvalidValue.
+hipError_t launch_decode_prep(int dtype, void *state, const void *q, const void *k, const void *v, void *o, int BH, int H,
+                              int dk, int dv, const float *sig, float cnt, const float *rot, long long pos, int R,
+                              float eps, hipStream_t stream);
 
 }  // namespace cott

@@ -87,6 +87,27 @@ class GPTCosAttention(nn.Module):
         self.state = None
         self.cur_s = 1
 
+    def _decode_one(self, query, key, value):
+        """One new token in recurrent inference, from the raw projections (B,1,H,D): rotation by position
+        cur_s - 1, normalisation, value scaling by cur_s ** sigmoid(norm_const) and the state update / read-out
+        (GPTCosAttention.py:216-241, 253-272, 453-475) as one kernel launch.  Returns (B,1,H*D)."""
+        b, _, h, d = query.shape
+        query, key, value = _common_dtype(query, key, value)
+        if self.state is None:
+            self.state = torch.zeros(b, h, d, value.shape[-1], device=query.device,
+                                     dtype=torch.float64 if query.dtype == torch.float64 else torch.float32)
+        cached = getattr(self, "_sig_cache", None)
+        if cached is None or cached[0] != self.norm_const._version or cached[1].device != query.device:
+            cached = (self.norm_const._version, self.norm_const.detach().sigmoid().reshape(h).float().to(query.device))
+            self._sig_cache = cached
+        table = self.embed_positions
+        if table.device != query.device:
+            table = self.embed_positions = table.to(query.device)
+        out = ops.decode_step_prepared(self.state, query, key, value, sig=cached[1], cnt=float(self.cur_s),
+                                       rotary=(table, self.cur_s - 1))
+        self.cur_s += 1
+        return out.reshape(b, 1, h * value.shape[-1])
+
     def _split_heads(self, tensor):
         return tensor.view(tensor.size()[:-1] + (self.num_attention_heads, self.head_dim))  # (B,S,H,D)
 
@@ -148,6 +169,14 @@ class GPTCosAttention(nn.Module):
         query = self._split_heads(self.q_proj(hidden_states))          # (B,S,H,D)
         key = self._split_heads(self.k_proj(hidden_states))
         value = self._split_heads(self.v_proj(hidden_states))
+        if (self.fast_inference and hidden_states.shape[1] == 1 and position_ids is None and layer_past is None
+                and use_cache is not True and not output_attentions and attention_mask is None
+                and self.head_dim in (32, 64, 128, 256) and self.rotary_dim is not None
+                and self.rotary_dim % 2 == 0 and self.rotary_dim <= self.head_dim):
+            attn_output = self._decode_one(query, key, value)
+            if not _autocast_on():
+                attn_output = attn_output.to(hidden_states.dtype)
+            return (self.resid_dropout(self.out_proj(attn_output)), None)
         if position_ids is None:
             start = self.cur_s - 1 if self.fast_inference else 0
             position_ids = torch.arange(start, start + hidden_states.shape[1], device=hidden_states.device)

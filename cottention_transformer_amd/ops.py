@@ -256,6 +256,51 @@ def decode_step(state, q, k, v, out=None):
     return out
 
 
+def decode_step_prepared(state, q, k, v, sig=None, cnt=0.0, rotary=None, out=None):
+    """decode_step on the RAW projections of the new token: rotation (rotary = (table (P,R) fp32, position int)),
+    L2 normalisation of q and k and v / max(cnt^sig[h], 1) run inside the kernel (one launch instead of
+    prepare_inputs + decode_step).  q, k: (B,H,Dk) or the (B,1,H,Dk) projection output; v likewise; sig: (H) or
+    None; cnt: number of tokens so far including this one."""
+    if q.dim() == 4 and q.shape[1] == 1:
+        q, k, v = q[:, 0], k[:, 0], v[:, 0]
+    _require_gpu(state=state, q=q, k=k, v=v)
+    if state.dim() != 4 or q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise RuntimeError("decode_step_prepared: state (B,H,Dk,Dv), q/k (B,H,Dk), v (B,H,Dv)")
+    b, h, dk, dv = state.shape
+    if q.shape != (b, h, dk) or k.shape != (b, h, dk) or v.shape != (b, h, dv):
+        raise RuntimeError("decode_step_prepared: q/k/v do not match the state shape")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("q, k and v must have the same dtype")
+    code = _dtype_code(q)
+    want = torch.float64 if q.dtype == torch.float64 else torch.float32
+    if state.dtype != want or not state.is_contiguous():
+        raise RuntimeError(f"decode_step_prepared: state must be a contiguous {want} tensor")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    if out is None:
+        out = torch.empty((b, h, dv), dtype=q.dtype, device=q.device)
+    elif out.shape != (b, h, dv) or out.dtype != q.dtype or not out.is_contiguous() or out.device != q.device:
+        raise RuntimeError("decode_step_prepared: bad `out` tensor")
+    if sig is not None:
+        if sig.shape != (h,):
+            raise RuntimeError(f"sig must have shape {(h,)}")
+        sig = sig.detach().to(device=q.device, dtype=torch.float32).contiguous()
+    table, pos, rdim, rows = None, 0, 0, 0
+    if rotary is not None:
+        table, pos = rotary
+        if table.dim() != 2 or table.dtype != torch.float32 or table.device != q.device or not table.is_contiguous():
+            raise RuntimeError("rotary table must be a contiguous float32 (positions, rotary_dim) tensor on the inputs' device")
+        rows, rdim = table.shape
+        pos = int(pos)
+    L = _loader.lib()
+    with _on(q.device):
+        rc = L.cott_decode_step_prep(state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                     sig.data_ptr() if sig is not None else None, float(cnt),
+                                     table.data_ptr() if table is not None else None, pos, rdim, rows, b, h, dk, dv, code,
+                                     _stream(q.device))
+    _check(rc, "cott_decode_step_prep")
+    return out
+
+
 def _prep_side_inputs(b, h, n, keep, cnt, sig, device):
     if keep is not None:
         if keep.shape != (b, n):

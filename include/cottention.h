@@ -133,6 +133,18 @@ COTT_API int cott_noncausal_bwd_bnhd(const void *q, const void *k, const void *v
 COTT_API int cott_decode_step(void *state, const void *q, const void *k, const void *v, void *o,
                      int B, int H, int Dk, int Dv, int dtype, void *stream);
 
+/* The same step on the RAW projections of the new token: the GPT-J rotation of the first rotary_dim columns of q
+ * and k by row `position` of rot_table ((table_rows, rotary_dim) fp32, [sin | cos]; NULL = no rotation; the row is
+ * clamped to the table), the L2 normalisation of q and k and v / max(cnt^sig[h], 1) (sig: (H) fp32 =
+ * sigmoid(norm_const), NULL = no scaling; cnt = tokens so far including this one) run inside the kernel: one
+ * launch per token and layer instead of the separate elementwise kernels of
+ * GPT_Trainer/GPTCosAttention.py:216-241,453-475 in front of :264-267.  q, k: (B,H,Dk) = the (B,1,H,Dk)
+ * projection output; Dv in {32,64,128,256}, Dk <= 256. */
+COTT_API int cott_decode_step_prep(void *state, const void *q, const void *k, const void *v, void *o,
+                          const float *sig, float cnt, const float *rot_table, long long position,
+                          int rotary_dim, int table_rows,
+                          int B, int H, int Dk, int Dv, int dtype, void *stream);
+
 /* ---- fused input preparation (the elementwise work the module does before the attention op) --
  *   q_out = keep * q / max(|q|_2, 1e-12)     (rows of Dk; same for k)
  *   v_out = keep * v / max(cnt^sig[h], 1)    (rows of Dv)

@@ -222,6 +222,42 @@ def test_decode_steps(ct, oracle, case):
     assert rel_l2(state, ref_state) <= (1e-12 if dt == F64 else 1e-6)
 
 
+@pytest.mark.parametrize("case", [(2, 3, 64, 64, BF, 64), (3, 2, 128, 128, F32, 32), (1, 4, 48, 32, HF, 16), (2, 2, 32, 64, F64, 0)],
+                         ids=lambda c: "x".join(map(str, c[:4])) + "-" + str(c[4]).split(".")[-1] + "-rot" + str(c[5]))
+def test_decode_step_on_raw_projections(ct, case):
+    """cott_decode_step_prep (rotation, normalisation and value scaling inside the decode kernel) over several
+    tokens against the CPU statements of those steps (oracle/torch_forms.py) followed by the plain recurrence."""
+    from oracle import torch_forms as tf
+    b, h, dk, dv, dt, rdim = case
+    say("decode on raw projections", case)
+    g = torch.Generator().manual_seed(dk + dv)
+    steps, npos = 5, 40
+    q, k = (torch.randn(steps, b, 1, h, dk, generator=g).to(dt) for _ in range(2))
+    v = torch.randn(steps, b, 1, h, dv, generator=g).to(dt)
+    sig = torch.sigmoid(torch.randn(h, generator=g))
+    table = tf.gptj_sinusoid_table(npos, rdim).float() if rdim else None
+    sdt = torch.float64 if dt == F64 else torch.float32
+    state = torch.zeros(b, h, dk, dv, dtype=sdt, device=DEV)
+    ref_state = torch.zeros(b, h, dk, dv, dtype=torch.float64)
+    for t in range(steps):
+        cnt, pos = float(t + 1), t + 3
+        out = ct.decode_step_prepared(state, q[t].to(DEV), k[t].to(DEV), v[t].to(DEV), sig=sig.to(DEV), cnt=cnt,
+                                      rotary=(table.to(DEV), pos) if rdim else None)
+        q64, k64, v64 = (x[t][:, 0].double() for x in (q, k, v))          # (B,H,D)
+        if rdim:
+            sn, cs = (x.reshape(1, 1, -1).expand(b, 1, -1) for x in torch.split(table[pos].double(), rdim // 2, dim=-1))
+            rot = lambda x: torch.cat([tf.gptj_rotate(x[..., :rdim].unsqueeze(1), sn, cs).squeeze(1), x[..., rdim:]], -1)
+            q64, k64 = rot(q64), rot(k64)
+        qn = q64 / q64.norm(dim=-1, keepdim=True).clamp(min=1e-12)
+        kn = k64 / k64.norm(dim=-1, keepdim=True).clamp(min=1e-12)
+        vs = v64 / (cnt ** sig.double()).clamp(min=1.0).reshape(1, h, 1)
+        ref_state += kn.unsqueeze(-1) * vs.unsqueeze(-2)
+        want = torch.einsum("bhi,bhij->bhj", qn, ref_state)
+        assert out.shape == (b, h, dv) and out.dtype == dt
+        assert rel_l2(out, want.numpy()) <= TOL[dt], t
+    assert rel_l2(state, ref_state.numpy()) <= (1e-12 if dt == F64 else 2e-6)
+
+
 def test_decode_after_prompt_equals_causal_forward(ct, oracle):
     # GPTCosAttention.py:253-272 vs :282: token-by-token decode reproduces the causal rows
     b, h, n, d = 2, 2, 48, 64
