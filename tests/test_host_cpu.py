@@ -103,6 +103,14 @@ def test_c_abi_argument_errors_without_a_gpu():
     # empty problems are a no-op
     assert L.cott_causal_fwd(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, 0, None, 0, None) == _loader.OK
     assert L.cott_decode_step(16, 16, 16, 16, 16, 1, 1, 32, 30, _loader.F32, None) == _loader.ERR_UNSUPPORTED
+    # decode on raw projections: one wavefront per head needs Dv in {32,64,128,256} and Dk <= 256
+    assert L.cott_decode_step_prep(16, 16, 16, 16, 16, None, 1.0, None, 0, 0, 0, 1, 1, 512, 64, _loader.BF16,
+                                   None) == _loader.ERR_UNSUPPORTED
+    assert L.cott_decode_step_prep(16, 16, 16, 16, 16, None, 1.0, 16, 0, 3, 8, 1, 1, 64, 64, _loader.BF16,
+                                   None) == _loader.ERR_INVALID
+    assert "rotary_dim" in _loader.last_error()
+    assert L.cott_decode_step_prep(None, None, None, None, None, None, 1.0, None, 0, 0, 0, 0, 4, 64, 64, _loader.BF16,
+                                   None) == _loader.OK
     # o / d_o in the projection layout (B,N,H,D): 16-bit MFMA shapes only, 32-bit offsets inside a batch element
     assert L.cott_causal_fwd_bnhd(16, 16, 16, 16, 1, 2, 64, 64, 64, _loader.F32, None, 0, None) == _loader.ERR_UNSUPPORTED
     assert "bf16 / fp16" in _loader.last_error()
