@@ -228,7 +228,7 @@ struct DecodePrep {
     int R, H, on;
 };
 
-template <class ST, class SF>
+template <class ST, class SF, bool PREP>
 __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, const typename ST::elem *__restrict__ q,
                                                           const typename ST::elem *__restrict__ k,
                                                           const typename ST::elem *__restrict__ v,
@@ -263,11 +263,11 @@ __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, co
             if (r < dk) s[u] = col[(size_t)r * nv];
         }
         if (!staged) {
-            vv.x = (SF)ST::load(v + 4 * mc);
-            vv.y = (SF)ST::load(v + 4 * mc + 1);
-            vv.z = (SF)ST::load(v + 4 * mc + 2);
-            vv.w = (SF)ST::load(v + 4 * mc + 3);
-            if (prep.on) {
+            if constexpr (PREP) {
+                vv.x = (SF)ST::load(v + 4 * mc);
+                vv.y = (SF)ST::load(v + 4 * mc + 1);
+                vv.z = (SF)ST::load(v + 4 * mc + 2);
+                vv.w = (SF)ST::load(v + 4 * mc + 3);
                 // element i = lane + 64 t of q and k lives in lane `lane`; the pair partner of the rotation (i ^ 1) in
                 // the neighbouring lane; every lane takes part in every shuffle
                 SF xq[4], xk[4], ssq = 0, ssk = 0;
@@ -309,6 +309,10 @@ __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, co
                     sq[i] = (SF)ST::load(q + i);
                     sk[i] = (SF)ST::load(k + i);
                 }
+                vv.x = (SF)ST::load(v + 4 * mc);
+                vv.y = (SF)ST::load(v + 4 * mc + 1);
+                vv.z = (SF)ST::load(v + 4 * mc + 2);
+                vv.w = (SF)ST::load(v + 4 * mc + 3);
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();

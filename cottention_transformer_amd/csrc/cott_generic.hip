@@ -59,9 +59,14 @@ hipError_t run_decode(void *state, const void *q, const void *k, const void *v, 
     if ((nv == 8 || nv == 16 || nv == 32 || nv == 64) && dk <= 1024) {
         // one wavefront per head, four heads per workgroup
         const size_t lds_w = (size_t)4 * 2 * dk * sizeof(SF);
-        decode_wave_kernel<ST, SF><<<dim3((unsigned)((BH + 3) / 4)), dim3(256), lds_w, stream>>>(
-            static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
-            static_cast<E *>(o), BH, dk, dv, prep);
+        if (prep.on)
+            decode_wave_kernel<ST, SF, true><<<dim3((unsigned)((BH + 3) / 4)), dim3(256), lds_w, stream>>>(
+                static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
+                static_cast<E *>(o), BH, dk, dv, prep);
+        else
+            decode_wave_kernel<ST, SF, false><<<dim3((unsigned)((BH + 3) / 4)), dim3(256), lds_w, stream>>>(
+                static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
+                static_cast<E *>(o), BH, dk, dv, prep);
         return hipGetLastError();
     }
     if (prep.on) return hipErrorInvalidValue;  // the fused preparation exists in the one-wavefront-per-head kernel only
