@@ -314,6 +314,26 @@ def run_extras(torch, ct, dev):
         "us": s_fused * 1e6, "tokens_per_s": 8 * 2048 / s_fused,
         "us_with_rotary_and_permute_as_torch_ops": s_torch * 1e6}
     del block_step
+    # the BERT self-attention block (projections, preparation, non-causal attention), fwd+bwd under bf16 autocast at
+    # the BERT-base shape B32 S512 E768 H12
+    from types import SimpleNamespace as _NS
+    from cottention_transformer_amd import modules as _modules
+    bert = _modules.BertCosAttention(_NS(hidden_size=768, num_attention_heads=12, attention_probs_dropout_prob=0.0)).to(dev)
+    bh_in = torch.randn(32, 512, 768, device=dev, requires_grad=True)
+    bg = torch.randn(32, 512, 768, device=dev, dtype=torch.bfloat16)
+
+    def bert_step():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = bert(bh_in)[0]
+        out.backward(bg)
+    s_b = time_region(torch, bert_step, 20, 3)
+    ex["bert_block_fwd_bwd_B32_S512_E768_H12_autocast_bf16"] = {"us": s_b * 1e6, "tokens_per_s": 32 * 512 / s_b}
+    del bert, bh_in, bg
+    # prompt pass that also hands the state to decoding (cott_causal_fwd_state), headline shape
+    qp, kp, vp, _ = make_inputs(torch, 8, 16, 2048, 64, 64, torch.bfloat16, dev)
+    s_p = time_region(torch, lambda: ct.causal_prefill(qp, kp, vp), 100, 10)
+    ex["prefill_with_state_B8_H16_N2048_D64"] = {"us": s_p * 1e6, "tokens_per_s": 8 * 2048 / s_p}
+    del qp, kp, vp
     ex["fp32_fwd_bwd_B8_H16_N2048_D64"] = {"us": s * 1e6, "tokens_per_s": 8 * 2048 / s, "GBps": byts / s / 1e9,
                                            "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS,
                                            "executed_tflops": flops / s / 1e12,
