@@ -1,0 +1,128 @@
+"""GPU parity at the FULL size of every benchmark configuration, through the C ABI, against the CPU oracle.
+
+The whole-tensor rel-L2 of a long sequence would hide one bad chunk (its share of the norm is 1/sqrt(chunks)), so
+every comparison here also bounds the worst 64-row block of every head.  Bars: rel-L2 <= 2e-2 for bf16 tensors
+(oracle in fp64 on the same rounded inputs), per block as well as overall; the fp32 decode state <= 1e-5."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from util import TOL, inputs, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+
+
+@pytest.fixture(scope="module")
+def ct():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    import cottention_transformer_amd as ct_
+    from cottention_transformer_amd import _loader
+    assert os.path.exists(_loader.lib_path()), "libcottention_hip.so must be prebuilt in-tree"
+    _loader.lib()
+    return ct_
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def worst_block(x, ref, rows=64):
+    """Largest rel-L2 over blocks of `rows` consecutive positions of any head; x, ref: (..., N, D)."""
+    x = x.detach().double().cpu().numpy() if hasattr(x, "detach") else np.asarray(x, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    n, d = ref.shape[-2:]
+    pad = (-n) % rows
+    if pad:
+        widths = [(0, 0)] * (ref.ndim - 2) + [(0, pad), (0, 0)]
+        x, ref = np.pad(x, widths), np.pad(ref, widths)
+    shape = ref.shape[:-2] + ((n + pad) // rows, rows * d)
+    num = np.linalg.norm((x - ref).reshape(shape), axis=-1)
+    den = np.linalg.norm(ref.reshape(shape), axis=-1)
+    return float(np.max(num / np.maximum(den, 1e-300)))
+
+
+def check(name, got, ref, tol):
+    whole, block = rel_l2(got, ref), worst_block(got, ref)
+    say(f"  {name}: rel-L2 {whole:.2e}, worst 64-row block {block:.2e}")
+    assert whole <= tol, name
+    assert block <= tol, name + " (one block)"
+
+
+LONG_CASES = [
+    # b, h, n, dk, dv, dtype                       launch plan the shape takes
+    (1, 16, 65536, 128, 128, BF),   # long-context benchmark configuration: 16 groups of 64 chunks, 128 x 128 tiles
+    (2, 4, 19217, 64, 64, BF),      # dQ + (dK, dV) pair workgroups with several groups of several chunks, ragged tail
+    (1, 4, 8192, 128, 128, HF),     # fp16, few chunks per group
+    (1, 3, 20000, 64, 128, BF),     # Dk != Dv: three separate gradient problems in groups
+]
+
+
+@pytest.mark.parametrize("case", LONG_CASES, ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_long_sequences_forward_and_backward(ct, oracle, case):
+    b, h, n, dk, dv, dt = case
+    say("long sequence", case)
+    q, k, v, do = inputs(b, h, n, dk, dv, dt, seed=n)
+    qd, kd, vd, gd = (x.to(DEV) for x in (q, k, v, do))
+    check("O", ct.causal_dot_product(qd, kd, vd), oracle.causal(q, k, v), TOL[dt])
+    check("O reversed", ct.causal_dot_product(qd, kd, vd, True), oracle.causal(q, k, v, True), TOL[dt])
+    for name, got, ref in zip(("dQ", "dK", "dV"), ct.causal_backward(qd, kd, vd, gd), oracle.causal_bwd(q, k, v, do)):
+        check(name, got, ref, TOL[dt])
+
+
+FUSED_NONCAUSAL_CASES = [
+    # shapes whose heads alone fill the chip: one workgroup per head runs both passes over several chunks
+    (32, 12, 512, 64, 64, BF),      # BERT benchmark configuration
+    (16, 16, 300, 64, 32, BF),      # ragged tail, Dk != Dv
+    (32, 8, 300, 128, 128, HF),     # 128-wide heads
+    (16, 16, 1000, 48, 80, BF),     # padded head dims
+]
+
+
+@pytest.mark.parametrize("case", FUSED_NONCAUSAL_CASES,
+                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_noncausal_many_heads_forward_and_backward(ct, oracle, case):
+    b, h, n, dk, dv, dt = case
+    say("non-causal, one workgroup per head", case)
+    q, k, v, do = inputs(b, h, n, dk, dv, dt, seed=n + 5)
+    qd, kd, vd, gd = (x.to(DEV) for x in (q, k, v, do))
+    check("O", ct.noncausal_dot_product(qd, kd, vd), oracle.noncausal(q, k, v), TOL[dt])
+    for name, got, ref in zip(("dQ", "dK", "dV"), ct.noncausal_backward(qd, kd, vd, gd), oracle.noncausal_bwd(q, k, v, do)):
+        check(name, got, ref, TOL[dt])
+
+
+def test_decode_512_steps_at_benchmark_size(ct, oracle):
+    """Decode benchmark configuration: fp32 state (256,16,128,128) ~ N(0, 0.01), bf16 q, k, v, 512 consecutive steps
+    (GPT_Trainer/GPTCosAttention.py:262-269).  The oracle follows every 8th batch element step by step in fp64
+    (outputs compared at steps 1, 256 and 512, its state at the end); the final state of ALL batch elements is
+    compared with s0 + sum_t k_t v_t^T accumulated in fp64."""
+    b, h, d, steps = 256, 16, 128, 512
+    sub = slice(0, b, 8)
+    g = torch.Generator(device=DEV).manual_seed(4)
+    s0 = 0.01 * torch.randn(b, h, d, d, generator=g, device=DEV)
+    qs = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g, device=DEV), dim=-1).to(BF)
+    ks = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g, device=DEV), dim=-1).to(BF)
+    vs = torch.randn(steps, b, h, d, generator=g, device=DEV).to(BF)
+    state = s0.clone()
+    ref_state = s0[sub].double().cpu().numpy().copy()
+    qc, kc, vc = (x[:, sub].cpu() for x in (qs, ks, vs))
+    out = torch.empty(b, h, d, dtype=BF, device=DEV)
+    for t in range(steps):
+        ct.decode_step(state, qs[t], ks[t], vs[t], out=out)
+        ref = oracle.decode_step(ref_state, qc[t], kc[t], vc[t])
+        if t + 1 in (1, 256, 512):
+            err = rel_l2(out[sub], ref)
+            say(f"  step {t + 1}: output rel-L2 {err:.2e}")
+            assert err <= 2e-2, t + 1
+    err = rel_l2(state[sub], ref_state)
+    say(f"  state after {steps} steps vs oracle: {err:.2e}")
+    assert err <= 1e-5
+    total = s0.double()
+    for t0 in range(0, steps, 64):
+        total += torch.einsum("tbhi,tbhj->bhij", ks[t0:t0 + 64].double(), vs[t0:t0 + 64].double())
+    err = float((state.double() - total).norm() / total.norm())
+    say(f"  state of all batch elements vs fp64 sum: {err:.2e}")
+    assert err <= 1e-5
