@@ -18,6 +18,8 @@ SIGNATURES = {
     "cott_last_error": (ctypes.c_char_p, []),
     "cott_causal_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_fwd": (_i, [_vp] * 4 + [_i] * 7 + [_vp, _sz, _vp]),
+    "cott_noalloc_scratch_bytes": (_sz, []),
+    "cott_causal_fwd_noalloc": (_i, [_vp] * 4 + [_i] * 7 + [_vp]),
     "cott_causal_fwd_state": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_prep_fwd": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
     "cott_prep_bwd": (_i, [_vp] * 13 + [_i] * 7 + [_vp]),

@@ -42,6 +42,12 @@ ProfScope::~ProfScope() {
 }
 }  // namespace cott
 
+// Scratch memory of cott_causal_fwd_noalloc: the group-state slots that the other entry points take from the
+// caller's workspace.  Every device the library runs on holds its own copy of this array until the process ends.
+// In host code the name is only a handle for hipGetSymbolAddress; kernels receive the address it returns.
+#define COTT_SCRATCH_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char scratch[COTT_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -375,6 +381,51 @@ int cott_causal_fwd(const void *q, const void *k, const void *v, void *o, int B,
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
     const Op op{q, k, v, o, Dk, Dv, reversed ? 1 : 0};
     return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device, looked up once per device.
+int scratch_of_current_device(const char *fn, void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: hipGetDevice failed: %s", fn, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(COTT_ERR_UNSUPPORTED, "%s: device index %d not below %d", fn, dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr)
+            return fail(COTT_ERR_HIP, "%s: hipGetSymbolAddress(scratch) failed on device %d: %s", fn, dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return COTT_OK;
+}
+}  // namespace
+
+size_t cott_noalloc_scratch_bytes(void) { return (size_t)COTT_SCRATCH_BYTES; }
+
+int cott_causal_fwd_noalloc(const void *q, const void *k, const void *v, void *o, int B, int H, int N, int Dk, int Dv,
+                            int dtype, int reversed, void *stream) {
+    const char *fn = "cott_causal_fwd_noalloc";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    const Op op{q, k, v, o, Dk, Dv, reversed ? 1 : 0};
+    const size_t need = ops_workspace(&op, 1, (long)B * H, N, dtype, true);
+    if (need > (size_t)COTT_SCRATCH_BYTES)
+        return fail(COTT_ERR_WORKSPACE, "%s: this shape needs %zu bytes of group-state slots, the built-in scratch holds %zu; "
+                    "use cott_causal_fwd with a workspace", fn, need, (size_t)COTT_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (need > 0)
+        if (int rc = scratch_of_current_device(fn, &ws)) return rc;
+    return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, ws, need, static_cast<hipStream_t>(stream));
 }
 
 int cott_causal_fwd_state(const void *q, const void *k, const void *v, void *o, const void *state_in, void *state_out,

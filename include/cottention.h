@@ -57,6 +57,19 @@ COTT_API int cott_causal_fwd(const void *q, const void *k, const void *v, void *
                     int B, int H, int N, int Dk, int Dv, int dtype, int reversed,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- causal forward that takes no workspace and allocates nothing ------------------------------
+ * cott_causal_fwd with the group-state slots (its workspace) kept in a device array built into the library
+ * instead of caller memory.  It has no counterpart in the reference; it is for callers that cannot allocate
+ * device memory around the call: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Same arguments, results (bit for bit) and errors as cott_causal_fwd; a shape whose slots exceed
+ * cott_noalloc_scratch_bytes() (32 MiB, enough for every plan this build makes) returns COTT_ERR_WORKSPACE.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); no call allocates or frees.
+ * All calls on one GPU share that GPU's array: calls that may overlap on one GPU (different streams or threads)
+ * race on it and must be ordered by the caller.  Keep cott_profile_enable off (it creates HIP events). */
+COTT_API size_t cott_noalloc_scratch_bytes(void);
+COTT_API int cott_causal_fwd_noalloc(const void *q, const void *k, const void *v, void *o,
+                            int B, int H, int N, int Dk, int Dv, int dtype, int reversed, void *stream);
+
 /* ---- causal forward with state hand-over (prefill -> decode, or a sequence fed in pieces) -----
  *   o[s,j] = sum_i q[s,i] * ( state_in[i,j] + sum_{s' <= s} k[s',i] * v[s',j] )
  *   state_out[i,j] = state_in[i,j] + sum_{s' < N} k[s',i] * v[s',j]

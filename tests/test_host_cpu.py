@@ -123,6 +123,36 @@ def test_c_abi_argument_errors_without_a_gpu():
     assert L.cott_causal_fwd_bnhd(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, None, 0, None) == _loader.OK
 
 
+def test_no_alloc_entry_point_checks_and_its_scratch_symbol(tmp_path):
+    """Argument checks of cott_causal_fwd_noalloc need no GPU; and the built-in scratch array must be a GLOBAL
+    symbol of the library's gfx950 code object, or the runtime cannot resolve it (hipGetSymbolAddress)."""
+    import shutil
+    import subprocess
+    from cottention_transformer_amd import _loader
+    L = _loader.lib()
+    assert L.cott_noalloc_scratch_bytes() == 32 << 20
+    assert L.cott_causal_fwd_noalloc(16, 16, 16, 16, 1, 1, 8, 24, 32, _loader.F32, 0, None) == _loader.ERR_INVALID
+    assert "divisible by 16" in _loader.last_error()
+    assert L.cott_causal_fwd_noalloc(None, 16, 16, 16, 1, 1, 8, 64, 64, _loader.F32, 0, None) == _loader.ERR_INVALID
+    assert L.cott_causal_fwd_noalloc(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, 0, None) == _loader.OK
+    # every plan of the forward pass fits the built-in scratch (at most one 64 KiB slot per workgroup of a full chip)
+    for shape in ((1, 16, 65536, 128, 128), (1, 1, 1 << 20, 128, 128), (3, 5, 30000, 64, 128)):
+        for dt in (_loader.BF16, _loader.F32):
+            assert L.cott_causal_workspace_bytes(*shape, dt) <= L.cott_noalloc_scratch_bytes()
+    objdump, readelf = "/opt/rocm/llvm/bin/llvm-objdump", "/opt/rocm/llvm/bin/llvm-readelf"
+    if not (os.path.exists(objdump) and os.path.exists(readelf)):
+        pytest.skip("llvm-objdump / llvm-readelf not installed")
+    lib = shutil.copy(_loader.lib_path(), tmp_path / "lib.so")
+    subprocess.run([objdump, "--offloading", str(lib)], check=True, stdout=subprocess.DEVNULL, cwd=tmp_path)
+    rows = []
+    for f in os.listdir(tmp_path):
+        if "gfx950" in f:
+            out = subprocess.run([readelf, "-s", "--wide", str(tmp_path / f)], check=True, capture_output=True, text=True).stdout
+            rows += [l for l in out.splitlines() if l.split()[-1:] == ["_ZL7scratch"]]
+    assert rows, "scratch array not found in the device code objects"
+    assert all("GLOBAL" in l and str(32 << 20) in l for l in rows), rows
+
+
 # ---- host layer mirrors the reference's checks ----------------------------------------------------
 
 def test_host_rejects_cpu_tensors_like_the_reference():
