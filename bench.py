@@ -36,6 +36,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--block-only", action="store_true",
                     help="run only the GPT attention block fwd+bwd (a secondary figure) for --steps steps: for profiling")
+    ap.add_argument("--long-only", type=int, default=0, metavar="N",
+                    help="run only the long-context configuration B1 H16 D128 bf16 at sequence length N (fwd and bwd "
+                         "separately, per-kernel durations) for --steps steps: for profiling")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -102,15 +105,17 @@ def main():
         print(json.dumps({"gpt_block_fwd_bwd_B8_S2048_E1024_H16_autocast_bf16_us": s * 1e6, "steps": args.steps,
                           "warmup": args.warmup}))
         return
-    B, H, N, D = 8, 16, 2048, 64
-    q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
-
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.long_only:
+        print(json.dumps(long_context(torch, ct, dev, args.long_only, args.steps, args.warmup)))
+        return
+    B, H, N, D = 8, 16, 2048, 64
+    q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
 
     def step():
         o = ct.causal_dot_product(q, k, v)
@@ -205,6 +210,37 @@ def cold_cache_kernel_times(torch, ct, dev, q, k, v, do):
     return out
 
 
+def long_context(torch, ct, dev, n, steps, warmup, kernels=True):
+    """Long-context configuration B=1 H=16 D=128 bf16 at sequence length n: forward, backward and both, with the
+    per-kernel durations the library records (HIP events around each launch)."""
+    from cottention_transformer_amd import _loader
+    q, k, v, do = make_inputs(torch, 1, 16, n, 128, 128, torch.bfloat16, dev)
+    fwd = lambda: ct.causal_dot_product(q, k, v)
+    bwd = lambda: ct.causal_backward(q, k, v, do)
+
+    def both():
+        fwd()
+        bwd()
+    s = time_region(torch, both, steps, warmup)
+    tb = 16 * n * 128 * 2
+    out = {"N": n, "us": s * 1e6, "fwd_us": time_region(torch, fwd, steps, 2) * 1e6,
+           "bwd_us": time_region(torch, bwd, steps, 2) * 1e6, "tokens_per_s": n / s, "GBps": 11 * tb / s / 1e9,
+           "frac_hbm": 11 * tb / s / 1e9 / HBM_PEAK_GBS}
+    if kernels:
+        for name, fn in (("fwd_kernels_us", fwd), ("bwd_kernels_us", bwd)):
+            _loader.profile_enable(True)
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            _loader.profile_enable(False)
+            out[name] = {}
+            for kname in _loader.KERNEL_IDS:
+                ms, cnt = _loader.profile_read(kname)
+                if cnt:
+                    out[name][kname] = 1e3 * ms / steps
+    return out
+
+
 def gpt_block_step(torch, dev):
     """step(use_cache): forward + backward of one GPT attention block (B8 S2048 E1024 H16) under bf16 autocast.
     use_cache=True makes the module return the rotated keys, i.e. rotary and head permutes run as torch ops."""
@@ -264,17 +300,10 @@ def run_extras(torch, ct, dev):
     del S, qs, ks, vs
     # long context fwd+bwd, B=1 H=16 D=128 bf16, N sweep
     sweep = {}
-    for n in (4096, 16384, 65536):
-        q, k, v, do = make_inputs(torch, 1, 16, n, 128, 128, torch.bfloat16, dev)
-
-        def step():
-            ct.causal_dot_product(q, k, v)
-            ct.causal_backward(q, k, v, do)
-        s = time_region(torch, step, 20, 3)
-        byts = 11 * 16 * n * 128 * 2
-        sweep[str(n)] = {"us": s * 1e6, "tokens_per_s": n / s, "GBps": byts / s / 1e9,
-                         "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS}
-        del q, k, v, do
+    for n in (4096, 8192, 16384, 32768, 65536):
+        sweep[str(n)] = long_context(torch, ct, dev, n, 20, 3, kernels=(n == 65536))
+    rates = [x["tokens_per_s"] for x in sweep.values()]
+    sweep["tokens_per_s_min_over_max"] = min(rates) / max(rates)
     ex["long_context_fwd_bwd_B1_H16_D128"] = sweep
     # fp32 storage at the headline shape (what the backward of an autocast training step runs: the autograd
     # function saves the fp32 inputs, Cuda_Kernel/Custom_Kernel.py:16,38); fp32 MFMA, peak 157.3 TFLOP/s

@@ -30,8 +30,7 @@ def hipcc():
 
 def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    extra = os.environ.get("COTT_EXTRA_HIPCC_FLAGS", "").split()  # tuning experiments, e.g. -DCOTT_PF_SMALL=8
-    cmd = [hipcc()] + HIPCC_FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [hipcc()] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:

@@ -72,22 +72,26 @@ size_t elem_size(int dtype) {
     return 0;
 }
 
-int env_int(const char *name, int dflt) {
+// Tuning switches exist only in builds made with -DCOTT_EXPERIMENTS; the shipped library reads no environment.
+int exp_int(const char *name, int dflt) {
+#ifdef COTT_EXPERIMENTS
     const char *s = getenv(name);
-    if (!s || !*s) return dflt;
-    return atoi(s);
+    if (s && *s) return atoi(s);
+#else
+    (void)name;
+#endif
+    return dflt;
 }
 
 // Workgroups a launch aims for: one per CU of a 256-CU part (a second workgroup on a CU adds only ~20 %
 // throughput to these LDS-heavy kernels, so grids just above the CU count run almost twice as long).
-// COTT_TARGET_WGS overrides.
 int target_workgroups() {
-    static const int v = [] { const int x = env_int("COTT_TARGET_WGS", 0); return x > 0 ? x : 256; }();
+    static const int v = [] { const int x = exp_int("COTT_TARGET_WGS", 0); return x > 0 ? x : 256; }();
     return v;
 }
-// COTT_SPLIT: -1 auto (default), 0 never, 1 always split the output columns of each op in two.
+// -1 auto, 0 never, 1 always split the output columns of each op in two.
 int split_policy() {
-    static const int v = env_int("COTT_SPLIT", -1);
+    static const int v = exp_int("COTT_SPLIT", -1);
     return v;
 }
 
@@ -114,12 +118,12 @@ struct Op {
 struct SetPlan {
     int halves;           // 1, or 2 = every op split into two column halves (two problems)
     int nchunks, cpg, G;  // sequence cut: chunks of 64, chunks per group, groups per head
+    int sub;              // pieces per group in the group-state pass (one workgroup and one slot each)
     size_t ws_bytes;      // group-state slots
 };
 
-// COTT_PAIR=0 switches the paired dK/dV workgroups off (experiments).
 bool pair_enabled() {
-    static const bool v = env_int("COTT_PAIR", 1) != 0;
+    static const bool v = exp_int("COTT_PAIR", 1) != 0;
     return v;
 }
 
@@ -185,6 +189,7 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
     const size_t state = cott::mfma_state_floats(di, dj / p.halves) * sizeof(float);
     // the fp32 kernels stage the non-causal state through the workspace even for one group
     const bool slots = p.G > 1 || (!causal && dtype == COTT_F32);
+    p.sub = 1;
     p.ws_bytes = slots ? (size_t)nops * p.halves * BH * p.G * state : 0;
     return p;
 }
@@ -200,20 +205,78 @@ bool use_pair(const Op *ops, int n, long BH, int N, int dtype, bool causal) {
 
 int pad_key(const Op &o) { return cott::mfma_pad(o.di) * 1000 + cott::mfma_pad(o.dj); }
 
+// How one set of ops with equal padded head dims (members[0..cnt) of ops[0..n)) is run.
+struct SetLayout {
+    SetPlan p;
+    bool pair;        // dQ + (dK, dV) pair workgroups
+    bool complement;  // the ops that sum over the past run in complement form (see ProblemT)
+    int twin_of[8];   // >= 0: member whose state, transposed, is this member's state
+};
+
+SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH, int N, int dtype, bool causal) {
+    SetLayout L;
+    const Op &first = ops[members[0]];
+    const bool half = dtype == COTT_BF16 || dtype == COTT_F16;
+    L.pair = use_pair(ops, n, BH, N, dtype, causal);  // then all three ops are in this set
+    L.p = L.pair ? plan_set(BH, N, 2, first.di, first.dj, causal, dtype, true)
+                 : plan_set(BH, N, cnt, first.di, first.dj, causal, dtype);
+    const SetPlan &p = L.p;
+    // Gradient sets cut into sequence groups: the op that sums over the past (dQ) is put in complement form and
+    // walks the sequence from the end like the two that sum over the future, so the three workgroups of a head
+    // and group read the same tiles at the same time and the second and third reader find them in L2.
+    bool any_rev = false;
+    for (int c = 0; c < cnt; ++c) any_rev = any_rev || ops[members[c]].reversed;
+    L.complement = causal && !L.pair && p.G > 1 && cnt > 1 && any_rev && p.halves == 1 && half;
+    // ... and when two of them are X = G(.,B,C), Y = G(.,C,B) with square padded head dims (dK and dV), their
+    // states are transposes of each other: the group-state pass computes X's only.
+    for (int c = 0; c < 8; ++c) L.twin_of[c] = -1;
+    if (causal && !L.pair && p.G > 1 && p.halves == 1 && half && cott::mfma_pad(first.di) == cott::mfma_pad(first.dj))
+        for (int c = 1; c < cnt; ++c)
+            for (int e = 0; e < c && L.twin_of[c] < 0; ++e) {
+                const Op &x = ops[members[e]], &y = ops[members[c]];
+                if (L.twin_of[e] < 0 && x.B == y.C && x.C == y.B && x.reversed == y.reversed && x.di == y.dj &&
+                    x.dj == y.di && !x.sin && !x.sout && !y.sin && !y.sout && !x.lay[1] == !y.lay[2] &&
+                    !x.lay[2] == !y.lay[1])
+                    L.twin_of[c] = e;
+            }
+    // The group-state pass only streams two operands into MFMAs and two of its workgroups fit a CU: when its grid
+    // is well short of the chip, every group is cut into pieces (one workgroup and one slot each).
+    if (p.G > 1 && half) {
+        long wgs = 0;
+        if (L.pair)
+            wgs = 2L * (p.G - 1);
+        else
+            for (int c = 0; c < cnt; ++c) {
+                if (L.twin_of[c] >= 0) continue;
+                const bool comp = L.complement && !ops[members[c]].reversed && !ops[members[c]].sin && !ops[members[c]].sout;
+                wgs += (long)p.halves * (causal && !comp ? p.G - 1 : p.G);
+            }
+        wgs *= BH;
+        static const int force = exp_int("COTT_SUB", 0);
+        int sub = force > 0 ? force : (int)((288 + wgs / 2) / (wgs > 0 ? wgs : 1));
+        if (sub > 4) sub = 4;
+        while (sub > 1 && (p.cpg + sub - 1) / sub < 4) --sub;
+        if (sub > 1) {
+            L.p.sub = sub;
+            L.p.ws_bytes *= (size_t)sub;
+        }
+    }
+    return L;
+}
+
 // Workspace needed by run_ops for the same arguments.
 size_t ops_workspace(const Op *ops, int n, long BH, int N, int dtype, bool causal) {
     if (BH <= 0 || N <= 0) return 0;
     for (int i = 0; i < n; ++i)
         if (!use_mfma(dtype, ops[i].di, ops[i].dj, N)) return 0;
-    if (use_pair(ops, n, BH, N, dtype, causal)) return plan_set(BH, N, 2, ops[0].di, ops[0].dj, causal, dtype, true).ws_bytes;
     size_t total = 0;
     bool done[8] = {false};
     for (int i = 0; i < n; ++i) {
         if (done[i]) continue;
-        int cnt = 0;
+        int members[8], cnt = 0;
         for (int j = i; j < n; ++j)
-            if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; ++cnt; }
-        total += plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal, dtype).ws_bytes;
+            if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; members[cnt++] = j; }
+        total += layout_set(ops, n, members, cnt, BH, N, dtype, causal).p.ws_bytes;
     }
     return total;
 }
@@ -267,10 +330,23 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         int members[8], cnt = 0;
         for (int j = i; j < n; ++j)
             if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; members[cnt++] = j; }
-        const bool pair = use_pair(ops, n, BH, N, dtype, causal);  // then all three ops are in this set
-        const SetPlan p = pair ? plan_set(BH, N, 2, ops[i].di, ops[i].dj, causal, dtype, true)
-                               : plan_set(BH, N, cnt, ops[i].di, ops[i].dj, causal, dtype);
+        const SetLayout L = layout_set(ops, n, members, cnt, BH, N, dtype, causal);
+        const SetPlan &p = L.p;
+        const bool pair = L.pair, complement = L.complement;
+        const int *twin_of = L.twin_of;
         a.pair = pair ? 1 : 0;
+        // Non-temporal loads: tensors several times the last-level cache, and no operand read by two problems
+        static const long stream_min_bytes = (long)exp_int("COTT_STREAM_MIN_MB", 128) << 20;
+        const bool big = (long)BH * N * (ops[i].di > ops[i].dj ? ops[i].di : ops[i].dj) * (long)esz >= stream_min_bytes;
+        a.stream_scan = causal && big && cnt == 1 && p.halves == 1 && (dtype == COTT_BF16 || dtype == COTT_F16);
+        bool distinct = causal && p.halves == 1 && (dtype == COTT_BF16 || dtype == COTT_F16);
+        for (int c = 0; c < cnt && distinct; ++c)
+            for (int e = 0; e < c; ++e) {
+                if (twin_of[c] >= 0 || twin_of[e] >= 0) continue;  // skipped by the group-state pass
+                const Op &x = ops[members[e]], &y = ops[members[c]];
+                if (x.B == y.B || x.B == y.C || x.C == y.B || x.C == y.C) distinct = false;
+            }
+        a.stream_state = distinct && big;
         for (int c = 0; c < cnt; ++c) {
             const Op &o = ops[members[c]];
             const int djh = o.dj / p.halves;
@@ -284,6 +360,8 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
                 d.dj = djh;
                 d.ldc = o.dj;
                 d.reversed = o.reversed;
+                d.comp = (complement && !o.reversed && !o.sin && !o.sout) ? 1 : 0;
+                d.seed_from = twin_of[c];  // (halves == 1 here: set index == member index)
                 const size_t ssz = dtype == COTT_F64 ? 8 : 4;
                 d.sin = o.sin ? static_cast<const char *>(o.sin) + (size_t)h * djh * ssz : nullptr;
                 d.sout = o.sout ? static_cast<char *>(o.sout) + (size_t)h * djh * ssz : nullptr;
@@ -295,7 +373,7 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         a.ws = p.ws_bytes ? reinterpret_cast<float *>(ws_cursor) : nullptr;
         ws_cursor += p.ws_bytes;
         a.BH = (int)BH; a.N = N;
-        a.nchunks = p.nchunks; a.cpg = p.cpg; a.G = p.G;
+        a.nchunks = p.nchunks; a.cpg = p.cpg; a.G = p.G; a.sub = p.sub;
         a.scan_prof_id = n > 1 ? cott::K_SCAN_GRAD : cott::K_SCAN;
         a.stream = stream;
         hipError_t e;

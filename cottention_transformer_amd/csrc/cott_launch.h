@@ -20,6 +20,11 @@ struct OpDesc {
     // of a position next to each other, as the projections of a transformer block produce and consume them.
     unsigned char lay[4] = {0, 0, 0, 0};
     int H = 1;  // heads per batch element; needed when any layout flag is set
+    // Complement form (16-bit causal MFMA kernels, sets with sequence groups only): the op is walked against its
+    // own direction so that it reads the same tiles at the same time as the other ops of its set.
+    int comp = 0;
+    // >= 0: index (within the set) of the op whose state, transposed, is this op's state (see ProblemT::seed_from)
+    int seed_from = -1;
 };
 
 // A set of ops launched together over the same (BH, N); MFMA path: all share padded head dims.
@@ -29,11 +34,15 @@ struct SetArgs {
     float *ws;            // count * BH * G * state_floats floats of group-state slots, or null when unused
     int BH, N;
     int nchunks, cpg, G;  // chunks of 64, chunks per group, groups per head
+    int sub = 1;          // pieces per group in the group-state pass (ws holds G * sub slots per head and problem)
     int scan_prof_id;     // K_SCAN for a forward launch, K_SCAN_GRAD for the three-gradient launch
     // pair > 0: op[pair] and op[pair + 1] are X = G(A,B,C) and Y = G(A2,C,B) with the same direction and square
     // padded head dims; one workgroup serves both (scan_pair_kernel).  The launch then has count - 1 problems
     // per head and the workspace count - 1 state slots per group.  pair must be count - 2.
     int pair = 0;
+    // non-temporal loads in the group-state pass / in the scan: for tensors far larger than the caches, when no
+    // two problems of the set read the same operand
+    bool stream_state = false, stream_scan = false;
     hipStream_t stream;
 };
 

@@ -36,6 +36,18 @@ struct ProblemT {
     const float *sin;
     float *sout;
     int di, dj, ldc, reversed, lds;
+    // reversed: the order in which the chunks are WALKED (1 = from the end of the sequence).  mask_rev: the side of
+    // the diagonal the op sums over (0: positions <= s, 1: positions >= s).  They differ for an op in complement
+    // form (comp = 1), which walks against its own direction: its state starts from the sum over everything the op
+    // has to see at the first chunk walked and is DEcreased chunk by chunk, so the state at a chunk still includes
+    // that chunk, and the score products take the other side of the diagonal with a minus sign:
+    //     out_c = A_c S_incl - ((A_c B_c^T) o (1 - mask)) C_c ,   S_incl <- S_incl - B_c^T C_c .
+    // This lets an op that sums over the past share every tile it reads with ops that sum over the future.
+    int mask_rev, comp;
+    // seed_from >= 0: this op's state is the TRANSPOSE of the state of problem `seed_from` of the same set (its B
+    // and C are that problem's C and B, same walking order, square padded head dims): the group-state pass skips
+    // it and its scan reads the other problem's slots transposed.
+    int seed_from;
     // Row strides of A, B and O in elements (C's is ldc) and, for each operand, where a head
     // starts: head bh is at (bh / H) * bs + (bh % H) * hs elements.  (BH,N,w) tensors have ld = w, hs = N * w,
     // bs = H * hs; (B,N,H,w) tensors, whose heads are interleaved inside a position, ld = H * w, hs = w,
@@ -51,6 +63,9 @@ template <class E>
 struct ProblemSetT {
     ProblemT<E> p[kMaxProblems];
     int count;
+    // 16-bit kernels: the group-state pass cuts every group of the scan into `sub` pieces, one workgroup and one
+    // slot each (slot (bh * G + grp) * sub + piece); the prefix pass leaves the scan's seed in the first of them
+    int sub;
 };
 typedef ProblemT<u16> Problem;  // 16-bit storage (bf16 / fp16)
 typedef ProblemSetT<u16> ProblemSet;
@@ -101,14 +116,14 @@ inline unsigned grid_for(int BH, int nprob, int G) {
 // [64][D] tile, global -> registers, through a buffer descriptor of the head.  Thread t of NT owns 16-byte
 // vectors t, t+NT, ...; rows past N read as zero (hardware range check).  Pure loads, no use of the
 // result here, so nothing waits on them until the tile is staged.
-template <int D, int NT = kThreads>
+template <int D, int NT = kThreads, bool STREAM = false>
 __device__ __forceinline__ void load_tile(u32x4 *r, rsrc_t rs, int row0, int ld, int tid) {
 #pragma unroll
     for (int u = 0; u < 8 * D / NT; ++u) {
         const int v = tid + NT * u;
         const int row = row0 + v / (D / 8);
         const int col = (v % (D / 8)) * 8;
-        r[u] = buf_load16(rs, (uint32_t)(row * ld + col) * 2u);
+        r[u] = buf_load16<STREAM>(rs, (uint32_t)(row * ld + col) * 2u);
     }
 }
 
@@ -128,8 +143,10 @@ __device__ __forceinline__ void store_tile(u16 *tile, const u32x4 *r, int d, int
 // (tile index t = w*TPW + u -> (t / NJT, t % NJT)).  Both operands are column fragments of the
 // row-major LDS tiles, fetched with transposing reads; all fragments of a 32-token step are read
 // before its MFMAs so the LDS latency is paid once per step, not once per tile.
+// `flip`: 0, or 0x80008000 to subtract the product instead (sign bits of the B fragments).
 template <class TR, int DI, int DJ>
-__device__ __forceinline__ void state_update(f32x4 *S, const u16 *sB, const u16 *sC, int w, int g, int m) {
+__device__ __forceinline__ void state_update(f32x4 *S, const u16 *sB, const u16 *sC, int w, int g, int m,
+                                             uint32_t flip = 0u) {
     using TL = Tiling<DI, DJ>;
     constexpr int ROWS = (TL::TPW + TL::NJT - 1) / TL::NJT;       // tile rows (values of `it`) per wavefront
     constexpr int COLS = TL::TPW < TL::NJT ? TL::TPW : TL::NJT;   // distinct `jt` per wavefront
@@ -141,6 +158,7 @@ __device__ __forceinline__ void state_update(f32x4 *S, const u16 *sB, const u16 
         for (int r = 0; r < ROWS; ++r) {
             const int it = (w * TL::TPW + r * TL::NJT) / TL::NJT;
             a[r] = cat(lds_col4(sB, TL::BS, k0, 16 * it, m), lds_col4(sB, TL::BS, k0 + 4, 16 * it, m));
+            a[r] ^= u32x4{flip, flip, flip, flip};
         }
 #pragma unroll
         for (int c = 0; c < COLS; ++c) {
@@ -199,42 +217,54 @@ __device__ __forceinline__ void chunk_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// Sum of B^T C over each group of chunks, written in register-native order:
-// float4 index (w*TPW + u)*64 + lane of slot (bh*G + grp).  `ngroups` of the G groups are launched
-// (the causal scan never needs the last group's sum).
-template <class TR, int DI, int DJ, int PF>
+// Sum of B^T C over each piece of each group of chunks, written in register-native order:
+// float4 index (w*TPW + u)*64 + lane of slot (bh*G + grp)*sub + piece.  `ngroups` of the G groups are launched
+// (the causal scan never needs the last group's sum, except for ops in complement form; all_groups: the non-causal
+// form, which needs every group of every op).
+template <class TR, int DI, int DJ, int PF, bool STREAM>
 __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg,
-                                                               int G, int ngroups) {
+                                                               int G, int ngroups, int all_groups) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS;
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, ngroups);
+    const int sub = set.sub;
+    const WorkItem wi = decode_workgroup(set.count, ngroups * sub);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
+    const int grp = wi.grp / sub, piece = wi.grp % sub;
+    // `ngroups` == G is launched when some op of the set is in complement form; the others skip their last group
+    if (grp == G - 1 && ngroups == G && !pr.comp && !all_groups) return;
+    if (pr.seed_from >= 0) return;
     const int di = pr.di, dj = pr.dj, ldb = pr.ldb, ldc = pr.ldc, reversed = pr.reversed;
     const rsrc_t rB = make_rsrc(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), ((uint32_t)(N - 1) * ldb + di) * 2u);
     const rsrc_t rC = make_rsrc(pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), ((uint32_t)(N - 1) * ldc + dj) * 2u);
-    const int p0 = wi.grp * cpg;
-    const int p1 = min(p0 + cpg, nchunks);
+    const int cps = (cpg + sub - 1) / sub;  // chunks per piece
+    const int p0 = grp * cpg + piece * cps;
+    const int p1 = min(p0 + cps, min((grp + 1) * cpg, nchunks));
 
     f32x4 S[TL::TPW];
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 *slot = reinterpret_cast<f32x4 *>(pr.gstate + ((size_t)wi.bh * G * sub + wi.grp) * TL::STATE_FLOATS);
+    if (p1 <= p0) {  // a piece past the end of its group: its slot is zero
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) slot[(w * TL::TPW + u) * 64 + l] = S[u];
+        return;
+    }
 
     u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
     auto load_chunk = [&](int s, int p) {
         const int pc = min(p, p1 - 1);
         const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
-        load_tile<DI>(rb[s], rB, row0, ldb, tid);
-        load_tile<DJ>(rc[s], rC, row0, ldc, tid);
+        load_tile<DI, kThreads, STREAM>(rb[s], rB, row0, ldb, tid);
+        load_tile<DJ, kThreads, STREAM>(rc[s], rC, row0, ldc, tid);
     };
     auto finish = [&]() {
-        f32x4 *out = reinterpret_cast<f32x4 *>(pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS);
 #pragma unroll
-        for (int u = 0; u < TL::TPW; ++u) out[(w * TL::TPW + u) * 64 + l] = S[u];
+        for (int u = 0; u < TL::TPW; ++u) slot[(w * TL::TPW + u) * 64 + l] = S[u];
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
@@ -254,26 +284,51 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     finish();
 }
 
-// Over the G slots of one head, element-wise: mode 0 -> exclusive prefix in place (slot g gets the
-// sum of slots < g; only the first `ncomputed` slots hold data), mode 1 -> total into slot 0.
+// Over the G * sub slots of one head, element-wise.  mode 0: the first slot of group g gets the sum of all slots of
+// the groups before g (only the first `ncomputed` groups hold data), or, for an op in complement form (all groups
+// hold data), the total minus that sum.  mode 1: total into slot 0.  Slots are read in batches of independent
+// loads and only written after they have been read.
 template <class E>
-__global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSetT<E> set, int BH, int G, int ncomputed,
+__global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSetT<E> set, int BH, int G, int sub, int ncomputed,
                                                                 int state_floats, int mode) {
+    constexpr int BATCH = 8;
     const int sf4 = state_floats / 4;
     const int blocks_per_state = (sf4 + kThreads - 1) / kThreads;
     const int e = (blockIdx.x % blocks_per_state) * kThreads + threadIdx.x;
     const int rest = blockIdx.x / blocks_per_state;
     const int prob = rest % set.count, bh = rest / set.count;
-    if (e >= sf4 || bh >= BH) return;
-    f32x4 *p = reinterpret_cast<f32x4 *>(set.p[prob].gstate + (size_t)bh * G * state_floats) + e;
-    f32x4 run = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < G; ++s) {
-        f32x4 t = {0.f, 0.f, 0.f, 0.f};
-        if (s < ncomputed) t = p[(size_t)s * sf4];
-        if (mode == 0) p[(size_t)s * sf4] = run;
-        run += t;
+    if (e >= sf4 || bh >= BH || set.p[prob].seed_from >= 0) return;
+    const int nslots = G * sub;
+    const bool comp = mode == 0 && set.p[prob].comp;
+    const int nread = (mode == 1 || comp) ? nslots : ncomputed * sub;
+    f32x4 *p = reinterpret_cast<f32x4 *>(set.p[prob].gstate + (size_t)bh * nslots * state_floats) + e;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    f32x4 total = zero;
+    if (mode == 1 || comp) {
+        for (int s0 = 0; s0 < nslots; s0 += BATCH) {
+            f32x4 t[BATCH];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) t[u] = (s0 + u < nslots) ? p[(size_t)(s0 + u) * sf4] : zero;
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) total += t[u];
+        }
+        if (mode == 1) {
+            p[0] = total;
+            return;
+        }
     }
-    if (mode == 1) p[0] = run;
+    f32x4 run = zero;
+    for (int s0 = 0; s0 < nslots; s0 += BATCH) {
+        f32x4 t[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) t[u] = (s0 + u < nread) ? p[(size_t)(s0 + u) * sf4] : zero;
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const int s = s0 + u;
+            if (s < nslots && s % sub == 0) p[(size_t)s * sf4] = comp ? total - run : run;
+            run += t[u];
+        }
+    }
 }
 
 // ---- the chunk recurrence --------------------------------------------------------------------------
@@ -294,7 +349,8 @@ __global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSetT<E> s
 
 // Position of a workgroup in the scan: chunks [p0, p1) in scan order of `nchunks`.
 struct ScanRange {
-    int N, nchunks, p0, p1, reversed;
+    int N, nchunks, p0, p1, reversed;  // reversed: walking order
+    int mask_rev, comp;                // see ProblemT
 };
 
 // Loader role: LT threads stage the B tile (rows of di) and the C tile (dj columns of rows of ldc).
@@ -307,7 +363,7 @@ struct StagedOut {
     const u16 *sO;  // [2 buffers][2 tiles][64 * OS]
 };
 
-template <int DI, int DJ, int PF, int LT>
+template <int DI, int DJ, int PF, int LT, bool STREAM = false>
 __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head, int di, int dj, int ldb, int ldc,
                                             const ScanRange &r, int tid, u16 *sB, u16 *sC,
                                             const StagedOut *so = nullptr) {
@@ -337,8 +393,8 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
     auto load_chunk = [&](int s, int p) {
         const int pc = min(p, r.p1 - 1);
         const int row0 = (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
-        load_tile<DI, LT>(rb[s], rB, row0, ldb, tid);
-        load_tile<DJ, LT>(rc[s], rC, row0, ldc, tid);
+        load_tile<DI, LT, STREAM>(rb[s], rB, row0, ldb, tid);
+        load_tile<DJ, LT, STREAM>(rc[s], rC, row0, ldc, tid);
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_chunk(s, r.p0 + s);
@@ -364,7 +420,7 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
 // [j][i] for the A_blk S product.  TWIN: also publish the copy of the TRANSPOSED state (which is
 // [i][j] of this one) in sS2, for a second problem whose B and C are this problem's C and B.
 template <class TR, int DI, int DJ, bool TWIN>
-__device__ __forceinline__ void state_role(const float *seed, const float *sin, float *sout, int lds, bool last_group,
+__device__ __forceinline__ void state_role(const float *seed, bool seed_transposed, const float *sin, float *sout, int lds, bool last_group,
                                            int di, int dj, const ScanRange &r, int w, int l, const u16 *sB,
                                            const u16 *sC, u16 *sS, u16 *sS2) {
     using TL = Tiling<DI, DJ>;
@@ -373,10 +429,24 @@ __device__ __forceinline__ void state_role(const float *seed, const float *sin, 
     f32x4 S[TL::TPW];
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (seed != nullptr) {
+    if (seed != nullptr && !seed_transposed) {
         const f32x4 *gs = reinterpret_cast<const f32x4 *>(seed);
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
+    }
+    if constexpr (DI == DJ) {
+        if (seed != nullptr && seed_transposed) {
+            // element [16it + 4g + q][16jt + m] of this state is element [16jt + m][16it + 4g + q] of the other one:
+            // its tile (jt, it), lane (m' = 4g + q, g' = m / 4), component m % 4
+#pragma unroll
+            for (int u = 0; u < TL::TPW; ++u) {
+                const int t = w * TL::TPW + u;
+                const int it = t / TL::NJT, jt = t % TL::NJT;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    S[u][q] = seed[((size_t)(jt * TL::NJT + it) * 64 + ((m >> 2) * 16 + 4 * g + q)) * 4 + (m & 3)];
+            }
+        }
     }
     // accumulator element r of tile (it, jt) is S[16it + 4g + r][16jt + m]
     if (sin != nullptr) {
@@ -408,7 +478,7 @@ __device__ __forceinline__ void state_role(const float *seed, const float *sin, 
     __syncthreads();
     for (int p = r.p0; p < r.p1; ++p) {
         const int buf = (p - r.p0) & 1;
-        state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
+        state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m, r.comp ? 0x80008000u : 0u);
         put_state(sS + (buf ^ 1) * SSZ, sS2 + (buf ^ 1) * SSZ);
         __syncthreads();
     }
@@ -431,7 +501,7 @@ __device__ __forceinline__ void state_role(const float *seed, const float *sin, 
 // sOt: null = store the outputs to memory from here; else the [2 buffers] of this problem's staged output tile
 // (buffer stride 2 * 64 * OS), written with 8-byte LDS stores and sent to memory by the loader wavefronts, so that
 // this wavefront's chain of LDS reads and MFMAs never waits for the vector-memory pipeline to take a store.
-template <class TR, int DI, int DJ, int PF, int IB>
+template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false>
 __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int lda, int ldc,
                                             const ScanRange &r, int blk0, int l, const u16 *sB, const u16 *sC,
                                             const u16 *sS, u16 *sOt = nullptr) {
@@ -441,6 +511,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
     const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     const int reversed = r.reversed;
+    const bool mask_rev = r.mask_rev != 0, comp = r.comp != 0;
     u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
     auto load_q = [&](int s, int p) {
         const int pc = min(p, r.p1 - 1);
@@ -449,7 +520,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
         for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
             for (int ks = 0; ks < TL::KS; ++ks)
-                qn[s][ib][ks] = buf_load16(rA, (uint32_t)((row + 16 * ib) * lda + 32 * ks + 8 * g) * 2u);
+                qn[s][ib][ks] = buf_load16<STREAM>(rA, (uint32_t)((row + 16 * ib) * lda + 32 * ks + 8 * g) * 2u);
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_q(s, r.p0 + s);
@@ -510,8 +581,8 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                         const int d0 = 16 * (jt - (blk0 + ib)) + 4 * g - m;  // key pos - query pos at element 0
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
-                            const bool keep = reversed ? (d0 + q >= 0) : (d0 + q <= 0);
-                            acc[q] = keep ? acc[q] : 0.f;
+                            const bool keep = mask_rev ? (d0 + q >= 0) : (d0 + q <= 0);
+                            acc[q] = (keep != comp) ? (comp ? -acc[q] : acc[q]) : 0.f;
                         }
                         pk[ib][jt] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
                     }
@@ -564,7 +635,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 }
 
 // One problem per workgroup: OW output wavefronts (IB = 4/OW blocks each), 4 state, LW loader.
-template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false>
+template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false, bool STREAM = false>
 __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set, int BH, int N, int nchunks,
                                                                   int cpg, int G) {
     using TL = Tiling<DI, DJ>;
@@ -592,6 +663,8 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     r.p0 = wi.grp * cpg;
     r.p1 = min(r.p0 + cpg, nchunks);
     r.reversed = pr.reversed;
+    r.mask_rev = pr.mask_rev;
+    r.comp = pr.comp;
     if (wv >= OW + 4) {
         StagedOut so;
         so.O[0] = pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh);
@@ -601,17 +674,18 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
         so.dj[1] = 0;
         so.ld[1] = 0;
         so.sO = sO;
-        loader_role<DI, DJ, PF, LT>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
-                                    di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC, STAGED ? &so : nullptr);
+        loader_role<DI, DJ, PF, LT, STREAM>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
+                                            di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC, STAGED ? &so : nullptr);
     } else if (wv >= OW) {
+        const float *slots = pr.seed_from >= 0 ? set.p[pr.seed_from].gstate : pr.gstate;
         state_role<TR, DI, DJ, false>(
-            pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr,
+            slots ? slots + ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS : nullptr, pr.seed_from >= 0,
             pr.sin ? pr.sin + (size_t)wi.bh * di * pr.lds : nullptr, pr.sout ? pr.sout + (size_t)wi.bh * di * pr.lds : nullptr,
             pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS, nullptr);
     } else {
-        output_role<TR, DI, DJ, PF, IB>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
-                                        pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r, IB * wv, l,
-                                        sB, sC, sS, STAGED ? sO : nullptr);
+        output_role<TR, DI, DJ, PF, IB, STREAM>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
+                                                pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r,
+                                                IB * wv, l, sB, sC, sS, STAGED ? sO : nullptr);
     }
 }
 
@@ -653,7 +727,9 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     r.p0 = wi.grp * cpg;
     r.p1 = min(r.p0 + cpg, nchunks);
     r.reversed = pr.reversed;
-    const float *seed = pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS : nullptr;
+    r.mask_rev = pr.mask_rev;
+    r.comp = 0;  // (the pair workgroups never run in complement form)
+    const float *seed = pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS : nullptr;
     if (wv >= NOUT + 4) {
         StagedOut so;
         so.O[0] = pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh);
@@ -667,9 +743,9 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
                                   di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (NOUT + 4), sB, sC, &so);
     } else if (wv >= NOUT) {
         if (pair)
-            state_role<TR, D, D, true>(seed, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, sS2);
+            state_role<TR, D, D, true>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, sS2);
         else
-            state_role<TR, D, D, false>(seed, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, nullptr);
+            state_role<TR, D, D, false>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, nullptr);
     } else if (!pair) {
         if (wv < 4) {
             output_role<TR, D, D, PF, 1>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r,
@@ -705,7 +781,7 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
     const int p0 = wi.grp * cpg;
     const int p1 = min(p0 + cpg, nchunks);
     {
-        const f32x4 *gs = reinterpret_cast<const f32x4 *>(pr.gstate + (size_t)wi.bh * G * TL::STATE_FLOATS);
+        const f32x4 *gs = reinterpret_cast<const f32x4 *>(pr.gstate + (size_t)wi.bh * G * set.sub * TL::STATE_FLOATS);
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) {
             const f32x4 sv = gs[(w * TL::TPW + u) * 64 + l];

@@ -18,7 +18,7 @@ hipError_t run_causal_f32(const SetArgs &a) {
         const int bps = (TL::STATE_FLOATS / 4 + kThreads - 1) / kThreads;
         ProfScope prof(K_STATE_PREFIX, a.stream);
         state_prefix_kernel<float><<<dim3((unsigned)(a.BH * a.count * bps)), dim3(kThreads), 0, a.stream>>>(
-            ps, a.BH, a.G, a.G - 1, TL::STATE_FLOATS, 0);
+            ps, a.BH, a.G, 1, a.G - 1, TL::STATE_FLOATS, 0);
     }
     ProfScope prof(a.scan_prof_id, a.stream);
     scan_f32_kernel<DI, DJ, false><<<dim3(grid_for(a.BH, a.count, a.G)), dim3(kThreads), 0, a.stream>>>(
@@ -40,7 +40,7 @@ hipError_t run_noncausal_f32(const SetArgs &a) {
         const int bps = (TL::STATE_FLOATS / 4 + kThreads - 1) / kThreads;
         ProfScope prof(K_STATE_PREFIX, a.stream);
         state_prefix_kernel<float><<<dim3((unsigned)(a.BH * a.count * bps)), dim3(kThreads), 0, a.stream>>>(
-            ps, a.BH, a.G, a.G, TL::STATE_FLOATS, 1);
+            ps, a.BH, a.G, 1, a.G, TL::STATE_FLOATS, 1);
     }
     ProfScope prof(K_APPLY, a.stream);
     scan_f32_kernel<DI, DJ, true><<<dim3(grid_for(a.BH, a.count, a.G)), dim3(kThreads), 0, a.stream>>>(
