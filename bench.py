@@ -80,9 +80,20 @@ def cpu_baseline(torch):
         tf.causal_cumsum(qa, ka, va).backward(g)
         times.append(time.perf_counter() - t0)
     t = statistics.median(times[1:])
+    # the reference's own CPU-runnable configuration, (1,2,128,64) fp32, same formulation
+    q1, k1, v1, g1 = tf.synthetic_inputs((1, 2, 128, 64), seed=0, dtype=torch.float32)
+    t1s = []
+    for it in range(23):
+        qa, ka, va = (x.clone().requires_grad_(True) for x in (q1, k1, v1))
+        t0 = time.perf_counter()
+        tf.causal_cumsum(qa, ka, va).backward(g1)
+        t1s.append(time.perf_counter() - t0)
+    t1 = statistics.median(t1s[3:])
     return {"value": b * n / t, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"(B,H,N,D)=({b},{h},{n},{d}) fp32: 1 of the 8 batch elements of the headline shape, torch cumsum "
-                      f"form fwd + autograd bwd, median of 24 passes after 1 warm-up; {t:.2f} s per pass"}
+                      f"form fwd + autograd bwd, median of 24 passes after 1 warm-up; {t:.2f} s per pass",
+            "cfg1_B1_H2_N128_D64_fp32": {"value": 128 / t1, "unit": "tokens/s", "ms_per_pass": t1 * 1e3,
+                                         "sample": "median of 20 passes after 3 warm-ups"}}
 
 
 def main():
@@ -155,10 +166,19 @@ def main():
     passes = {"scan": 4, "scan_grad": 7, "group_state": 2}
     alg_bytes = passes.get(dominant, 4) * tensor_bytes
     achieved = alg_bytes / (kern[dominant]["avg_us"] * 1e-6) / 1e9
+    # the same kernels with cold caches: what a training step sees (other kernels run between forward and backward)
+    cold = cold_cache_kernel_times(torch, ct, dev, q, k, v, do)
+    cold_dom = cold["bwd_kernel_us"] if dominant == "scan_grad" else cold["fwd_kernel_us"]
+    cold_step_us = cold["fwd_kernel_us"] + cold["bwd_kernel_us"]
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
                 "kernel": dominant, "avg_us": kern[dominant]["avg_us"],
                 "algorithmic_bytes_per_launch": alg_bytes,
+                "cold_avg_us": cold_dom, "cold_achieved": alg_bytes / (cold_dom * 1e-6) / 1e9,
+                "cold_frac": alg_bytes / (cold_dom * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                "cold_whole_step": {"fwd_kernel_us": cold["fwd_kernel_us"], "bwd_kernel_us": cold["bwd_kernel_us"],
+                                    "tokens_per_s": B * N / (cold_step_us * 1e-6),
+                                    "frac_hbm": 11 * tensor_bytes / (cold_step_us * 1e-6) / 1e9 / HBM_PEAK_GBS},
                 "whole_step": {"algorithmic_bytes": 11 * tensor_bytes,
                                "achieved_GBps": 11 * tensor_bytes / sec / 1e9,
                                "frac_hbm": 11 * tensor_bytes / sec / 1e9 / HBM_PEAK_GBS,
@@ -166,8 +186,8 @@ def main():
                                "frac_mfma_bf16": 14.0 * B * H * N * D * D / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS}}
 
     extras = {"fwd_us": sec_f * 1e6, "bwd_us": sec_b * 1e6, "kernels": kern}
+    extras["cold_cache_headline"] = cold
     if not args.no_extras:
-        extras["cold_cache_headline"] = cold_cache_kernel_times(torch, ct, dev, q, k, v, do)
         extras.update(run_extras(torch, ct, dev))
 
     out = {
@@ -185,27 +205,28 @@ def main():
     print(json.dumps(out))
 
 
-def cold_cache_kernel_times(torch, ct, dev, q, k, v, do):
-    """Kernel durations at the headline shape when nothing is left in L2 or the 256 MB last-level cache from the
-    previous call (a read of 1 GiB of other data runs before every launch; a read, so that no dirty lines of the
-    evicting kernel are written back during the measurement), which is how a training step meets these kernels.
-    The step loop above re-uses its 256 MiB of tensors every iteration and so is served partly from that cache."""
+def cold_kernel_us(torch, fn, kernel, big):
+    """Average duration of one kernel family when nothing is left in L2 or the 256 MB last-level cache from the
+    previous call (a read of 1 GiB of other data, `big`, runs before every launch; a read, so that no dirty lines of
+    the evicting kernel are written back during the measurement), which is how a training step meets these kernels.
+    A loop over the same tensors is served partly from that cache."""
     from cottention_transformer_amd import _loader
-    big = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
-
-    def run(fn, kernel):
+    fn()
+    torch.cuda.synchronize()
+    _loader.profile_enable(True)
+    for _ in range(20):
+        big.sum()
         fn()
-        torch.cuda.synchronize()
-        _loader.profile_enable(True)
-        for _ in range(20):
-            big.sum()
-            fn()
-        torch.cuda.synchronize()
-        _loader.profile_enable(False)
-        ms, n = _loader.profile_read(kernel)
-        return 1e3 * ms / n
-    out = {"fwd_kernel_us": run(lambda: ct.causal_dot_product(q, k, v), "scan"),
-           "bwd_kernel_us": run(lambda: ct.causal_backward(q, k, v, do), "scan_grad")}
+    torch.cuda.synchronize()
+    _loader.profile_enable(False)
+    ms, n = _loader.profile_read(kernel)
+    return 1e3 * ms / n
+
+
+def cold_cache_kernel_times(torch, ct, dev, q, k, v, do):
+    big = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
+    out = {"fwd_kernel_us": cold_kernel_us(torch, lambda: ct.causal_dot_product(q, k, v), "scan", big),
+           "bwd_kernel_us": cold_kernel_us(torch, lambda: ct.causal_backward(q, k, v, do), "scan_grad", big)}
     del big
     return out
 
@@ -259,6 +280,44 @@ def gpt_block_step(torch, dev):
     return step
 
 
+def module_anchor(torch, dev):
+    """Forward latency of the two attention modules at batch 1, hidden 2048, 16 heads (D = 128), the one point the
+    reference publishes for this path: its module-level plots (tests/MemoryTest.py:118-143, 233-278: eval mode, fp32,
+    no autocast, time.time() without device synchronisation, GPU not stated) read about 13 ms (Cos-GPT) and 11 ms
+    (Cos-BERT) at S = 16384.  Here: synchronised, median of 10 after 3 warm-ups, fp32 as there and under bf16
+    autocast."""
+    from types import SimpleNamespace
+    from cottention_transformer_amd import modules
+    gpt = modules.GPTCosAttention(SimpleNamespace(max_position_embeddings=16384, attn_pdrop=0.0, resid_pdrop=0.0,
+                                                  hidden_size=2048, num_attention_heads=16, rotary_dim=64)).to(dev).eval()
+    bert = modules.BertCosAttention(SimpleNamespace(hidden_size=2048, num_attention_heads=16,
+                                                    attention_probs_dropout_prob=0.0)).to(dev).eval()
+    out = {"reference_plot_readoff_ms_at_S16384": {"cos_gpt": 13.0, "cos_bert": 11.0, "hardware": "unstated GPU"}}
+
+    def lat(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(10):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        return statistics.median(ts) * 1e3
+
+    with torch.no_grad():
+        for s_len in (1024, 2048, 4096, 8192, 16384):
+            x = torch.randn(1, s_len, 2048, device=dev)
+            row = {"cos_gpt_fp32_ms": lat(lambda: gpt(x)), "cos_bert_fp32_ms": lat(lambda: bert(x))}
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                row["cos_gpt_bf16_autocast_ms"] = lat(lambda: gpt(x))
+                row["cos_bert_bf16_autocast_ms"] = lat(lambda: bert(x))
+            out[f"S{s_len}"] = row
+            del x
+    return out
+
+
 def run_extras(torch, ct, dev):
     """Secondary configurations of the same path (not the headline value)."""
     ex = {}
@@ -274,7 +333,14 @@ def run_extras(torch, ct, dev):
     byts = 7 * b * h * n * d * 2
     ex["noncausal_bwd_B32_H12_N512_D64"] = {"us": s * 1e6, "tokens_per_s": b * n / s, "GBps": byts / s / 1e9,
                                             "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS}
-    del q, k, v, do
+    big = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
+    cf = cold_kernel_us(torch, lambda: ct.noncausal_dot_product(q, k, v), "apply", big)
+    cb = cold_kernel_us(torch, lambda: ct.noncausal_backward(q, k, v, do), "apply", big)
+    tb = b * h * n * d * 2
+    ex["noncausal_cold_cache_B32_H12_N512_D64"] = {
+        "fwd_kernel_us": cf, "fwd_frac_hbm": 4 * tb / (cf * 1e-6) / 1e9 / HBM_PEAK_GBS, "fwd_tokens_per_s": b * n / (cf * 1e-6),
+        "bwd_kernel_us": cb, "bwd_frac_hbm": 7 * tb / (cb * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    del q, k, v, do, big
     # recurrent decode, state (256,16,128,128) fp32, 512 consecutive steps with fresh q,k,v per step
     b, h, d, steps = 256, 16, 128, 512
     g = torch.Generator(device=dev).manual_seed(0)
@@ -298,6 +364,26 @@ def run_extras(torch, ct, dev):
                                            "note": "state is 256 MiB = the size of the last-level cache; "
                                                    "GB/s is algorithmic bytes / time"}
     del S, qs, ks, vs
+    # the same step on a state four times the last-level cache (B=1024: 1 GiB), where every byte comes from memory
+    b, steps = 1024, 64
+    S = (0.01 * torch.randn(b, h, d, d, generator=g, device=dev, dtype=torch.float32)).contiguous()
+    qs = torch.nn.functional.normalize(torch.randn(8, b, h, d, generator=g, device=dev), dim=-1).to(torch.bfloat16)
+    ks = torch.nn.functional.normalize(torch.randn(8, b, h, d, generator=g, device=dev), dim=-1).to(torch.bfloat16)
+    vs = torch.randn(8, b, h, d, generator=g, device=dev).to(torch.bfloat16)
+    out = torch.empty(b, h, d, dtype=torch.bfloat16, device=dev)
+    for t in range(4):
+        ct.decode_step(S, qs[t], ks[t], vs[t], out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(steps):
+        ct.decode_step(S, qs[t % 8], ks[t % 8], vs[t % 8], out=out)
+    torch.cuda.synchronize()
+    s = time.perf_counter() - t0
+    byts = steps * (2 * b * h * d * d * 4 + 4 * b * h * d * 2)
+    ex["decode_B1024_H16_D128_state_1GiB"] = {"us_per_step": s / steps * 1e6, "tokens_per_s": b * steps / s,
+                                              "GBps": byts / s / 1e9, "frac_hbm": byts / s / 1e9 / HBM_PEAK_GBS,
+                                              "note": "state is 4x the last-level cache: achieved HBM rate"}
+    del S, qs, ks, vs, out
     # long context fwd+bwd, B=1 H=16 D=128 bf16, N sweep
     sweep = {}
     for n in (4096, 8192, 16384, 32768, 65536):
@@ -316,7 +402,7 @@ def run_extras(torch, ct, dev):
     byts = 11 * 8 * 16 * 2048 * 64 * 4
     flops = 28.0 * 8 * 16 * 2048 * 64 * 64   # executed by the chunked form (scores recomputed per gradient)
     # fused input preparation (normalise q,k; scale v; mask; fp32 -> bf16) at the headline shape, next to the same
-    # sequence written with torch elementwise ops as the reference module does (GPTCosAttention.py:216-235)
+    # sequence written with torch elementwise ops as the reference module does (GPTCosAttention.py:229-248)
     keep = torch.rand(8, 2048, device=dev) > 0.1
     cnt = keep.float().cumsum(-1)
     sig = torch.sigmoid(torch.randn(16, device=dev))
@@ -358,6 +444,7 @@ def run_extras(torch, ct, dev):
     s_b = time_region(torch, bert_step, 20, 3)
     ex["bert_block_fwd_bwd_B32_S512_E768_H12_autocast_bf16"] = {"us": s_b * 1e6, "tokens_per_s": 32 * 512 / s_b}
     del bert, bh_in, bg
+    ex["module_forward_latency_batch1_hidden2048_heads16"] = module_anchor(torch, dev)
     # prompt pass that also hands the state to decoding (cott_causal_fwd_state), headline shape
     qp, kp, vp, _ = make_inputs(torch, 8, 16, 2048, 64, 64, torch.bfloat16, dev)
     s_p = time_region(torch, lambda: ct.causal_prefill(qp, kp, vp), 100, 10)

@@ -45,7 +45,7 @@ class CustomAttention(torch.autograd.Function):
 
 class CustomAttentionMergedHeads(torch.autograd.Function):
     """CustomAttention with the head merge folded in: apply(Q, K, V) -> O of shape (N, S, H, Dv), i.e. the rows
-    of the (N, S, H*Dv) input of the output projection (GPT_Trainer/GPTCosAttention.py:479,500), and a backward
+    of the (N, S, H*Dv) input of the output projection (GPT_Trainer/GPTCosAttention.py:106-113, called at :500), and a backward
     that reads the gradient in that layout.  Only where ops.merged_heads_supported() holds for the dtype the
     forward computes in; callers fall back to CustomAttention + permute otherwise."""
 
@@ -85,7 +85,7 @@ class NonCausalAttention(torch.autograd.Function):
 
 class NonCausalAttentionMergedHeads(torch.autograd.Function):
     """NonCausalAttention returning O as (N, S, H, Dv) and reading its gradient in that layout
-    (BERT_Trainer/BertCosAttention.py:251-252); same conditions as CustomAttentionMergedHeads."""
+    (BERT_Trainer/BertCosAttention.py:317); same conditions as CustomAttentionMergedHeads."""
 
     @staticmethod
     def forward(ctx, Q, K, V):
@@ -104,8 +104,8 @@ class NonCausalAttentionMergedHeads(torch.autograd.Function):
 
 class PrepareInputs(torch.autograd.Function):
     """(q, k, v, keep, cnt, sig, out_dtype[, rot_table, position_ids, bnhd]) -> (q_hat, k_hat, v_scaled), (B,H,N,D):
-    the normalise / value-scale / mask steps in front of the attention op (GPT_Trainer/GPTCosAttention.py:216-241),
-    optionally with the rotary embedding and the head permute before them (:453-475), as one fused operator with a
+    the normalise / value-scale / mask steps in front of the attention op (GPT_Trainer/GPTCosAttention.py:229-248),
+    optionally with the rotary embedding and the head permute before them (:462-476), as one fused operator with a
     fused backward.  `sig` = sigmoid(norm_const) per head, differentiable; the other side inputs are constants."""
 
     @staticmethod

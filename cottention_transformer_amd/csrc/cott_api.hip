@@ -83,10 +83,30 @@ int exp_int(const char *name, int dflt) {
     return dflt;
 }
 
-// Workgroups a launch aims for: one per CU of a 256-CU part (a second workgroup on a CU adds only ~20 %
+// Workgroups a launch aims for: one per CU (a second workgroup on a CU adds only ~20 %
 // throughput to these LDS-heavy kernels, so grids just above the CU count run almost twice as long).
+// CUs of the current device, asked once per process (256 on an unpartitioned MI355X; the fallback when the query
+// fails).  A partitioned device reports fewer and gets correspondingly smaller launch plans.
+int device_cus() {
+    static const int v = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
+        return cus;
+    }();
+    return v;
+}
+int device_xcds() {
+    static const int v = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 8;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess || n <= 0) return 8;
+        return n;
+    }();
+    return v;
+}
 int target_workgroups() {
-    static const int v = [] { const int x = exp_int("COTT_TARGET_WGS", 0); return x > 0 ? x : 256; }();
+    static const int v = [] { const int x = exp_int("COTT_TARGET_WGS", 0); return x > 0 ? x : device_cus(); }();
     return v;
 }
 // -1 auto, 0 never, 1 always split the output columns of each op in two.
@@ -374,6 +394,8 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         ws_cursor += p.ws_bytes;
         a.BH = (int)BH; a.N = N;
         a.nchunks = p.nchunks; a.cpg = p.cpg; a.G = p.G; a.sub = p.sub;
+        a.cus = device_cus();
+        a.xcds = device_xcds();
         a.scan_prof_id = n > 1 ? cott::K_SCAN_GRAD : cott::K_SCAN;
         a.stream = stream;
         hipError_t e;
@@ -462,6 +484,13 @@ int cott_causal_fwd(const void *q, const void *k, const void *v, void *o, int B,
 }
 
 namespace {
+// dst[i] = src ? src[i] : 0 over n 16-byte vectors: the state pass-through of an empty sequence.  A kernel rather than
+// hipMemsetAsync / hipMemcpyAsync so that the call can be recorded into a HIP graph like every other launch here.
+__global__ __launch_bounds__(256) void state_passthrough_kernel(uint4 *dst, const uint4 *src, size_t n) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src ? src[i] : uint4{0u, 0u, 0u, 0u};
+}
+
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
 void *g_scratch_ptr[kMaxDevices] = {nullptr};
@@ -518,13 +547,16 @@ int cott_causal_fwd_state(const void *q, const void *k, const void *v, void *o, 
     if ((reinterpret_cast<uintptr_t>(state_in) & smask) || (reinterpret_cast<uintptr_t>(state_out) & smask))
         return fail(COTT_ERR_INVALID, "%s: state pointers must be 16-byte (fp64: 32-byte) aligned", fn);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (N == 0) {  // nothing to scan: the state passes through
-        if (state_out && state_in && state_out != state_in) {
-            hipError_t e = hipMemcpyAsync(state_out, state_in, (size_t)BH * Dk * Dv * ssz, hipMemcpyDeviceToDevice, st);
-            if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: state copy failed: %s", fn, hipGetErrorString(e));
-        } else if (state_out && !state_in) {
-            hipError_t e = hipMemsetAsync(state_out, 0, (size_t)BH * Dk * Dv * ssz, st);
-            if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: state clear failed: %s", fn, hipGetErrorString(e));
+    if (N == 0) {  // nothing to scan: the state passes through (or starts at zero)
+        if (state_out && state_out != state_in) {
+            const size_t bytes = (size_t)BH * Dk * Dv * ssz;
+            if (bytes % 16 != 0) return fail(COTT_ERR_UNSUPPORTED, "%s: state size %zu is not a multiple of 16 bytes", fn, bytes);
+            const size_t n16 = bytes / 16;
+            const unsigned blocks = (unsigned)((n16 + 255) / 256 < 2048 ? (n16 + 255) / 256 : 2048);
+            state_passthrough_kernel<<<dim3(blocks ? blocks : 1), dim3(256), 0, st>>>(
+                static_cast<uint4 *>(state_out), static_cast<const uint4 *>(state_in), n16);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return fail(COTT_ERR_HIP, "%s: state pass-through failed: %s", fn, hipGetErrorString(e));
         }
         return COTT_OK;
     }

@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256) void decode_kernel(SF *__restrict__ S, const t
 // then served from it on the next step.
 // Optional preparation of the raw projections of the ONE new token inside the decode step (on = 1): GPT-J
 // rotation of the first R columns of q and k by the table row `pos`, L2 normalisation of q and k, and
-// v / max(cnt^sig[h], 1) -- what GPT_Trainer/GPTCosAttention.py:216-241,453-475 do with separate kernels before
+// v / max(cnt^sig[h], 1) -- what GPT_Trainer/GPTCosAttention.py:229-248,462-476 do with separate kernels before
 // the recurrence of :264-267.  dk <= 256.
 struct DecodePrep {
     const float *sig;  // (H) sigmoid(norm_const), or null: no value scaling

@@ -59,6 +59,13 @@ hipError_t run_decode(void *state, const void *q, const void *k, const void *v, 
     if ((nv == 8 || nv == 16 || nv == 32 || nv == 64) && dk <= 1024) {
         // one wavefront per head, four heads per workgroup
         const size_t lds_w = (size_t)4 * 2 * dk * sizeof(SF);
+        if (lds_w > 48 * 1024) {  // (fp64 with dk = 1024: 64 KiB)
+            hipError_t e = prep.on ? hipFuncSetAttribute(reinterpret_cast<const void *>(decode_wave_kernel<ST, SF, true>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_w)
+                                   : hipFuncSetAttribute(reinterpret_cast<const void *>(decode_wave_kernel<ST, SF, false>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_w);
+            if (e != hipSuccess) return e;
+        }
         if (prep.on)
             decode_wave_kernel<ST, SF, true><<<dim3((unsigned)((BH + 3) / 4)), dim3(256), lds_w, stream>>>(
                 static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
@@ -71,6 +78,11 @@ hipError_t run_decode(void *state, const void *q, const void *k, const void *v, 
     }
     if (prep.on) return hipErrorInvalidValue;  // the fused preparation exists in the one-wavefront-per-head kernel only
     const size_t lds = (size_t)2 * dk * sizeof(SF) + 256 * 4 * sizeof(SF);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(decode_kernel<ST, SF>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
     decode_kernel<ST, SF><<<dim3((unsigned)BH), dim3(256), lds, stream>>>(
         static_cast<SF *>(state), static_cast<const E *>(q), static_cast<const E *>(k), static_cast<const E *>(v),
         static_cast<E *>(o), dk, dv);

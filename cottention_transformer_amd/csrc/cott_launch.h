@@ -43,6 +43,7 @@ struct SetArgs {
     // non-temporal loads in the group-state pass / in the scan: for tensors far larger than the caches, when no
     // two problems of the set read the same operand
     bool stream_state = false, stream_scan = false;
+    int cus = 256, xcds = 8;  // CUs and XCDs of the device (placement and occupancy choices)
     hipStream_t stream;
 };
 

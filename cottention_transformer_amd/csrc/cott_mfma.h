@@ -21,7 +21,6 @@ namespace cott {
 constexpr int kChunk = 64;     // positions per chunk
 constexpr int kThreads = 256;  // 4 wavefronts per workgroup
 constexpr int kMaxProblems = 6;
-constexpr int kXcds = 8;       // workgroup i is dispatched to XCD i % 8
 
 // One generic op.  A, B: rows of `di` elements, contiguous.  C, O: `dj` columns taken from rows of
 // `ldc` elements (the pointers already include the first column), so a problem can own a column
@@ -63,6 +62,7 @@ template <class E>
 struct ProblemSetT {
     ProblemT<E> p[kMaxProblems];
     int count;
+    int xcds;  // XCDs of the device: workgroup i is dispatched to XCD i % xcds (8 on an unpartitioned MI355X)
     // 16-bit kernels: the group-state pass cuts every group of the scan into `sub` pieces, one workgroup and one
     // slot each (slot (bh * G + grp) * sub + piece); the prefix pass leaves the scan's seed in the first of them
     int sub;
@@ -92,25 +92,25 @@ struct Tiling {
     static constexpr int OS = DJ + 8;            // ... of a staged output tile [64][DJ] (8-byte writes, 16-byte reads)
 };
 
-// Workgroup -> (head, problem, group).  Linear id i runs on XCD i % 8; per XCD the ids are ordered
+// Workgroup -> (head, problem, group).  Linear id i runs on XCD i % xcds; per XCD the ids are ordered
 // (head block, group, problem), so the workgroups of one head and group are neighbours in the
 // dispatch order of ONE XCD.
 struct WorkItem {
     int bh, prob, grp;
 };
-__device__ __forceinline__ WorkItem decode_workgroup(int nprob, int G) {
+__device__ __forceinline__ WorkItem decode_workgroup(int nprob, int G, int xcds) {
     const int i = blockIdx.x;
-    const int xcd = i % kXcds;
-    int slot = i / kXcds;
+    const int xcd = i % xcds;
+    int slot = i / xcds;
     WorkItem wi;
     wi.prob = slot % nprob;
     slot /= nprob;
     wi.grp = slot % G;
-    wi.bh = (slot / G) * kXcds + xcd;
+    wi.bh = (slot / G) * xcds + xcd;
     return wi;
 }
-inline unsigned grid_for(int BH, int nprob, int G) {
-    return (unsigned)(((BH + kXcds - 1) / kXcds) * kXcds * nprob * G);
+inline unsigned grid_for(int BH, int nprob, int G, int xcds) {
+    return (unsigned)(((BH + xcds - 1) / xcds) * xcds * nprob * G);
 }
 
 // [64][D] tile, global -> registers, through a buffer descriptor of the head.  Thread t of NT owns 16-byte
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int sub = set.sub;
-    const WorkItem wi = decode_workgroup(set.count, ngroups * sub);
+    const WorkItem wi = decode_workgroup(set.count, ngroups * sub, set.xcds);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
     const int grp = wi.grp / sub, piece = wi.grp % sub;
@@ -653,7 +653,7 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     __shared__ __attribute__((aligned(16))) u16 sO[STAGED ? 2 * 2 * kChunk * TL::OS : 8];
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const WorkItem wi = decode_workgroup(set.count, G);
+    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
@@ -715,7 +715,7 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     __shared__ __attribute__((aligned(16))) u16 sO[2 * 2 * kChunk * TL::OS];
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const WorkItem wi = decode_workgroup(set.count, G);
+    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
@@ -772,7 +772,7 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
     __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, G);
+    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, lda = pr.lda, ldo = pr.ldo;
@@ -839,7 +839,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
     __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, 1);
+    const WorkItem wi = decode_workgroup(set.count, 1, set.xcds);
     if (wi.bh >= BH) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, lda = pr.lda, ldb = pr.ldb, ldc = pr.ldc, ldo = pr.ldo;

@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kThreads) void group_state_f32_kernel(ProblemSetF32
     __shared__ __attribute__((aligned(16))) float sC[CH * TL::CS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, ngroups);
+    const WorkItem wi = decode_workgroup(set.count, ngroups, set.xcds);
     if (wi.bh >= BH) return;
     const ProblemF32 &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kThreads) void scan_f32_kernel(ProblemSetF32 set, i
     __shared__ __attribute__((aligned(16))) float sP[APPLY ? 4 : CH * TL::PS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, G);
+    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
     if (wi.bh >= BH) return;
     const ProblemF32 &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = APPLY ? 0 : pr.reversed;

@@ -12,7 +12,7 @@ hipError_t run_causal_f32(const SetArgs &a) {
     if (a.G > 1) {
         {
             ProfScope prof(K_GROUP_STATE, a.stream);
-            group_state_f32_kernel<DI, DJ><<<dim3(grid_for(a.BH, a.count, a.G - 1)), dim3(kThreads), 0, a.stream>>>(
+            group_state_f32_kernel<DI, DJ><<<dim3(grid_for(a.BH, a.count, a.G - 1, a.xcds)), dim3(kThreads), 0, a.stream>>>(
                 ps, a.BH, a.N, a.nchunks, a.cpg, a.G, a.G - 1);
         }
         const int bps = (TL::STATE_FLOATS / 4 + kThreads - 1) / kThreads;
@@ -21,7 +21,7 @@ hipError_t run_causal_f32(const SetArgs &a) {
             ps, a.BH, a.G, 1, a.G - 1, TL::STATE_FLOATS, 0);
     }
     ProfScope prof(a.scan_prof_id, a.stream);
-    scan_f32_kernel<DI, DJ, false><<<dim3(grid_for(a.BH, a.count, a.G)), dim3(kThreads), 0, a.stream>>>(
+    scan_f32_kernel<DI, DJ, false><<<dim3(grid_for(a.BH, a.count, a.G, a.xcds)), dim3(kThreads), 0, a.stream>>>(
         ps, a.BH, a.N, a.nchunks, a.cpg, a.G);
     return hipGetLastError();
 }
@@ -33,7 +33,7 @@ hipError_t run_noncausal_f32(const SetArgs &a) {
     const ProblemSetF32 ps = make_set<float, DI, DJ>(a);
     {
         ProfScope prof(K_GROUP_STATE, a.stream);
-        group_state_f32_kernel<DI, DJ><<<dim3(grid_for(a.BH, a.count, a.G)), dim3(kThreads), 0, a.stream>>>(
+        group_state_f32_kernel<DI, DJ><<<dim3(grid_for(a.BH, a.count, a.G, a.xcds)), dim3(kThreads), 0, a.stream>>>(
             ps, a.BH, a.N, a.nchunks, a.cpg, a.G, a.G);
     }
     if (a.G > 1) {
@@ -43,7 +43,7 @@ hipError_t run_noncausal_f32(const SetArgs &a) {
             ps, a.BH, a.G, 1, a.G, TL::STATE_FLOATS, 1);
     }
     ProfScope prof(K_APPLY, a.stream);
-    scan_f32_kernel<DI, DJ, true><<<dim3(grid_for(a.BH, a.count, a.G)), dim3(kThreads), 0, a.stream>>>(
+    scan_f32_kernel<DI, DJ, true><<<dim3(grid_for(a.BH, a.count, a.G, a.xcds)), dim3(kThreads), 0, a.stream>>>(
         ps, a.BH, a.N, a.nchunks, a.cpg, a.G);
     return hipGetLastError();
 }

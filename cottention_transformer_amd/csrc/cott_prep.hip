@@ -1,7 +1,7 @@
 // Fused input preparation of the cosine-attention module and its backward: L2-normalise the rows
 // of q and k, scale the rows of v by 1 / max(cnt^sig, 1), multiply all three by the 0/1 keep mask
 // and convert to the dtype the attention kernels run in -- one pass over each tensor
-// (GPT_Trainer/GPTCosAttention.py:216-241, BERT_Trainer/BertCosAttention.py:162-178 do this with
+// (GPT_Trainer/GPTCosAttention.py:229-248, BERT_Trainer/BertCosAttention.py:162-178 do this with
 // eight separate elementwise / reduction kernels).  Bandwidth-bound: every element is read once
 // and written once, rows are reduced with lane shuffles inside a wavefront.
 #include "cott_common.h"

@@ -1,9 +1,9 @@
 """Attention modules with the reference's constructor, parameter names and forward signatures, running the
 cosine-attention core on the HIP path.
 
-    GPTCosAttention   <- GPT_Trainer/GPTCosAttention.py:38-508 (GPT-J attention block: q/k/v projections, rotary
+    GPTCosAttention   <- GPT_Trainer/GPTCosAttention.py:40-508 (GPT-J attention block: q/k/v projections, rotary
                          embedding, causal cosine attention, output projection; optional recurrent inference)
-    BertCosAttention  <- BERT_Trainer/BertCosAttention.py:56-334 (BERT self-attention block, non-causal form)
+    BertCosAttention  <- BERT_Trainer/BertCosAttention.py:60-334 (BERT self-attention block, non-causal form)
 
 Parameter / buffer names match (q_proj, k_proj, v_proj, out_proj, norm_const; query, key, value, norm_const), so a
 state_dict of the reference modules loads unchanged.  What differs is inside: the normalise / value-scale / mask
@@ -28,7 +28,7 @@ def _autocast_on():
 
 def _common_dtype(q, k, v):
     """Under autocast the projections are bf16 but the rotary table is fp32, so q and k arrive as fp32 and v as
-    bf16; the reference's normalize / divide promote everything to fp32 as well (GPTCosAttention.py:216-228)."""
+    bf16; the reference's normalize / divide promote everything to fp32 as well (GPTCosAttention.py:229-241)."""
     dt = torch.promote_types(torch.promote_types(q.dtype, k.dtype), v.dtype)
     return q.to(dt), k.to(dt), v.to(dt)
 
@@ -43,7 +43,7 @@ def rotary_table(num_pos, dim):
 
 def apply_rotary(x, sin, cos):
     """Rotates consecutive pairs (x[2i], x[2i+1]) by the angle of column i.  x: (B,S,H,R); sin, cos: (B,S,R/2)
-    (`apply_rotary_pos_emb` of GPT-J, used at GPTCosAttention.py:463-472)."""
+    (`apply_rotary_pos_emb` of GPT-J, used at GPTCosAttention.py:462-476)."""
     s, c = sin[:, :, None, :], cos[:, :, None, :]
     even, odd = x[..., 0::2], x[..., 1::2]
     return torch.stack([even * c - odd * s, odd * c + even * s], dim=-1).flatten(-2)
@@ -51,7 +51,7 @@ def apply_rotary(x, sin, cos):
 
 def _keep_from_additive_mask(attention_mask, batch, length, device):
     """The modules receive the additive mask of the surrounding model, (B,1,1,S) with 0 at real tokens; both turn
-    it into a boolean keep mask with `attention_mask == 0` (GPTCosAttention.py:219, BertCosAttention.py:165)."""
+    it into a boolean keep mask with `attention_mask == 0` (GPTCosAttention.py:232, BertCosAttention.py:163)."""
     if attention_mask is None:
         return torch.ones(batch, length, dtype=torch.bool, device=device)
     return (attention_mask == 0).reshape(batch, length)
@@ -76,7 +76,7 @@ class GPTCosAttention(nn.Module):
         self.out_proj = nn.Linear(self.embed_dim, self.embed_dim, bias=False)
         self.rotary_dim = config.rotary_dim
         self.embed_positions = rotary_table(max_positions, self.rotary_dim or self.embed_dim)
-        # learnable exponent of the value scaling, one per head (GPTCosAttention.py:91)
+        # learnable exponent of the value scaling, one per head (GPTCosAttention.py:89)
         self.norm_const = nn.Parameter(0.5 * torch.ones(1, self.num_attention_heads, 1, 1))
         # recurrent inference (GPTCosAttention.py:77-87): state is created on first use, per batch element
         self.fast_inference = bool(getattr(config, "fast_inference", False))
@@ -90,7 +90,7 @@ class GPTCosAttention(nn.Module):
     def _decode_one(self, query, key, value):
         """One new token in recurrent inference, from the raw projections (B,1,H,D): rotation by position
         cur_s - 1, normalisation, value scaling by cur_s ** sigmoid(norm_const) and the state update / read-out
-        (GPTCosAttention.py:216-241, 253-272, 453-475) as one kernel launch.  Returns (B,1,H*D)."""
+        (GPTCosAttention.py:229-248, 253-272, 462-476) as one kernel launch.  Returns (B,1,H*D)."""
         b, _, h, d = query.shape
         query, key, value = _common_dtype(query, key, value)
         if self.state is None:
@@ -128,7 +128,7 @@ class GPTCosAttention(nn.Module):
 
     def _cos_attn(self, query, key, value, attention_mask=None, head_mask=None, rotary=None, bnhd=False,
                   merge_heads=False):
-        """GPTCosAttention.py:200-282.  query, key, value: (B,H,S,D), already rotated -- or, with `bnhd`, (B,S,H,D)
+        """GPTCosAttention.py:161-282.  query, key, value: (B,H,S,D), already rotated -- or, with `bnhd`, (B,S,H,D)
         as the projections produce them, with rotary=(table, position_ids) still to be applied; in that case the
         rotation, the head permute and the preparation steps are one fused pass.
         merge_heads: the caller wants the output as (B,S,H,D) (:500); returned that way, with None in place of
@@ -142,7 +142,7 @@ class GPTCosAttention(nn.Module):
         sig = self.norm_const.sigmoid().reshape(h)
         table, pos = rotary if rotary is not None else (None, None)
         if self.fast_inference:
-            # value scaling by absolute position (:223), then the recurrence (:253-272) from the stored state
+            # value scaling by absolute position (:236), then the recurrence (:253-272) from the stored state
             cnt = (self.cur_s + torch.arange(s, device=query.device, dtype=torch.float32)).expand(b, s)
             dt = query.dtype
             q, k, v = ops.prepare_inputs(query, key, value, keep, cnt, sig, out_dtype=dt, rotary=rotary, bnhd=bnhd,
@@ -251,7 +251,7 @@ class BertCosAttention(nn.Module):
                                       dt, None, None, True)
         # Q (K^T V)  (:249); (QK^T)V at :222 is the same product
         if ops.merged_heads_supported(q.dtype, s, h, q.shape[-1], v.shape[-1]):
-            context_layer = NonCausalAttentionMergedHeads.apply(q, k, v)  # already (B,S,H,D) (:251)
+            context_layer = NonCausalAttentionMergedHeads.apply(q, k, v)  # already (B,S,H,D) (:317)
             if not _autocast_on():
                 context_layer = context_layer.to(hidden_states.dtype)
         else:

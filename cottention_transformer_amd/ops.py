@@ -187,7 +187,7 @@ def causal_backward(q, k, v, grad_out, merged_heads=False):
 
 def noncausal_dot_product(q, k, v, merged_heads=False):
     """o = q (k^T v) per (batch, head): BERT_Trainer/BertCosAttention.py:249.  merged_heads: o as (B,N,H,Dv)
-    (the context-layer permute of :251-252 without its copy; see merged_heads_supported)."""
+    (the context-layer permute of :317 without its copy; see merged_heads_supported)."""
     _require_gpu(Q=q, K=k, V=v)
     b, h, n, dk, dv = _shapes(q, k, v)
     if not (q.dtype == k.dtype == v.dtype):
@@ -352,12 +352,12 @@ def prepare_inputs(q, k, v, keep=None, cnt=None, sig=None, out_dtype=None, rotar
     """Fused input preparation of the cosine-attention module, one pass per tensor:
         q_out = keep * q / max(|q|, 1e-12),  k_out likewise,  v_out = keep * v / max(cnt ** sig[h], 1)
     converted to `out_dtype` (default: the input dtype) and returned as (B,H,N,D).  Replaces
-    GPT_Trainer/GPTCosAttention.py:216-241 and BERT_Trainer/BertCosAttention.py:162-178.
+    GPT_Trainer/GPTCosAttention.py:229-248 and BERT_Trainer/BertCosAttention.py:162-178.
     keep: (B,N) bool/0-1, True = real token; cnt: (B,N) number of kept keys each position attends to;
     sig: (H,) = sigmoid(norm_const).
     rotary=(table, position_ids): also applies the GPT-J rotary embedding to the first table.size(1) columns of
-    q and k (GPTCosAttention.py:453-472); bnhd=True: q, k, v are given as (B,N,H,D), the layout the projections
-    produce, and the head permute of :474-475 happens in the same pass."""
+    q and k (GPTCosAttention.py:462-476); bnhd=True: q, k, v are given as (B,N,H,D), the layout the projections
+    produce, and the head permute of :478-479 happens in the same pass."""
     _require_gpu(Q=q, K=k, V=v)
     b, h, n, dk, dv = _prep_shapes(q, k, v, bnhd)
     if not (q.dtype == k.dtype == v.dtype):

@@ -100,7 +100,7 @@ COTT_API int cott_causal_bwd(const void *q, const void *k, const void *v, const 
  * The same two operations with the attention output o (forward) and its gradient d_o (backward) laid out
  * (B,N,H,Dv), i.e. as the rows of the (B,N,H*Dv) tensor that the output projection reads and
  * differentiates.  Replaces the permute + contiguous copy of the head merge around the op
- * (GPT_Trainer/GPTCosAttention.py:500 `_merge_heads`, called at :479, and its backward).  q, k, v and
+ * (GPT_Trainer/GPTCosAttention.py:106-113 `_merge_heads`, called at :500, and its backward).  q, k, v and
  * dq, dk, dv stay (B,H,N,D) (cott_prep_ex_* already reads and writes the projection layout on that side).
  * bf16 / fp16, head dims 32..128 in steps of 16, N*H*D <= 2^30; other cases return COTT_ERR_UNSUPPORTED
  * and the caller permutes.  Workspace: cott_causal_workspace_bytes / cott_causal_bwd_workspace_bytes. */
@@ -127,7 +127,7 @@ COTT_API int cott_noncausal_bwd(const void *q, const void *k, const void *v, con
                        void *workspace, size_t workspace_bytes, void *stream);
 
 /* Non-causal form with o / d_o laid out (B,N,H,Dv): the context-layer permute of
- * BERT_Trainer/BertCosAttention.py:251-252 and its backward without the copy.  Same limits as
+ * BERT_Trainer/BertCosAttention.py:317 and its backward without the copy.  Same limits as
  * cott_causal_fwd_bnhd; workspace: cott_noncausal_workspace_bytes. */
 COTT_API int cott_noncausal_fwd_bnhd(const void *q, const void *k, const void *v, void *o,
                             int B, int H, int N, int Dk, int Dv, int dtype,
@@ -151,7 +151,7 @@ COTT_API int cott_decode_step(void *state, const void *q, const void *k, const v
  * clamped to the table), the L2 normalisation of q and k and v / max(cnt^sig[h], 1) (sig: (H) fp32 =
  * sigmoid(norm_const), NULL = no scaling; cnt = tokens so far including this one) run inside the kernel: one
  * launch per token and layer instead of the separate elementwise kernels of
- * GPT_Trainer/GPTCosAttention.py:216-241,453-475 in front of :264-267.  q, k: (B,H,Dk) = the (B,1,H,Dk)
+ * GPT_Trainer/GPTCosAttention.py:229-248,462-476 in front of :264-267.  q, k: (B,H,Dk) = the (B,1,H,Dk)
  * projection output; Dv in {32,64,128,256}, Dk <= 256. */
 COTT_API int cott_decode_step_prep(void *state, const void *q, const void *k, const void *v, void *o,
                           const float *sig, float cnt, const float *rot_table, long long position,
@@ -162,8 +162,8 @@ COTT_API int cott_decode_step_prep(void *state, const void *q, const void *k, co
  *   q_out = keep * q / max(|q|_2, 1e-12)     (rows of Dk; same for k)
  *   v_out = keep * v / max(cnt^sig[h], 1)    (rows of Dv)
  * in one pass per tensor, converting in_dtype -> out_dtype on the way.  Replaces the eight
- * elementwise / reduction kernels of GPT_Trainer/GPTCosAttention.py:216-241 (normalize :216-217,
- * value scaling :222-228, mask multiplies :232-235) and BERT_Trainer/BertCosAttention.py:162-178
+ * elementwise / reduction kernels of GPT_Trainer/GPTCosAttention.py:229-248 (normalize :229-230,
+ * value scaling :234-241, mask multiplies :243-248) and BERT_Trainer/BertCosAttention.py:162-178
  * (for a 0/1 mask the order mask/normalise/scale does not matter).
  * keep: (B,N) bytes, 0 = padded position, or NULL.  cnt: (B,N) fp32, the number of kept keys a
  * position attends to (GPT: running count, :228; BERT: the total, :178) and sig: (H) fp32 =
@@ -178,10 +178,10 @@ COTT_API int cott_prep_bwd(const void *q, const void *k, const void *v,
                   float *dsig_rows, const unsigned char *keep, const float *cnt, const float *sig,
                   int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream);
 
-/* The same with the two steps that surround it in the GPT block folded in (GPTCosAttention.py:434-476):
+/* The same with the two steps that surround it in the GPT block folded in (GPTCosAttention.py:444-479):
  * in_bnhd != 0: q, k, v (and, backward, dq, dk, dv) are laid out (B,N,H,D), as the projections produce them
- * (the outputs / incoming gradients stay (B,H,N,D)), which removes the permute + contiguous copies of :474-475 and
- * Custom_Kernel.py:11-13;  rot_table != NULL: the GPT-J rotary embedding (apply_rotary_pos_emb, :463-472) is
+ * (the outputs / incoming gradients stay (B,H,N,D)), which removes the permute + contiguous copies of :478-479 and
+ * Custom_Kernel.py:11-13;  rot_table != NULL: the GPT-J rotary embedding (apply_rotary_pos_emb, :462-476) is
  * applied to the first rotary_dim columns of q and k before normalisation.  rot_table: (table_rows, rotary_dim)
  * fp32, row p = [sin(p f_i) | cos(p f_i)]; pos: (B,N) int64 row index per position; an index outside [0, table_rows) is clamped
  * to the table on the device, nothing reports it. */

@@ -70,9 +70,9 @@ def synthetic_inputs(shape_qk, dv=None, seed=0, dtype=torch.float32, with_grad_o
 
 def input_prep_gpt(q, k, v, keep=None, sig=None):
     """CPU statement of the module-side preparation in front of the causal op, in the reference's order
-    (GPT_Trainer/GPTCosAttention.py:216-235): L2-normalise q and k (:216-217); divide v by
-    clamp(cnt ** sig, min=1) with cnt[b,s] = number of kept keys at positions <= s (:228, causal mask times
-    padding mask, summed over keys); multiply q, k, v by the keep mask (:232-235).
+    (GPT_Trainer/GPTCosAttention.py:229-248): L2-normalise q and k (:229-230); divide v by
+    clamp(cnt ** sig, min=1) with cnt[b,s] = number of kept keys at positions <= s (:241, causal mask times
+    padding mask, summed over keys); multiply q, k, v by the keep mask (:243-248).
     q,k: (B,H,N,Dk), v: (B,H,N,Dv), keep: (B,N) bool (True = real token) or None, sig: (H,) or None.
     Returns (q_hat, k_hat, v_scaled, cnt)."""
     b, h, n, _ = q.shape
@@ -140,7 +140,7 @@ def _gpt_qkv(hidden, wq, wk, wv, num_heads, rotary_dim, max_pos, position_ids):
 
 
 def gpt_attention_block(hidden, wq, wk, wv, wo, norm_const, num_heads, rotary_dim, max_pos, keep=None, position_ids=None):
-    """Training/evaluation path of the GPT block (GPT_Trainer/GPTCosAttention.py:429-506 with _cos_attn :200-282):
+    """Training/evaluation path of the GPT block (GPT_Trainer/GPTCosAttention.py:430-506 with _cos_attn :200-282):
     projections, rotary, input preparation, causal cosine attention, merge heads, output projection.
     hidden: (B,S,E); weights as nn.Linear stores them; norm_const: (H,); keep: (B,S) bool."""
     b, s, e = hidden.shape
@@ -176,7 +176,7 @@ def gpt_attention_block_recurrent(hidden, wq, wk, wv, wo, norm_const, num_heads,
 
 
 def bert_attention_block(hidden, wq, bq, wk, bk, wv, bv, norm_const, num_heads, keep=None):
-    """BERT self-attention block (BERT_Trainer/BertCosAttention.py:104-334): projections with bias, mask, normalise,
+    """BERT self-attention block (BERT_Trainer/BertCosAttention.py:111-334): projections with bias, mask, normalise,
     value scaling by the number of real tokens, Q (K^T V), merge heads."""
     b, s, e = hidden.shape
     d = e // num_heads

@@ -77,7 +77,7 @@ def test_gpt_block_forward_backward(mods, autocast):
 
 
 def test_gpt_block_recurrent_inference(mods):
-    # GPTCosAttention.py:77-87,222-223,253-272: a prompt, then single tokens, against the per-token loop on the CPU
+    # GPTCosAttention.py:77-87,234-236,253-272: a prompt, then single tokens, against the per-token loop on the CPU
     from oracle import torch_forms as tf
     say("gpt recurrent")
     torch.manual_seed(0)

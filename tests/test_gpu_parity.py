@@ -204,7 +204,7 @@ def test_noncausal_forward_backward(ct, oracle, case):
 
 
 @pytest.mark.parametrize("case", [(2, 3, 128, 128, BF), (1, 2, 64, 32, HF), (2, 2, 64, 64, F32), (1, 2, 32, 48, F64),
-                                  (1, 1, 128, 2048, F32)], ids=lambda c: "x".join(map(str, c[:4])) + "-" + str(c[4]).split(".")[-1])
+                                  (1, 1, 128, 2048, F32), (1, 2, 8192, 8, F32), (1, 1, 4096, 12, F64)], ids=lambda c: "x".join(map(str, c[:4])) + "-" + str(c[4]).split(".")[-1])
 def test_decode_steps(ct, oracle, case):
     b, h, dk, dv, dt = case
     say("decode", case)
@@ -314,6 +314,8 @@ def test_prefill_hands_state_to_next_piece_and_to_decode(ct, oracle, case):
     assert none is None and torch.equal(o3, o1)
     oe, se = ct.causal_prefill(qd[:, :, :0], kd[:, :, :0], vd[:, :, :0], state=s1)
     assert oe.shape == (b, h, 0, dv) and torch.equal(se, s1)
+    oe, se = ct.causal_prefill(qd[:, :, :0], kd[:, :, :0], vd[:, :, :0])       # no state in: the state out is zero
+    assert se.shape == (b, h, dk, dv) and not se.any()
 
 
 def test_padded_rows_and_noncontiguous_inputs(ct, oracle):
@@ -440,7 +442,7 @@ PREP_CASES = [
 @pytest.mark.parametrize("case", PREP_CASES,
                          ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1] + "-" + str(c[6]).split(".")[-1])
 def test_fused_input_preparation_forward_and_backward(ct, case):
-    # GPT_Trainer/GPTCosAttention.py:216-235 and BERT_Trainer/BertCosAttention.py:162-178 against their CPU statement
+    # GPT_Trainer/GPTCosAttention.py:229-248 and BERT_Trainer/BertCosAttention.py:162-178 against their CPU statement
     # (oracle/torch_forms.py, pinned by loops in tests/test_oracle_pinning.py), gradients by torch.autograd in fp64.
     from oracle import torch_forms as tf
     b, h, n, dk, dv, dt_in, dt_out, masked = case
@@ -509,7 +511,7 @@ def test_prepare_inputs_autograd_function_feeds_attention(ct, oracle):
                                   (1, 4, 130, 256, 64, HF, F32, 64), (2, 2, 40, 512, 512, F32, F32, 256)],
                          ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1] + "-rot" + str(c[7]))
 def test_input_preparation_with_rotary_and_projection_layout(ct, case):
-    # GPTCosAttention.py:434-476: split heads (B,S,H,D), rotary on the first R columns of q and k, permute to
+    # GPTCosAttention.py:444-479: split heads (B,S,H,D), rotary on the first R columns of q and k, permute to
     # (B,H,S,D), then the preparation steps -- against the same sequence written with the CPU forms.
     from oracle import torch_forms as tf
     b, h, n, dk, dv, dt_in, dt_out, rdim = case

@@ -49,7 +49,7 @@ def _weights(e, seed):
 
 def test_gpt_block_training_path_equals_recurrent_path():
     # With no padding the running count of kept keys at position s is s+1 = cur_s + s for cur_s = 1, so the
-    # training path (cumsum form, GPTCosAttention.py:228,282) and the recurrent path (:223,253-272) must agree.
+    # training path (cumsum form, GPTCosAttention.py:241,282) and the recurrent path (:223,253-272) must agree.
     b, s, heads, e, rot = 2, 19, 2, 64, 16
     wq, wk, wv, wo = _weights(e, 1)
     g = torch.Generator().manual_seed(2)
@@ -72,12 +72,12 @@ def test_module_parameter_names_match_the_reference_checkpoints():
     cfg = SimpleNamespace(max_position_embeddings=32, attn_pdrop=0.0, resid_pdrop=0.0, hidden_size=64,
                           num_attention_heads=2, rotary_dim=16)
     m = modules.GPTCosAttention(cfg)
-    # GPT_Trainer/GPTCosAttention.py:67-70,91 (its mask buffers are non-persistent, :43-51)
+    # GPT_Trainer/GPTCosAttention.py:67-70,89 (its mask buffers are non-persistent, :43-51)
     assert sorted(m.state_dict()) == ["k_proj.weight", "norm_const", "out_proj.weight", "q_proj.weight", "v_proj.weight"]
     assert m.norm_const.shape == (1, 2, 1, 1) and float(m.norm_const.flatten()[0]) == 0.5
     cfg = SimpleNamespace(hidden_size=64, num_attention_heads=2, attention_probs_dropout_prob=0.0, is_decoder=False)
     m = modules.BertCosAttention(cfg)
-    # BERT_Trainer/BertCosAttention.py:69-71,77
+    # BERT_Trainer/BertCosAttention.py:73-75,81
     assert sorted(m.state_dict()) == ["key.bias", "key.weight", "norm_const", "query.bias", "query.weight",
                                       "value.bias", "value.weight"]
     with pytest.raises(RuntimeError):                                    # no CPU fallback behind the modules
