@@ -228,7 +228,9 @@ struct DecodePrep {
     int R, H, on;
 };
 
-template <class ST, class SF, bool PREP>
+// NT bit 0: non-temporal state loads, bit 1: non-temporal state stores (a state far larger than the last-level
+// cache is not found there again by the next step).
+template <class ST, class SF, bool PREP, int NT = 0>
 __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, const typename ST::elem *__restrict__ q,
                                                           const typename ST::elem *__restrict__ k,
                                                           const typename ST::elem *__restrict__ v,
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, co
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int r = r0 + u * rpw;
-            if (r < dk) s[u] = col[(size_t)r * nv];
+            if (r < dk) s[u] = (NT & 1) ? __builtin_nontemporal_load(&col[(size_t)r * nv]) : col[(size_t)r * nv];
         }
         if (!staged) {
             if constexpr (PREP) {
@@ -324,7 +326,10 @@ __global__ __launch_bounds__(256) void decode_wave_kernel(SF *__restrict__ S, co
             const int r = r0 + u * rpw;
             if (r < dk) {
                 s[u] += sk[r] * vv;
-                col[(size_t)r * nv] = s[u];
+                if (NT & 2)
+                    __builtin_nontemporal_store(s[u], &col[(size_t)r * nv]);
+                else
+                    col[(size_t)r * nv] = s[u];
                 acc += sq[r] * s[u];
             }
         }

@@ -126,3 +126,25 @@ def test_decode_512_steps_at_benchmark_size(ct, oracle):
     err = float((state.double() - total).norm() / total.norm())
     say(f"  state of all batch elements vs fp64 sum: {err:.2e}")
     assert err <= 1e-5
+
+
+def test_decode_on_a_state_beyond_the_last_level_cache(ct, oracle):
+    """A state of 400 MiB (B=400, H=16, D=128) takes the decode kernel's streaming variant (non-temporal state
+    accesses): three steps, outputs of every 16th batch element against the oracle and the final state of all of
+    them against s0 + sum_t k_t v_t^T in fp64."""
+    b, h, d, steps = 400, 16, 128, 3
+    sub = slice(0, b, 16)
+    g = torch.Generator(device=DEV).manual_seed(9)
+    s0 = 0.01 * torch.randn(b, h, d, d, generator=g, device=DEV)
+    qs = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g, device=DEV), dim=-1).to(BF)
+    ks = torch.nn.functional.normalize(torch.randn(steps, b, h, d, generator=g, device=DEV), dim=-1).to(BF)
+    vs = torch.randn(steps, b, h, d, generator=g, device=DEV).to(BF)
+    state = s0.clone()
+    ref_state = s0[sub].double().cpu().numpy().copy()
+    for t in range(steps):
+        out = ct.decode_step(state, qs[t], ks[t], vs[t])
+        ref = oracle.decode_step(ref_state, qs[t, sub].cpu(), ks[t, sub].cpu(), vs[t, sub].cpu())
+        assert rel_l2(out[sub], ref) <= 2e-2, t
+    assert rel_l2(state[sub], ref_state) <= 1e-6
+    total = s0.double() + torch.einsum("tbhi,tbhj->bhij", ks.double(), vs.double())
+    assert float((state.double() - total).norm() / total.norm()) <= 1e-6
