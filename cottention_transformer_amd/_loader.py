@@ -20,6 +20,8 @@ SIGNATURES = {
     "cott_causal_fwd": (_i, [_vp] * 4 + [_i] * 7 + [_vp, _sz, _vp]),
     "cott_noalloc_scratch_bytes": (_sz, []),
     "cott_causal_fwd_noalloc": (_i, [_vp] * 4 + [_i] * 7 + [_vp]),
+    "cott_causal_fwd_prep_supported": (_i, [_i] * 7),
+    "cott_causal_fwd_prep": (_i, [_vp] * 11 + [ctypes.c_longlong] + [_i] * 10 + [_vp]),
     "cott_causal_fwd_state": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_prep_fwd": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
     "cott_prep_bwd": (_i, [_vp] * 13 + [_i] * 7 + [_vp]),

@@ -128,3 +128,37 @@ class PrepareInputs(torch.autograd.Function):
         if dsig is not None:
             dsig = dsig.to(sig.dtype)
         return dq, dk, dv, None, None, dsig, None, None, None, None
+
+
+class PreparedCausalAttention(torch.autograd.Function):
+    """(q, k, v, keep, cnt, sig, rot_table, first_position, bnhd, merged_heads) -> O: the preparation steps of
+    PrepareInputs and the causal attention op as ONE forward launch on the raw projections
+    (ops.causal_dot_product_prepared).  The kernel also leaves the prepared q, k, v for the backward pass, which is
+    the attention gradient on them followed by the fused backward of the preparation.  Positions are consecutive:
+    the table row of position s is first_position + s.  Only where ops.fused_preparation_supported() holds."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, keep, cnt, sig, rot_table=None, first_position=0, bnhd=False, merged_heads=False):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        rotary = (rot_table, int(first_position)) if rot_table is not None else None
+        out, prepared = ops.causal_dot_product_prepared(q, k, v, keep, cnt, sig, rotary=rotary, bnhd=bnhd,
+                                                        merged_heads=merged_heads, want_prepared=True)
+        ctx.save_for_backward(q, k, v, keep, cnt, sig, rot_table, *prepared)
+        ctx.first_position, ctx.bnhd, ctx.merged = int(first_position), bool(bnhd), bool(merged_heads)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k, v, keep, cnt, sig, rot_table, qh, kh, vh = ctx.saved_tensors
+        gq, gk, gv = ops.causal_backward(qh, kh, vh, grad_output.contiguous().to(qh.dtype), merged_heads=ctx.merged)
+        rotary = None
+        if rot_table is not None:
+            b, n = (q.shape[0], q.shape[1]) if ctx.bnhd else (q.shape[0], q.shape[2])
+            pos = torch.arange(ctx.first_position, ctx.first_position + n, device=q.device).expand(b, n)
+            rotary = (rot_table, pos)
+        want = sig is not None and ctx.needs_input_grad[5]
+        dq, dk, dv, dsig = ops.prepare_inputs_backward(q, k, v, gq, gk, gv, keep, cnt, sig, want_dsig=want, rotary=rotary,
+                                                       bnhd=ctx.bnhd, check_positions=False)
+        if dsig is not None:
+            dsig = dsig.to(sig.dtype)
+        return dq, dk, dv, None, None, dsig, None, None, None, None

@@ -317,7 +317,7 @@ int check_common(const char *fn, int B, int H, int N, int di, int dj, int dtype)
 
 // Runs n generic ops (n <= 3) over the same (BH, N) on the best available kernel family.
 int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, int dtype, void *ws, size_t ws_bytes,
-            hipStream_t stream) {
+            hipStream_t stream, const cott::SetArgs::Prep *prep = nullptr) {
     bool mfma = true;
     for (int i = 0; i < n; ++i) mfma = mfma && use_mfma(dtype, ops[i].di, ops[i].dj, N);
     const size_t esz = elem_size(dtype);
@@ -338,6 +338,9 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         return COTT_OK;
     }
     const size_t need = ops_workspace(ops, n, BH, N, dtype, causal);
+    if (prep != nullptr && need > 0)
+        return fail(COTT_ERR_UNSUPPORTED, "%s: B*H = %ld heads are cut into sequence groups at N = %d; the fused preparation "
+                    "needs one group per head (prepare the inputs with cott_prep_ex_fwd instead)", fn, BH, N);
     if (need > 0 && (ws == nullptr || ws_bytes < need || !aligned16(ws)))
         return fail(COTT_ERR_WORKSPACE, "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", fn, need,
                     ws ? ws_bytes : (size_t)0);
@@ -352,6 +355,12 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
             if (!done[j] && pad_key(ops[j]) == pad_key(ops[i])) { done[j] = true; members[cnt++] = j; }
         const SetLayout L = layout_set(ops, n, members, cnt, BH, N, dtype, causal);
         const SetPlan &p = L.p;
+        if (prep != nullptr) {
+            if (p.G != 1)
+                return fail(COTT_ERR_UNSUPPORTED, "%s: B*H = %ld heads are cut into %d sequence groups at N = %d; the fused "
+                            "preparation needs one group per head (prepare the inputs with cott_prep_ex_fwd instead)", fn, BH, p.G, N);
+            a.prep = *prep;
+        }
         const bool pair = L.pair, complement = L.complement;
         const int *twin_of = L.twin_of;
         a.pair = pair ? 1 : 0;
@@ -382,6 +391,7 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
                 d.reversed = o.reversed;
                 d.comp = (complement && !o.reversed && !o.sin && !o.sout) ? 1 : 0;
                 d.seed_from = twin_of[c];  // (halves == 1 here: set index == member index)
+                d.c0 = h * djh;
                 const size_t ssz = dtype == COTT_F64 ? 8 : 4;
                 d.sin = o.sin ? static_cast<const char *>(o.sin) + (size_t)h * djh * ssz : nullptr;
                 d.sout = o.sout ? static_cast<char *>(o.sout) + (size_t)h * djh * ssz : nullptr;
@@ -481,6 +491,68 @@ int cott_causal_fwd(const void *q, const void *k, const void *v, void *o, int B,
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
     const Op op{q, k, v, o, Dk, Dv, reversed ? 1 : 0};
     return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim) {
+    if (B < 0 || H < 0 || N < 0 || (dtype != COTT_BF16 && dtype != COTT_F16) || Dk % 16 != 0 || Dk < 32) return 0;
+    if (!use_mfma(dtype, Dk, Dv, N)) return 0;
+    if (rotary_dim != 0 && (rotary_dim < 8 || rotary_dim % 8 != 0 || rotary_dim > Dk)) return 0;
+    const long dmax = Dk > Dv ? Dk : Dv;
+    if ((long)N * H * dmax > (1L << 30) || (long)B * H > (1L << 22)) return 0;
+    if ((long)B * H * N == 0) return 1;
+    const SetPlan p = plan_set((long)B * H, N, 1, Dk, Dv, true, dtype);
+    // one group per head, and tiles small enough that the prepared q tile fits LDS beside them
+    return p.G == 1 && cott::mfma_pad(Dk) * cott::mfma_pad(Dv / p.halves) <= 128 * 64;
+}
+
+int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
+                         const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
+                         long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, int B, int H, int N, int Dk,
+                         int Dv, int dtype, void *stream) {
+    const char *fn = "cott_causal_fwd_prep";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if (dtype != COTT_BF16 && dtype != COTT_F16)
+        return fail(COTT_ERR_UNSUPPORTED, "%s: needs bf16 / fp16 tensors", fn);
+    if (!use_mfma(dtype, Dk, Dv, N))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: needs head dims 32..128 in steps of 16", fn);
+    if ((cnt == nullptr) != (sig == nullptr)) return fail(COTT_ERR_INVALID, "%s: cnt and sig go together", fn);
+    if (rot_table != nullptr) {
+        if (rotary_dim < 8 || rotary_dim % 8 != 0 || rotary_dim > Dk)
+            return fail(COTT_ERR_INVALID, "%s: rotary_dim must be a multiple of 8 in [8, Dk] (got %d)", fn, rotary_dim);
+        if (table_rows < 1) return fail(COTT_ERR_INVALID, "%s: empty rotary table", fn);
+    }
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (!cott_causal_fwd_prep_supported(B, H, N, Dk, Dv, dtype, rot_table ? rotary_dim : 0))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation needs one group per head and tiles of at most 128 x 64 "
+                    "(cott_causal_fwd_prep_supported); prepare the inputs with cott_prep_ex_fwd instead", fn);
+    if (in_bnhd || o_bnhd) {
+        const long dmax = Dk > Dv ? Dk : Dv;
+        if ((long)N * H * dmax > (1L << 30))
+            return fail(COTT_ERR_UNSUPPORTED, "%s: N*H*D = %ld exceeds 2^30", fn, (long)N * H * dmax);
+    }
+    if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(q_out) || !aligned16(k_out) ||
+        !aligned16(v_out) || !aligned16(rot_table))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op op{q, k, v, o, Dk, Dv, 0};
+    op.H = H;
+    if (in_bnhd) op.lay[0] = op.lay[1] = op.lay[2] = 1;
+    if (o_bnhd) op.lay[3] = 1;
+    cott::SetArgs::Prep prep;
+    prep.on = true;
+    prep.keep = keep;
+    prep.cnt = cnt;
+    prep.sig = sig;
+    prep.rot = rot_table;
+    prep.pos0 = pos0;
+    prep.R = rot_table ? rotary_dim : 0;
+    prep.table_rows = table_rows;
+    prep.H = H;
+    prep.dv = Dv;
+    prep.qo = q_out;
+    prep.ko = k_out;
+    prep.vo = v_out;
+    return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, nullptr, 0, static_cast<hipStream_t>(stream), &prep);
 }
 
 namespace {

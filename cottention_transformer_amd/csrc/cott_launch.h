@@ -23,6 +23,7 @@ struct OpDesc {
     // Complement form (16-bit causal MFMA kernels, sets with sequence groups only): the op is walked against its
     // own direction so that it reads the same tiles at the same time as the other ops of its set.
     int comp = 0;
+    int c0 = 0;  // first column of the C / O slice within the full rows (column halves)
     // >= 0: index (within the set) of the op whose state, transposed, is this op's state (see ProblemT::seed_from)
     int seed_from = -1;
 };
@@ -44,6 +45,17 @@ struct SetArgs {
     // two problems of the set read the same operand
     bool stream_state = false, stream_scan = false;
     int cus = 256, xcds = 8;  // CUs and XCDs of the device (placement and occupancy choices)
+    // Input preparation inside the causal forward (16-bit, one group per head): q, k, v of the ops are the raw
+    // projections; see PrepSide in cott_mfma.h for the meaning of the fields.  prep_on = false: none.
+    struct Prep {
+        bool on = false;
+        const unsigned char *keep = nullptr;
+        const float *cnt = nullptr, *sig = nullptr, *rot = nullptr;
+        long long pos0 = 0;
+        int R = 0, table_rows = 0, H = 1, dv = 0;
+        float eps = 1e-12f;
+        void *qo = nullptr, *ko = nullptr, *vo = nullptr;
+    } prep;
     hipStream_t stream;
 };
 

@@ -47,6 +47,7 @@ struct ProblemT {
     // and C are that problem's C and B, same walking order, square padded head dims): the group-state pass skips
     // it and its scan reads the other problem's slots transposed.
     int seed_from;
+    int c0;  // first column of this problem's C / O slice within the full rows (column halves)
     // Row strides of A, B and O in elements (C's is ldc) and, for each operand, where a head
     // starts: head bh is at (bh / H) * bs + (bh % H) * hs elements.  (BH,N,w) tensors have ld = w, hs = N * w,
     // bs = H * hs; (B,N,H,w) tensors, whose heads are interleaved inside a position, ld = H * w, hs = w,
@@ -91,6 +92,56 @@ struct Tiling {
     static constexpr int STATE_FLOATS = DI * DJ;
     static constexpr int OS = DJ + 8;            // ... of a staged output tile [64][DJ] (8-byte writes, 16-byte reads)
 };
+
+// ---- input preparation inside the causal forward (scan_kernel<..., PREP = true>) ------------------------
+// q, k, v are the RAW projections; every tile is prepared on its way from registers to LDS (k, v: loader
+// wavefronts) or to the MFMA operands (q: output wavefronts):
+//     q_hat = keep * rot(q) / max(|q|, eps),  k_hat likewise,  v_hat = keep * v / max(cnt ^ sig[h], 1)
+// with rot the GPT-J rotation of the first R columns by the table row of the position (row = pos0 + s, clamped to
+// the table).  The prepared rows also go to qo / ko / vo, (BH,N,D) tensors, for the backward pass.
+struct PrepSide {
+    const unsigned char *keep;  // (B,N) 0 / 1, or null
+    const float *cnt;           // (B,N) and
+    const float *sig;           // (H): value scaling, or both null
+    const float *rot;           // (table_rows, R) [sin | cos], or null
+    long long pos0;
+    int R, table_rows, H;
+    int dv;                     // full width of the value rows (a problem may own a column slice of them)
+    float eps;
+    u16 *qo, *ko, *vo;          // prepared tensors for the backward pass, or null
+};
+
+template <class TR>
+__device__ __forceinline__ void unpack8(u32x4 v, float *x) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[2 * i] = TR::to_float((u16)(v[i] & 0xffffu));
+        x[2 * i + 1] = TR::to_float((u16)(v[i] >> 16));
+    }
+}
+template <class TR>
+__device__ __forceinline__ u32x4 pack8(const float *x) {
+    return u32x4{TR::pack2(x[0], x[1]), TR::pack2(x[2], x[3]), TR::pack2(x[4], x[5]), TR::pack2(x[6], x[7])};
+}
+// the four pairs (x[2e], x[2e+1]) turned by the angles whose sines and cosines are sn[e], cs[e]
+__device__ __forceinline__ void rotate8(float *x, f32x4 sn, f32x4 cs) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float ev = x[2 * e], od = x[2 * e + 1];
+        x[2 * e] = ev * cs[e] - od * sn[e];
+        x[2 * e + 1] = od * cs[e] + ev * sn[e];
+    }
+}
+__device__ __forceinline__ int table_row(const PrepSide &ps, int s) {
+    long long t = ps.pos0 + s;
+    return (int)(t < 0 ? 0 : (t >= ps.table_rows ? ps.table_rows - 1 : t));
+}
+// keep / max(cnt ^ sig, 1) of one position (keep alone when there is no value scaling)
+__device__ __forceinline__ float value_scale(float keep, float cnt, float sig, bool scaled) {
+    if (!scaled) return keep;
+    const float p = cnt > 0.f ? __expf(sig * __logf(cnt)) : 0.f;
+    return p > 1.f ? keep * __builtin_amdgcn_rcpf(p) : keep;
+}
 
 // Workgroup -> (head, problem, group).  Linear id i runs on XCD i % xcds; per XCD the ids are ordered
 // (head block, group, problem), so the workgroups of one head and group are neighbours in the
@@ -415,6 +466,146 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
     if (so != nullptr && r.p1 > r.p0) write_out(r.p1 - 1);
 }
 
+// Loader role with the input preparation folded in (see PrepSide): same pipeline as loader_role, for THREE tiles:
+// the A rows (q) are staged here too, prepared, into sA, from where the output wavefronts take them, so that the
+// preparation stays off their per-chunk chain.  The side inputs of a chunk (keep, count, table entries; the A and
+// B tiles have the same rows and columns per thread and share the table entries) are fetched together with it, PF
+// chunks ahead, and the prepared rows are also written to qo / ko / vo.  first_half: this workgroup writes qo and ko
+// (with column halves both workgroups of a head stage the same q and k tiles).  A row of DI elements lives in
+// DI / 8 consecutive lanes, which reduce its squared norm with lane shuffles.
+template <class TR, int DI, int DJ, int PF, int LT>
+__device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B_head, const u16 *C_head, int di, int dj,
+                                                 int lda, int ldb, int ldc, const ScanRange &r, int tid, u16 *sA, u16 *sB,
+                                                 u16 *sC, const StagedOut *so, const PrepSide &ps, int bh, int c0,
+                                                 bool first_half) {
+    using TL = Tiling<DI, DJ>;
+    constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SO = kChunk * TL::OS;
+    constexpr int NB = 8 * DI / LT, NC = 8 * DJ / LT;
+    const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
+    const rsrc_t rB = make_rsrc(B_head, ((uint32_t)(r.N - 1) * ldb + di) * 2u);
+    const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
+    const uint32_t qk_bytes = first_half ? (uint32_t)r.N * di * 2u : 0u;
+    const rsrc_t rQo = make_rsrc(ps.qo ? ps.qo + (size_t)bh * r.N * di : nullptr, ps.qo ? qk_bytes : 0u);
+    const rsrc_t rKo = make_rsrc(ps.ko ? ps.ko + (size_t)bh * r.N * di : nullptr, ps.ko ? qk_bytes : 0u);
+    const rsrc_t rVo = make_rsrc(ps.vo ? ps.vo + (size_t)bh * r.N * ps.dv + c0 : nullptr,
+                                 ps.vo ? ((uint32_t)(r.N - 1) * ps.dv + dj) * 2u : 0u);
+    const size_t tok0 = (size_t)(bh / ps.H) * r.N;
+    const bool scaled = ps.cnt != nullptr && ps.sig != nullptr;
+    const float sig = scaled ? ps.sig[bh % ps.H] : 0.f;
+    auto write_out = [&](int p) {
+        const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
+        const rsrc_t rO = make_rsrc(so->O[0], ((uint32_t)(r.N - 1) * so->ld[0] + so->dj[0]) * 2u);
+        const u16 *tile = so->sO + (((p - r.p0) & 1) * 2) * SO;
+#pragma unroll
+        for (int u = 0; u < (8 * DJ + LT - 1) / LT; ++u) {
+            const int v = tid + LT * u;
+            const int row = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+            if (v < 8 * DJ) {
+                const u32x4 val = *reinterpret_cast<const u32x4 *>(tile + row * TL::OS + col);
+                const uint32_t off = (col < so->dj[0]) ? (uint32_t)((row0 + row) * so->ld[0] + col) * 2u : kOobOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(val, rO, (int)off, 0, 0);
+            }
+        }
+    };
+    u32x4 ra[PF][NB], rb[PF][NB], rc[PF][NC];
+    f32x4 sn[PF][NB], cs[PF][NB];
+    float keep_ab[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
+    auto row0_of = [&](int p) {
+        const int pc = min(p, r.p1 - 1);
+        return (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
+    };
+    auto load_chunk = [&](int s, int p) {
+        const int row0 = row0_of(p);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int v = tid + LT * u;
+            const int row = row0 + v / (DI / 8), col = (v % (DI / 8)) * 8;
+            ra[s][u] = buf_load16(rA, (uint32_t)(row * lda + col) * 2u);
+            rb[s][u] = buf_load16(rB, (uint32_t)(row * ldb + col) * 2u);
+            const int srow = min(row, r.N - 1);
+            keep_ab[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            if (ps.rot != nullptr && col < ps.R) {
+                const float *t = ps.rot + (size_t)table_row(ps, srow) * ps.R + col / 2;
+                sn[s][u] = *reinterpret_cast<const f32x4 *>(t);
+                cs[s][u] = *reinterpret_cast<const f32x4 *>(t + ps.R / 2);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NC; ++u) {
+            const int v = tid + LT * u;
+            const int row = row0 + v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+            rc[s][u] = buf_load16(rC, (uint32_t)(row * ldc + col) * 2u);
+            const int srow = min(row, r.N - 1);
+            keep_c[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            cnt_c[s][u] = scaled ? ps.cnt[tok0 + srow] : 0.f;
+        }
+    };
+    // one raw 16-byte piece of a q or k row -> rotated, normalised, masked
+    auto prep_row_piece = [&](u32x4 raw, int col, f32x4 sn_, f32x4 cs_, float keep) {
+        float x[8];
+        unpack8<TR>(raw, x);
+        if (col >= di) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = 0.f;
+        }
+        if (ps.rot != nullptr && col < ps.R) rotate8(x, sn_, cs_);
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+        for (int off = 1; off < DI / 8; off <<= 1) ss += __shfl_xor(ss, off, 64);
+        const float nrm = __builtin_amdgcn_sqrtf(ss);
+        const float mul = keep * __builtin_amdgcn_rcpf(nrm > ps.eps ? nrm : ps.eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= mul;
+        return pack8<TR>(x);
+    };
+    // registers of stage s (chunk p) -> prepared tiles in the LDS buffers ta, tb, tc and in qo / ko / vo
+    auto stage = [&](int s, int p, u16 *ta, u16 *tb, u16 *tc) {
+        const int row0 = row0_of(p);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int v = tid + LT * u;
+            const int lrow = v / (DI / 8), col = (v % (DI / 8)) * 8;
+            const u32x4 ya = prep_row_piece(ra[s][u], col, sn[s][u], cs[s][u], keep_ab[s][u]);
+            const u32x4 yb = prep_row_piece(rb[s][u], col, sn[s][u], cs[s][u], keep_ab[s][u]);
+            *reinterpret_cast<u32x4 *>(ta + lrow * TL::BS + col) = ya;
+            *reinterpret_cast<u32x4 *>(tb + lrow * TL::BS + col) = yb;
+            const uint32_t off = (col < di) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(ya, rQo, (int)off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(yb, rKo, (int)off, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < NC; ++u) {
+            const int v = tid + LT * u;
+            const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+            float x[8];
+            unpack8<TR>(rc[s][u], x);
+            const float mul = (col < dj) ? value_scale(keep_c[s][u], cnt_c[s][u], sig, scaled) : 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] *= mul;
+            const u32x4 y = (col < dj) ? pack8<TR>(x) : u32x4{0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4 *>(tc + lrow * TL::CS + col) = y;
+            const uint32_t off = (col < dj) ? (uint32_t)((row0 + lrow) * ps.dv + col) * 2u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);
+        }
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_chunk(s, r.p0 + s);
+    stage(0, r.p0, sA, sB, sC);
+    load_chunk(0, r.p0 + PF);
+    __syncthreads();
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+        const int s1 = (s + 1) % PF;
+        const int buf = (p - r.p0) & 1;
+        stage(s1, p + 1, sA + (buf ^ 1) * SB, sB + (buf ^ 1) * SB, sC + (buf ^ 1) * SC);
+        load_chunk(s1, p + 1 + PF);
+        if (so != nullptr && p > r.p0) write_out(p - 1);
+        chunk_barrier();
+    });
+    if (so != nullptr && r.p1 > r.p0) write_out(r.p1 - 1);
+}
+
 // State role (wavefront w of 4).  seed: register-native group prefix or null; sin / sout: row-major
 // fp32 hand-over states or null (sout only written when `last_group`).  sS: 16-bit copy transposed to
 // [j][i] for the A_blk S product.  TWIN: also publish the copy of the TRANSPOSED state (which is
@@ -501,10 +692,12 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
 // sOt: null = store the outputs to memory from here; else the [2 buffers] of this problem's staged output tile
 // (buffer stride 2 * 64 * OS), written with 8-byte LDS stores and sent to memory by the loader wavefronts, so that
 // this wavefront's chain of LDS reads and MFMAs never waits for the vector-memory pipeline to take a store.
-template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false>
+// PREP: the A rows are not loaded from memory here: the loader wavefronts stage them, prepared, in sA (a tile like
+// sB, double-buffered; see loader_role_prep).
+template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false>
 __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int lda, int ldc,
                                             const ScanRange &r, int blk0, int l, const u16 *sB, const u16 *sC,
-                                            const u16 *sS, u16 *sOt = nullptr) {
+                                            const u16 *sS, u16 *sOt = nullptr, const u16 *sA = nullptr) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
@@ -514,13 +707,15 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     const bool mask_rev = r.mask_rev != 0, comp = r.comp != 0;
     u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
     auto load_q = [&](int s, int p) {
-        const int pc = min(p, r.p1 - 1);
-        const int row = (reversed ? r.nchunks - 1 - pc : pc) * kChunk + 16 * blk0 + m;
+        if constexpr (!PREP) {
+            const int pc = min(p, r.p1 - 1);
+            const int row = (reversed ? r.nchunks - 1 - pc : pc) * kChunk + 16 * blk0 + m;
 #pragma unroll
-        for (int ib = 0; ib < IB; ++ib)
+            for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
-            for (int ks = 0; ks < TL::KS; ++ks)
-                qn[s][ib][ks] = buf_load16<STREAM>(rA, (uint32_t)((row + 16 * ib) * lda + 32 * ks + 8 * g) * 2u);
+                for (int ks = 0; ks < TL::KS; ++ks)
+                    qn[s][ib][ks] = buf_load16<STREAM>(rA, (uint32_t)((row + 16 * ib) * lda + 32 * ks + 8 * g) * 2u);
+        }
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_q(s, r.p0 + s);
@@ -532,11 +727,20 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
             const int buf = (p - r.p0) & 1;
             const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
             const int row0 = (reversed ? r.nchunks - 1 - p : p) * kChunk;
+            if constexpr (!PREP) {
 #pragma unroll
-            for (int ib = 0; ib < IB; ++ib)
+                for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
-                for (int ks = 0; ks < TL::KS; ++ks)
-                    qc[ib][ks] = (32 * ks + 8 * g < di) ? qn[s][ib][ks] : u32x4{0u, 0u, 0u, 0u};
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        qc[ib][ks] = (32 * ks + 8 * g < di) ? qn[s][ib][ks] : u32x4{0u, 0u, 0u, 0u};
+            } else {
+                const u16 *cA = sA + buf * SB;
+#pragma unroll
+                for (int ib = 0; ib < IB; ++ib)
+#pragma unroll
+                    for (int ks = 0; ks < TL::KS; ++ks)
+                        qc[ib][ks] = *reinterpret_cast<const u32x4 *>(cA + (16 * (blk0 + ib) + m) * TL::BS + 32 * ks + 8 * g);
+            }
             load_q(s, p + PF);
 
             // Operand fragments of the output products come in batches of JB column tiles; the reads of a batch are
@@ -635,9 +839,10 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 }
 
 // One problem per workgroup: OW output wavefronts (IB = 4/OW blocks each), 4 state, LW loader.
-template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false, bool STREAM = false>
+// PREP: q, k, v are the raw projections and are prepared inside the kernel (PrepSide; forward direction, G = 1).
+template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false, bool STREAM = false, bool PREP = false>
 __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set, int BH, int N, int nchunks,
-                                                                  int cpg, int G) {
+                                                                  int cpg, int G, PrepSide prep) {
     using TL = Tiling<DI, DJ>;
     static_assert(OW == 2 || OW == 4, "two or four output wavefronts");
     static_assert(LW == 2 || LW == 4, "two or four loader wavefronts");
@@ -651,6 +856,7 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     // STAGED: output tiles go through LDS and leave as 16-byte row segments from the loader wavefronts (StagedOut;
     // the layout has room for two tiles per buffer, this kernel uses the first)
     __shared__ __attribute__((aligned(16))) u16 sO[STAGED ? 2 * 2 * kChunk * TL::OS : 8];
+    __shared__ __attribute__((aligned(16))) u16 sA[PREP ? 2 * SB : 8];  // PREP: the prepared A rows, staged like sB
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
@@ -674,8 +880,15 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
         so.dj[1] = 0;
         so.ld[1] = 0;
         so.sO = sO;
-        loader_role<DI, DJ, PF, LT, STREAM>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
-                                            di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC, STAGED ? &so : nullptr);
+        if constexpr (PREP)
+            loader_role_prep<TR, DI, DJ, PF, LT>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
+                                                 pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh),
+                                                 pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), di, dj, pr.lda, pr.ldb, ldc,
+                                                 r, (int)threadIdx.x - 64 * (OW + 4), sA, sB, sC, STAGED ? &so : nullptr,
+                                                 prep, wi.bh, pr.c0, pr.c0 == 0);
+        else
+            loader_role<DI, DJ, PF, LT, STREAM>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
+                                                di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC, STAGED ? &so : nullptr);
     } else if (wv >= OW) {
         const float *slots = pr.seed_from >= 0 ? set.p[pr.seed_from].gstate : pr.gstate;
         state_role<TR, DI, DJ, false>(
@@ -683,9 +896,9 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
             pr.sin ? pr.sin + (size_t)wi.bh * di * pr.lds : nullptr, pr.sout ? pr.sout + (size_t)wi.bh * di * pr.lds : nullptr,
             pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS, nullptr);
     } else {
-        output_role<TR, DI, DJ, PF, IB, STREAM>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
-                                                pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r,
-                                                IB * wv, l, sB, sC, sS, STAGED ? sO : nullptr);
+        output_role<TR, DI, DJ, PF, IB, STREAM, PREP>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
+                                                      pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r,
+                                                      IB * wv, l, sB, sC, sS, STAGED ? sO : nullptr, sA);
     }
 }
 

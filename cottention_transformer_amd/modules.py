@@ -16,7 +16,7 @@ from torch import nn
 
 from . import ops
 from .autograd import (CustomAttention, CustomAttentionMergedHeads, NonCausalAttention,
-                       NonCausalAttentionMergedHeads, PrepareInputs, _autocast_target)
+                       NonCausalAttentionMergedHeads, PreparedCausalAttention, PrepareInputs, _autocast_target)
 
 
 def _autocast_on():
@@ -127,12 +127,14 @@ class GPTCosAttention(nn.Module):
         return query, key
 
     def _cos_attn(self, query, key, value, attention_mask=None, head_mask=None, rotary=None, bnhd=False,
-                  merge_heads=False):
+                  merge_heads=False, first_position=None):
         """GPTCosAttention.py:161-282.  query, key, value: (B,H,S,D), already rotated -- or, with `bnhd`, (B,S,H,D)
         as the projections produce them, with rotary=(table, position_ids) still to be applied; in that case the
         rotation, the head permute and the preparation steps are one fused pass.
         merge_heads: the caller wants the output as (B,S,H,D) (:500); returned that way, with None in place of
-        the second value, when the training path can write it directly, else (B,H,S,D) as usual."""
+        the second value, when the training path can write it directly, else (B,H,S,D) as usual.
+        first_position: the positions are first_position, first_position + 1, ... (the caller made them itself); the
+        preparation then runs inside the attention kernel where that is built."""
         if bnhd:
             b, s, h, _ = query.shape
         else:
@@ -156,8 +158,15 @@ class GPTCosAttention(nn.Module):
                 out, self.state = ops.causal_prefill(q, k, v, state=self.state)
             self.cur_s += s
             return out, out
-        cnt = keep.to(torch.float32).cumsum(-1)                        # kept keys at positions <= s (:228)
+        cnt = keep.to(torch.float32).cumsum(-1)                        # kept keys at positions <= s (:241)
         dt = _autocast_target(query)
+        if (bnhd and first_position is not None and merge_heads and query.dtype == dt
+                and ops.fused_preparation_supported(dt, b, h, s, query.shape[-1], value.shape[-1],
+                                                    0 if table is None else table.shape[-1])
+                and ops.merged_heads_supported(dt, s, h, query.shape[-1], value.shape[-1])):
+            # one forward launch: rotation, normalisation, value scaling, mask and the attention op
+            return PreparedCausalAttention.apply(query, key, value, None if attention_mask is None else keep, cnt, sig,
+                                                 table, first_position, True, True), None
         q, k, v = PrepareInputs.apply(query, key, value, keep, cnt, sig, dt, table, pos, bnhd)
         if merge_heads and ops.merged_heads_supported(q.dtype, s, h, q.shape[-1], v.shape[-1]):
             return CustomAttentionMergedHeads.apply(q, k, v), None
@@ -177,10 +186,12 @@ class GPTCosAttention(nn.Module):
             if not _autocast_on():
                 attn_output = attn_output.to(hidden_states.dtype)
             return (self.resid_dropout(self.out_proj(attn_output)), None)
+        first_position = None
         if position_ids is None:
             start = self.cur_s - 1 if self.fast_inference else 0
             position_ids = torch.arange(start, start + hidden_states.shape[1], device=hidden_states.device)
             position_ids = position_ids[None, :].expand(hidden_states.shape[0], -1)
+            first_position = start
         if layer_past is None and use_cache is not True and self.rotary_dim is not None and self.rotary_dim % 4 == 0:
             # nobody needs the rotated keys themselves: rotation, head permute and preparation in one pass
             table = self.embed_positions
@@ -189,7 +200,7 @@ class GPTCosAttention(nn.Module):
             present = None
             attn_output, attn_weights = self._cos_attn(query, key, value, attention_mask, head_mask,
                                                        rotary=(table, position_ids), bnhd=True,
-                                                       merge_heads=not output_attentions)
+                                                       merge_heads=not output_attentions, first_position=first_position)
         else:
             query, key = self._rotate(query, key, position_ids)
             key, query, value = key.permute(0, 2, 1, 3), query.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3)

@@ -133,6 +133,61 @@ def causal_dot_product(q, k, v, reversed=False, merged_heads=False):
     return o
 
 
+_prep_supported_cache = {}
+
+
+def fused_preparation_supported(dtype, b, h, n, dk, dv, rotary_dim=0):
+    """Whether causal_dot_product_prepared has a kernel for the shape: bf16 / fp16, head dims 32..128 in steps of 16,
+    a rotary width that is a multiple of 8, enough heads that no head is cut into sequence groups, and not the
+    undivided 128 x 128 tiles (cott_causal_fwd_prep_supported)."""
+    if dtype not in (torch.bfloat16, torch.float16):
+        return False
+    key = (dtype, b, h, n, dk, dv, rotary_dim)
+    ok = _prep_supported_cache.get(key)
+    if ok is None:
+        ok = _prep_supported_cache[key] = bool(
+            _loader.lib().cott_causal_fwd_prep_supported(b, h, n, dk, dv, _DTYPES[dtype], rotary_dim))
+    return ok
+
+
+def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=None, bnhd=False, merged_heads=False,
+                                want_prepared=True):
+    """Causal forward on the RAW projections q, k, v: rotation, normalisation, value scaling and masking
+    (prepare_inputs) happen inside the attention kernel (GPT_Trainer/GPTCosAttention.py:229-248, 462-476 in front
+    of :282 as one launch).  rotary = (table (P,R) fp32, first position): the table row of position s is
+    first position + s.  bnhd: q, k, v are (B,N,H,D); merged_heads: o is returned as (B,N,H,Dv).
+    Returns (o, (q_hat, k_hat, v_hat)) with the prepared tensors (B,H,N,D) that the backward pass needs, or
+    (o, None) when want_prepared is false.  Raises where fused_preparation_supported() is false."""
+    _require_gpu(Q=q, K=k, V=v)
+    b, h, n, dk, dv = _prep_shapes(q, k, v, bnhd)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("Q, K and V must have the same dtype")
+    code = _dtype_code(q)
+    keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
+    table, pos0, rdim, rows = None, 0, 0, 0
+    if rotary is not None:
+        table, pos0 = rotary
+        if table.dim() != 2 or table.size(1) % 8 != 0 or table.size(1) > dk:
+            raise RuntimeError("rotary table must be (positions, rotary_dim), rotary_dim a multiple of 8 and <= Dk")
+        table = table.to(device=q.device, dtype=torch.float32).contiguous()
+        rows, rdim = table.shape
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    o = torch.empty((b, n, h, dv) if merged_heads else (b, h, n, dv), dtype=q.dtype, device=q.device)
+    prepared = None
+    if want_prepared:
+        prepared = (torch.empty((b, h, n, dk), dtype=q.dtype, device=q.device),
+                    torch.empty((b, h, n, dk), dtype=q.dtype, device=q.device),
+                    torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device))
+    L = _loader.lib()
+    with _on(q.device):
+        rc = L.cott_causal_fwd_prep(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                    *((t.data_ptr() for t in prepared) if prepared else (None, None, None)),
+                                    _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), int(pos0), rdim, rows, int(bool(bnhd)),
+                                    int(bool(merged_heads)), b, h, n, dk, dv, code, _stream(q.device))
+    _check(rc, "cott_causal_fwd_prep")
+    return o, prepared
+
+
 def causal_prefill(q, k, v, state=None, return_state=True):
     """Causal forward over a whole prompt (or one piece of a sequence) with the recurrence state handed over:
     returns (o, state_out) with o[s] = q[s] (state + sum_{s'<=s} k[s'] v[s']^T) and

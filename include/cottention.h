@@ -195,6 +195,28 @@ COTT_API int cott_prep_ex_bwd(const void *q, const void *k, const void *v,
                      const float *rot_table, const long long *pos, int rotary_dim, int table_rows, int in_bnhd,
                      int B, int H, int N, int Dk, int Dv, int in_dtype, int grad_dtype, void *stream);
 
+/* ---- causal forward on the RAW projections: the input preparation inside the attention kernel ------------
+ *   o = cott_causal_fwd(q_hat, k_hat, v_hat)  with
+ *   q_hat = keep * rot(q) / max(|rot(q)|, 1e-12),  k_hat likewise,  v_hat = keep * v / max(cnt^sig[h], 1)
+ * in ONE launch: the rows are rotated, normalised, scaled and masked on their way into the kernel's tiles, so the
+ * separate pass of cott_prep_ex_fwd (one read and one write of q, k, v) disappears from the forward of the block
+ * (GPT_Trainer/GPTCosAttention.py:229-248 normalise / scale / mask and :462-476 rotary, in front of :282).
+ * q_out, k_out, v_out: (B,H,N,D) receive q_hat, k_hat, v_hat for the backward pass (cott_causal_bwd on them, then
+ * cott_prep_ex_bwd); any of them may be NULL.  keep, cnt, sig as in cott_prep_fwd.  rot_table: (table_rows,
+ * rotary_dim) fp32 as in cott_prep_ex_fwd, rotary_dim a multiple of 8, or NULL; the table row of position s is
+ * pos0 + s (clamped to the table): positions that are not consecutive take cott_prep_ex_fwd.  in_bnhd: q, k, v
+ * are (B,N,H,D); o_bnhd: o is (B,N,H,Dv).  bf16 / fp16, head dims 32..128 in steps of 16, B*H large enough that a
+ * head is not cut into sequence groups, and not the undivided 128 x 128 tiles (no room in LDS for the prepared q
+ * tile): cott_causal_fwd_prep_supported() says (1 / 0) whether a shape qualifies; otherwise the call returns
+ * COTT_ERR_UNSUPPORTED and the caller prepares the inputs with cott_prep_ex_fwd.  Needs no workspace. */
+COTT_API int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim);
+COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o,
+                         void *q_out, void *k_out, void *v_out,
+                         const unsigned char *keep, const float *cnt, const float *sig,
+                         const float *rot_table, long long pos0, int rotary_dim, int table_rows,
+                         int in_bnhd, int o_bnhd,
+                         int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
+
 /* ---- per-kernel timing -----------------------------------------------------------------------
  * While enabled, every kernel launch made by the entry points above is bracketed by a pair of HIP
  * events on the launch stream (this is the one place the library creates HIP objects).

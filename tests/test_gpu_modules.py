@@ -76,6 +76,43 @@ def test_gpt_block_forward_backward(mods, autocast):
         assert rel_l2(a.float(), r.numpy()) <= tol, name
 
 
+@pytest.mark.parametrize("masked", [False, True], ids=["no-mask", "masked"])
+def test_gpt_block_with_the_preparation_inside_the_attention_kernel(mods, masked):
+    """Enough heads that no head is cut into sequence groups, bf16 autocast, positions made by the block itself: the
+    forward of the block then runs rotation, normalisation, value scaling, mask and attention as one launch
+    (PreparedCausalAttention).  Same check as above, against the fp64 CPU statement of the block."""
+    from unittest import mock
+    from oracle import torch_forms as tf
+    from cottention_transformer_amd import ops
+    say("gpt block, fused preparation", masked)
+    torch.manual_seed(0)
+    cfg = gpt_cfg(e=1024, heads=16, rot=32, max_pos=256)
+    m = mods.GPTCosAttention(cfg).to(DEV)
+    with torch.no_grad():
+        m.norm_const.copy_(torch.linspace(-1.0, 1.0, 16).reshape(1, 16, 1, 1))
+    b, s = 16, 136
+    g = torch.Generator().manual_seed(2)
+    hidden = torch.randn(b, s, cfg.hidden_size, generator=g)
+    keep = (torch.rand(b, s, generator=g) > 0.15) if masked else torch.ones(b, s, dtype=torch.bool)
+    gout = torch.randn(b, s, cfg.hidden_size, generator=g)
+    w = [getattr(m, n).weight.detach().double().cpu().requires_grad_(True) for n in ("q_proj", "k_proj", "v_proj", "out_proj")]
+    nc = m.norm_const.detach().double().cpu().reshape(-1).requires_grad_(True)
+    h64 = hidden.double().requires_grad_(True)
+    ref = tf.gpt_attention_block(h64, *w, nc, cfg.num_attention_heads, cfg.rotary_dim, cfg.max_position_embeddings, keep)
+    ref_grads = torch.autograd.grad(ref, [h64, *w, nc], gout.double())
+    hd = hidden.to(DEV).requires_grad_(True)
+    with mock.patch.object(ops, "causal_dot_product_prepared", wraps=ops.causal_dot_product_prepared) as spy:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, present = m(hd, attention_mask=additive_mask(keep).to(DEV) if masked else None)
+        assert spy.call_count == 1, "the fused forward was not taken"
+    assert rel_l2(out.float(), ref.detach().numpy()) <= 3e-2
+    out.backward(gout.to(DEV).to(out.dtype))
+    got = [hd.grad, m.q_proj.weight.grad, m.k_proj.weight.grad, m.v_proj.weight.grad, m.out_proj.weight.grad,
+           m.norm_const.grad.reshape(-1)]
+    for name, a, r in zip(("hidden", "wq", "wk", "wv", "wo", "norm_const"), got, ref_grads):
+        assert rel_l2(a.float(), r.numpy()) <= 3e-2, name
+
+
 def test_gpt_block_recurrent_inference(mods):
     # GPTCosAttention.py:77-87,234-236,253-272: a prompt, then single tokens, against the per-token loop on the CPU
     from oracle import torch_forms as tf

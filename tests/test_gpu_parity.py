@@ -617,3 +617,85 @@ def test_calls_can_be_captured_in_a_hip_graph_and_replayed(ct, oracle):
         assert torch.equal(o, want_o), f"replay {rep}"
         for got, want in zip((dq, dk, dv), want_g):
             assert torch.equal(got, want), f"replay {rep}"
+
+
+FUSED_PREP_CASES = [
+    # b, h, n, dk, dv, dtype, rotary_dim, projections' layout, masked   launch form
+    (8, 16, 256, 64, 64, BF, 64, True, True),      # two column halves per head, outputs staged through LDS
+    (8, 16, 130, 128, 128, BF, 64, True, True),    # 128-wide heads in column halves, rotation of half of the columns
+    (32, 16, 200, 48, 80, HF, 32, False, True),    # padded head dims, two workgroups per CU
+    (16, 16, 63, 32, 64, BF, 0, False, False),     # no rotation, no mask, a single partial chunk
+    (8, 32, 1000, 64, 64, HF, 16, True, True),     # several chunks, ragged tail
+]
+
+
+@pytest.mark.parametrize("case", FUSED_PREP_CASES,
+                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1] + f"-rot{c[6]}")
+def test_input_preparation_inside_the_forward_kernel(ct, oracle, case):
+    """cott_causal_fwd_prep: rotary, normalisation, value scaling and mask inside the causal forward kernel
+    (GPT_Trainer/GPTCosAttention.py:229-248, 462-476, 282 as one launch) against the CPU statements of those steps
+    (oracle/torch_forms.py) followed by the causal oracle; the prepared tensors it leaves for the backward pass
+    against the same statements; and the autograd function built on it against autograd through the CPU forms."""
+    from oracle import torch_forms as tf
+    b, h, n, dk, dv, dt, rdim, bnhd, masked = case
+    say("fused preparation", case)
+    assert ct.fused_preparation_supported(dt, b, h, n, dk, dv, rdim)
+    g = torch.Generator().manual_seed(n + dk + rdim)
+    shape = (lambda d: (b, n, h, d)) if bnhd else (lambda d: (b, h, n, d))
+    q, k, v = (torch.randn(shape(d), generator=g).to(dt) for d in (dk, dk, dv))
+    keep = (torch.rand(b, n, generator=g) > 0.2) if masked else None
+    sig = torch.sigmoid(torch.randn(h, generator=g))
+    go = torch.randn(b, h, n, dv, generator=g).to(dt)
+    pos0 = 5
+    table = tf.gptj_sinusoid_table(n + 40, rdim).float() if rdim else None
+    # CPU reference in fp64, (B,H,N,D)
+    q64, k64, v64, s64 = (t.double().requires_grad_(True) for t in (q, k, v, sig))
+    qh, kh, vh = ((t.permute(0, 2, 1, 3) if bnhd else t) for t in (q64, k64, v64))
+    if rdim:
+        sin, cos = torch.split(table.double()[pos0:pos0 + n][None].expand(b, n, rdim), rdim // 2, dim=-1)
+        rot = lambda x: torch.cat([tf.gptj_rotate(x.permute(0, 2, 1, 3)[..., :rdim], sin, cos).permute(0, 2, 1, 3),
+                                   x[..., rdim:]], -1)
+        qh, kh = rot(qh), rot(kh)
+    rq, rk, rv, cnt = tf.input_prep_gpt(qh, kh, vh, keep, s64)
+    ro = tf.causal_cumsum(rq, rk, rv) if n <= 300 else None
+    ref_o = oracle.causal(rq.detach(), rk.detach(), rv.detach())
+    # the kernel
+    args = dict(keep=None if keep is None else keep.to(DEV), cnt=cnt.float().to(DEV), sig=sig.to(DEV),
+                rotary=(table.to(DEV), pos0) if rdim else None, bnhd=bnhd)
+    for merged in (False, True):
+        o, prepared = ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV), merged_heads=merged, **args)
+        assert o.shape == ((b, n, h, dv) if merged else (b, h, n, dv)) and o.dtype == dt
+        assert rel_l2(o.permute(0, 2, 1, 3) if merged else o, ref_o) <= TOL[dt], merged
+        for name, got, ref in zip("qkv", prepared, (rq, rk, rv)):
+            assert got.shape == ref.shape and rel_l2(got, ref.detach().numpy()) <= TOL[dt], name
+        if keep is not None:
+            assert torch.all(prepared[0][~keep.to(DEV)[:, None, :].expand(b, h, n)] == 0)
+    # the same numbers as the two-kernel path on the same prepared operands (the products are the same code)
+    o2 = ct.causal_dot_product(*prepared)
+    assert rel_l2(o2, o.permute(0, 2, 1, 3).double().cpu().numpy()) <= 1e-2
+    o_np, none = ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV), want_prepared=False, **args)
+    assert none is None and rel_l2(o_np, ref_o) <= TOL[dt]
+    if ro is None:
+        return
+    # gradients through the autograd function
+    ref_grads = torch.autograd.grad(ro, [q64, k64, v64, s64], go.double())
+    qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sig))
+    out = ct.PreparedCausalAttention.apply(qd, kd, vd, args["keep"], args["cnt"], sd, table.to(DEV) if rdim else None, pos0,
+                                           bnhd, False)
+    assert rel_l2(out, ref_o) <= TOL[dt]
+    out.backward(go.to(DEV))
+    for name, got, ref in zip(("dq", "dk", "dv", "dsig"), (qd.grad, kd.grad, vd.grad, sd.grad), ref_grads):
+        assert got.shape == ref.shape and rel_l2(got, ref.numpy()) <= 2e-2, name
+
+
+def test_fused_preparation_is_refused_where_not_built(ct):
+    assert not ct.fused_preparation_supported(F32, 8, 16, 256, 64, 64)
+    assert not ct.fused_preparation_supported(BF, 1, 2, 4096, 64, 64)        # few heads: sequence groups
+    assert not ct.fused_preparation_supported(BF, 8, 16, 256, 64, 64, 12)    # rotary width not a multiple of 8
+    assert not ct.fused_preparation_supported(BF, 16, 16, 130, 128, 128)     # undivided 128 x 128 tiles
+    q, k, v, _ = inputs(1, 2, 4096, 64, 64, BF, seed=1)
+    with pytest.raises(RuntimeError, match="one group per head"):
+        ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV))
+    q, k, v, _ = inputs(8, 16, 64, 64, 64, F32, seed=1)
+    with pytest.raises(RuntimeError, match="bf16 / fp16"):
+        ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV))
