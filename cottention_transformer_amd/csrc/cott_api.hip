@@ -152,7 +152,8 @@ bool pair_enabled() {
 bool pair_eligible(const Op *ops, int n, int dtype, bool causal) {
     if (!pair_enabled() || !causal || n != 3 || !(dtype == COTT_F16 || dtype == COTT_BF16)) return false;
     const Op &x = ops[1], &y = ops[2];
-    if (!(x.B == y.C && x.C == y.B && x.reversed == y.reversed && x.di == y.dj && x.dj == y.di)) return false;
+    // (both sum over the future: the pair workgroups leave out the score tiles on the other side of the diagonal)
+    if (!(x.B == y.C && x.C == y.B && x.reversed == 1 && y.reversed == 1 && x.di == y.dj && x.dj == y.di)) return false;
     const int pd = cott::mfma_pad(ops[0].di);
     if (pd > 64) return false;
     for (int i = 0; i < 3; ++i)

@@ -694,13 +694,22 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
 // this wavefront's chain of LDS reads and MFMAs never waits for the vector-memory pipeline to take a store.
 // PREP: the A rows are not loaded from memory here: the loader wavefronts stage them, prepared, in sA (a tile like
 // sB, double-buffered; see loader_role_prep).
-template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false>
+// SKIP != 0 (two blocks per wavefront, mask on the side of the future, no complement form): the wavefront owns the
+// blocks {0, 3} (SKIP = 1) or {1, 2} (SKIP = 2) of a chunk instead of two neighbours, and leaves out the score tiles
+// that lie entirely on the masked side of the diagonal together with the products that would only see their zeros:
+// 5 of 8 score tiles and 3 of 4 steps of the score-times-C products remain for either wavefront.
+template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false, int SKIP = 0>
 __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int lda, int ldc,
                                             const ScanRange &r, int blk0, int l, const u16 *sB, const u16 *sC,
                                             const u16 *sS, u16 *sOt = nullptr, const u16 *sA = nullptr) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
+    static_assert(SKIP == 0 || IB == 2, "block pairing needs two blocks per wavefront");
+    // block (16 positions of the chunk) number `ib` of this wavefront; whether its score tile against key tile jt
+    // can hold anything (SKIP: keys >= queries are kept)
+    auto blk = [&](int ib) { return SKIP == 0 ? blk0 + ib : (SKIP == 1 ? (ib == 0 ? 0 : 3) : (ib == 0 ? 1 : 2)); };
+    auto live = [&](int ib, int jt) { return SKIP == 0 || jt >= blk(ib); };
     const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
     const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     const int reversed = r.reversed;
@@ -709,12 +718,12 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     auto load_q = [&](int s, int p) {
         if constexpr (!PREP) {
             const int pc = min(p, r.p1 - 1);
-            const int row = (reversed ? r.nchunks - 1 - pc : pc) * kChunk + 16 * blk0 + m;
+            const int row = (reversed ? r.nchunks - 1 - pc : pc) * kChunk + m;
 #pragma unroll
             for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
                 for (int ks = 0; ks < TL::KS; ++ks)
-                    qn[s][ib][ks] = buf_load16<STREAM>(rA, (uint32_t)((row + 16 * ib) * lda + 32 * ks + 8 * g) * 2u);
+                    qn[s][ib][ks] = buf_load16<STREAM>(rA, (uint32_t)((row + 16 * blk(ib)) * lda + 32 * ks + 8 * g) * 2u);
         }
     };
 #pragma unroll
@@ -739,7 +748,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                 for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
                     for (int ks = 0; ks < TL::KS; ++ks)
-                        qc[ib][ks] = *reinterpret_cast<const u32x4 *>(cA + (16 * (blk0 + ib) + m) * TL::BS + 32 * ks + 8 * g);
+                        qc[ib][ks] = *reinterpret_cast<const u32x4 *>(cA + (16 * blk(ib) + m) * TL::BS + 32 * ks + 8 * g);
             }
             load_q(s, p + PF);
 
@@ -770,19 +779,25 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
             {
                 u32x4 kf[4][TL::KS];
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt)
+                for (int jt = 0; jt < 4; ++jt) {
+                    if (!(live(0, jt) || live(IB - 1, jt))) continue;
 #pragma unroll
                     for (int ks = 0; ks < TL::KS; ++ks)
                         kf[jt][ks] = *reinterpret_cast<const u32x4 *>(cB + (16 * jt + m) * TL::BS + 32 * ks + 8 * g);
+                }
                 read_batch(0, 0);
 #pragma unroll
                 for (int ib = 0; ib < IB; ++ib)
 #pragma unroll
                     for (int jt = 0; jt < 4; ++jt) {
+                        if (!live(ib, jt)) {
+                            pk[ib][jt] = u32x2{0u, 0u};
+                            continue;
+                        }
                         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int ks = 0; ks < TL::KS; ++ks) acc = TR::mfma(kf[jt][ks], qc[ib][ks], acc);
-                        const int d0 = 16 * (jt - (blk0 + ib)) + 4 * g - m;  // key pos - query pos at element 0
+                        const int d0 = 16 * (jt - blk(ib)) + 4 * g - m;  // key pos - query pos at element 0
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
                             const bool keep = mask_rev ? (d0 + q >= 0) : (d0 + q <= 0);
@@ -792,7 +807,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                     }
             }
 
-            const int orow = row0 + 16 * blk0 + m;
+            const int orow = row0 + m;
 #pragma unroll
             for (int bt = 0; bt < NBATCH; ++bt) {
                 const int j0 = bt * JB, slot = bt & 1;
@@ -809,7 +824,8 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                         f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int kb = 0; kb < 2; ++kb)
-                            o = TR::mfma(vf[slot][jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
+                            if (live(ib, 2 * kb) || live(ib, 2 * kb + 1))
+                                o = TR::mfma(vf[slot][jj][kb], cat(pk[ib][2 * kb], pk[ib][2 * kb + 1]), o);
                         if constexpr (TL::KS >= 4) {
                             f32x4 o2 = {0.f, 0.f, 0.f, 0.f}, o3 = o2;
 #pragma unroll
@@ -826,9 +842,9 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                         const u32x2 val = {TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
                         if (sOt != nullptr) {
                             *reinterpret_cast<u32x2 *>(sOt + buf * (2 * kChunk * TL::OS) +
-                                                       (16 * (blk0 + ib) + m) * TL::OS + col) = val;
+                                                       (16 * blk(ib) + m) * TL::OS + col) = val;
                         } else {
-                            const uint32_t off = (col < dj) ? (uint32_t)((orow + 16 * ib) * ldc + col) * 2u : kOobOffset;
+                            const uint32_t off = (col < dj) ? (uint32_t)((orow + 16 * blk(ib)) * ldc + col) * 2u : kOobOffset;
                             buf_store8(rO, off, val);
                         }
                     }
@@ -967,13 +983,27 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
             for (int p = r.p0 - 1; p < r.p1; ++p) __syncthreads();  // idle: keep the barrier count
         }
     } else if (wv < OWP) {
-        output_role<TR, D, D, PF, IBP>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r,
-                                       IBP * wv, l, sB, sC, sS, sO);
+        const u16 *A_head = pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh);
+        if constexpr (IBP == 2) {  // the pair sums over the future: blocks {0, 3} and {1, 2}, dead score tiles left out
+            if (wv == 0)
+                output_role<TR, D, D, PF, 2, false, false, 1>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS, sO);
+            else
+                output_role<TR, D, D, PF, 2, false, false, 2>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS, sO);
+        } else {
+            output_role<TR, D, D, PF, IBP>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, IBP * wv, l, sB, sC, sS, sO);
+        }
     } else {
         // Y: contracted dim dj of X, output dim di of X; its row-read tile is X's C tile and vice versa
         // the second problem's own operands (A2, O2) are plain (BH,N,w) tensors
-        output_role<TR, D, D, PF, IBP>(pr.A2 + (size_t)wi.bh * N * dj, nullptr, dj, di, dj, di, r, IBP * (wv - OWP), l, sC,
-                                       sB, sS2, sO + SO);
+        const u16 *A_head = pr.A2 + (size_t)wi.bh * N * dj;
+        if constexpr (IBP == 2) {
+            if (wv == OWP)
+                output_role<TR, D, D, PF, 2, false, false, 1>(A_head, nullptr, dj, di, dj, di, r, 0, l, sC, sB, sS2, sO + SO);
+            else
+                output_role<TR, D, D, PF, 2, false, false, 2>(A_head, nullptr, dj, di, dj, di, r, 0, l, sC, sB, sS2, sO + SO);
+        } else {
+            output_role<TR, D, D, PF, IBP>(A_head, nullptr, dj, di, dj, di, r, IBP * (wv - OWP), l, sC, sB, sS2, sO + SO);
+        }
     }
 }
 
