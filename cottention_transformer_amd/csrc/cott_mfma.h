@@ -608,12 +608,12 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
 
 // State role (wavefront w of 4).  seed: register-native group prefix or null; sin / sout: row-major
 // fp32 hand-over states or null (sout only written when `last_group`).  sS: 16-bit copy transposed to
-// [j][i] for the A_blk S product.  TWIN: also publish the copy of the TRANSPOSED state (which is
-// [i][j] of this one) in sS2, for a second problem whose B and C are this problem's C and B.
-template <class TR, int DI, int DJ, bool TWIN>
+// [j][i] for the A_blk S product (a twin problem whose B and C are this problem's C and B reads the same copy
+// transposed, see output_role).
+template <class TR, int DI, int DJ>
 __device__ __forceinline__ void state_role(const float *seed, bool seed_transposed, const float *sin, float *sout, int lds, bool last_group,
                                            int di, int dj, const ScanRange &r, int w, int l, const u16 *sB,
-                                           const u16 *sC, u16 *sS, u16 *sS2) {
+                                           const u16 *sC, u16 *sS) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
@@ -650,27 +650,21 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
                 if (i0 + q < di && j < dj) S[u][q] += sin[(size_t)(i0 + q) * lds + j];
         }
     }
-    auto put_state = [&](u16 *dst, u16 *dst2) {
+    auto put_state = [&](u16 *dst) {
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) {
             const int t = w * TL::TPW + u;
             const int it = t / TL::NJT, jt = t % TL::NJT;
             u32x2 pk = {TR::pack2(S[u][0], S[u][1]), TR::pack2(S[u][2], S[u][3])};
             *reinterpret_cast<u32x2 *>(dst + (16 * jt + m) * TL::SS + 16 * it + 4 * g) = pk;
-            if (TWIN) {
-                dst2[(16 * it + 4 * g + 0) * TL::SS + 16 * jt + m] = (u16)(pk.x & 0xffffu);
-                dst2[(16 * it + 4 * g + 1) * TL::SS + 16 * jt + m] = (u16)(pk.x >> 16);
-                dst2[(16 * it + 4 * g + 2) * TL::SS + 16 * jt + m] = (u16)(pk.y & 0xffffu);
-                dst2[(16 * it + 4 * g + 3) * TL::SS + 16 * jt + m] = (u16)(pk.y >> 16);
-            }
         }
     };
-    put_state(sS, sS2);
+    put_state(sS);
     __syncthreads();
     for (int p = r.p0; p < r.p1; ++p) {
         const int buf = (p - r.p0) & 1;
         state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m, r.comp ? 0x80008000u : 0u);
-        put_state(sS + (buf ^ 1) * SSZ, sS2 + (buf ^ 1) * SSZ);
+        put_state(sS + (buf ^ 1) * SSZ);
         __syncthreads();
     }
     if (sout != nullptr && last_group) {
@@ -698,7 +692,9 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
 // blocks {0, 3} (SKIP = 1) or {1, 2} (SKIP = 2) of a chunk instead of two neighbours, and leaves out the score tiles
 // that lie entirely on the masked side of the diagonal together with the products that would only see their zeros:
 // 5 of 8 score tiles and 3 of 4 steps of the score-times-C products remain for either wavefront.
-template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false, int SKIP = 0>
+// TRS: sS holds the 16-bit copy of the TRANSPOSE of this problem's state (the copy published for a twin problem whose
+// B and C are this problem's C and B); it is then read with transposing LDS reads.
+template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false, int SKIP = 0, bool TRS = false>
 __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int lda, int ldc,
                                             const ScanRange &r, int blk0, int l, const u16 *sB, const u16 *sC,
                                             const u16 *sS, u16 *sOt = nullptr, const u16 *sA = nullptr) {
@@ -769,7 +765,9 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
 #pragma unroll
                     for (int ks = 0; ks < TL::KS; ++ks)
                         sf[slot][jj][ks] =
-                            *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
+                            TRS ? cat(lds_col4(cS, TL::SS, 32 * ks + 8 * g, 16 * jt, m),
+                                      lds_col4(cS, TL::SS, 32 * ks + 8 * g + 4, 16 * jt, m))
+                                : *reinterpret_cast<const u32x4 *>(cS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
                 }
             };
 
@@ -907,10 +905,10 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
                                                 di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC, STAGED ? &so : nullptr);
     } else if (wv >= OW) {
         const float *slots = pr.seed_from >= 0 ? set.p[pr.seed_from].gstate : pr.gstate;
-        state_role<TR, DI, DJ, false>(
+        state_role<TR, DI, DJ>(
             slots ? slots + ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS : nullptr, pr.seed_from >= 0,
             pr.sin ? pr.sin + (size_t)wi.bh * di * pr.lds : nullptr, pr.sout ? pr.sout + (size_t)wi.bh * di * pr.lds : nullptr,
-            pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS, nullptr);
+            pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS);
     } else {
         output_role<TR, DI, DJ, PF, IB, STREAM, PREP>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
                                                       pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r,
@@ -940,7 +938,6 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
     __shared__ __attribute__((aligned(16))) u16 sS[2 * SSZ];
-    __shared__ __attribute__((aligned(16))) u16 sS2[2 * SSZ];
     __shared__ __attribute__((aligned(16))) u16 sO[2 * 2 * kChunk * TL::OS];
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -971,10 +968,8 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
         loader_role<D, D, PF, LT>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
                                   di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (NOUT + 4), sB, sC, &so);
     } else if (wv >= NOUT) {
-        if (pair)
-            state_role<TR, D, D, true>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, sS2);
-        else
-            state_role<TR, D, D, false>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, nullptr);
+        // one 16-bit copy of the state serves both problems of a pair: the second reads it transposed
+        state_role<TR, D, D>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS);
     } else if (!pair) {
         if (wv < 4) {
             output_role<TR, D, D, PF, 1>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r,
@@ -998,11 +993,12 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
         const u16 *A_head = pr.A2 + (size_t)wi.bh * N * dj;
         if constexpr (IBP == 2) {
             if (wv == OWP)
-                output_role<TR, D, D, PF, 2, false, false, 1>(A_head, nullptr, dj, di, dj, di, r, 0, l, sC, sB, sS2, sO + SO);
+                output_role<TR, D, D, PF, 2, false, false, 1, true>(A_head, nullptr, dj, di, dj, di, r, 0, l, sC, sB, sS, sO + SO);
             else
-                output_role<TR, D, D, PF, 2, false, false, 2>(A_head, nullptr, dj, di, dj, di, r, 0, l, sC, sB, sS2, sO + SO);
+                output_role<TR, D, D, PF, 2, false, false, 2, true>(A_head, nullptr, dj, di, dj, di, r, 0, l, sC, sB, sS, sO + SO);
         } else {
-            output_role<TR, D, D, PF, IBP>(A_head, nullptr, dj, di, dj, di, r, IBP * (wv - OWP), l, sC, sB, sS2, sO + SO);
+            output_role<TR, D, D, PF, IBP, false, false, 0, true>(A_head, nullptr, dj, di, dj, di, r, IBP * (wv - OWP), l, sC,
+                                                                  sB, sS, sO + SO);
         }
     }
 }
