@@ -688,10 +688,12 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
 // this wavefront's chain of LDS reads and MFMAs never waits for the vector-memory pipeline to take a store.
 // PREP: the A rows are not loaded from memory here: the loader wavefronts stage them, prepared, in sA (a tile like
 // sB, double-buffered; see loader_role_prep).
-// SKIP != 0 (two blocks per wavefront, mask on the side of the future, no complement form): the wavefront owns the
-// blocks {0, 3} (SKIP = 1) or {1, 2} (SKIP = 2) of a chunk instead of two neighbours, and leaves out the score tiles
-// that lie entirely on the masked side of the diagonal together with the products that would only see their zeros:
-// 5 of 8 score tiles and 3 of 4 steps of the score-times-C products remain for either wavefront.
+// SKIP != 0 (two blocks per wavefront): the wavefront owns the blocks {0, 3} (SKIP = 1, 3) or {1, 2} (SKIP = 2, 4) of
+// a chunk instead of two neighbours, and leaves out the score tiles that lie entirely on the masked side of the
+// diagonal together with the products that would only see their zeros: 5 of 8 score tiles and 3 of 4 steps of the
+// score-times-C products remain for either wavefront.  SKIP = 1, 2: the scores of keys at or after the query are the
+// ones that count (ops that sum over the future, or over the past in complement form); SKIP = 3, 4: those of keys
+// at or before it.  The caller picks the variant that matches the problem's mask.
 // TRS: sS holds the 16-bit copy of the TRANSPOSE of this problem's state (the copy published for a twin problem whose
 // B and C are this problem's C and B); it is then read with transposing LDS reads.
 template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false, int SKIP = 0, bool TRS = false>
@@ -704,8 +706,8 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     static_assert(SKIP == 0 || IB == 2, "block pairing needs two blocks per wavefront");
     // block (16 positions of the chunk) number `ib` of this wavefront; whether its score tile against key tile jt
     // can hold anything (SKIP: keys >= queries are kept)
-    auto blk = [&](int ib) { return SKIP == 0 ? blk0 + ib : (SKIP == 1 ? (ib == 0 ? 0 : 3) : (ib == 0 ? 1 : 2)); };
-    auto live = [&](int ib, int jt) { return SKIP == 0 || jt >= blk(ib); };
+    auto blk = [&](int ib) { return SKIP == 0 ? blk0 + ib : ((SKIP & 1) ? (ib == 0 ? 0 : 3) : (ib == 0 ? 1 : 2)); };
+    auto live = [&](int ib, int jt) { return SKIP == 0 || (SKIP <= 2 ? jt >= blk(ib) : jt <= blk(ib)); };
     const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
     const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     const int reversed = r.reversed;
@@ -910,9 +912,30 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
             pr.sin ? pr.sin + (size_t)wi.bh * di * pr.lds : nullptr, pr.sout ? pr.sout + (size_t)wi.bh * di * pr.lds : nullptr,
             pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS);
     } else {
-        output_role<TR, DI, DJ, PF, IB, STREAM, PREP>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
-                                                      pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldo, r,
-                                                      IB * wv, l, sB, sC, sS, STAGED ? sO : nullptr, sA);
+        const u16 *A_head = pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh);
+        u16 *O_head = pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh);
+        if constexpr (IB == 2) {
+            // two wavefronts of two blocks: blocks {0,3} and {1,2}, dead score tiles left out (see output_role)
+            const bool future = (pr.mask_rev != 0) != (pr.comp != 0);
+            if (future) {
+                if (wv == 0)
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 1>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
+                                                                    STAGED ? sO : nullptr, sA);
+                else
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 2>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
+                                                                    STAGED ? sO : nullptr, sA);
+            } else {
+                if (wv == 0)
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 3>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
+                                                                    STAGED ? sO : nullptr, sA);
+                else
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 4>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
+                                                                    STAGED ? sO : nullptr, sA);
+            }
+        } else {
+            output_role<TR, DI, DJ, PF, IB, STREAM, PREP>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, IB * wv, l, sB, sC, sS,
+                                                          STAGED ? sO : nullptr, sA);
+        }
     }
 }
 
