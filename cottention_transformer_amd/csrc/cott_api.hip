@@ -261,7 +261,9 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
                     L.twin_of[c] = e;
             }
     // The group-state pass only streams two operands into MFMAs and two of its workgroups fit a CU: when its grid
-    // is well short of the chip, every group is cut into pieces (one workgroup and one slot each).
+    // does not fill the chip, every group is cut into up to four pieces (one workgroup and one slot each).  With k
+    // workgroups on the fullest CU the pass takes about k * (1.15 if k == 2) / pieces of its one-piece time
+    // (measured at B1 H16 N65536 D128: 144 workgroups 194 us, 288: 193, 432: 158, 576: 187; 240 -> 480: 84 -> 90).
     if (p.G > 1 && half) {
         long wgs = 0;
         if (L.pair)
@@ -274,9 +276,20 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
             }
         wgs *= BH;
         static const int force = exp_int("COTT_SUB", 0);
-        int sub = force > 0 ? force : (int)((288 + wgs / 2) / (wgs > 0 ? wgs : 1));
-        if (sub > 4) sub = 4;
-        while (sub > 1 && (p.cpg + sub - 1) / sub < 4) --sub;
+        const long cus = device_cus();
+        int sub = 1;
+        double best = 1e30;
+        for (int s = 1; s <= 4; ++s) {
+            if (s > 1 && (p.cpg + s - 1) / s < 4) break;
+            const long k = (wgs * s + cus - 1) / cus;
+            if (k > 2) break;
+            const double cost = (double)k * (k == 2 ? 1.15 : 1.0) / s;
+            if (cost < best - 1e-9) {
+                best = cost;
+                sub = s;
+            }
+        }
+        if (force > 0) sub = force;
         if (sub > 1) {
             L.p.sub = sub;
             L.p.ws_bytes *= (size_t)sub;
