@@ -167,6 +167,7 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
     const long tgt = target_workgroups() * (dtype == COTT_F32 ? 2 : 1);
     const bool can_split = !no_split && dtype != COTT_F32 && dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
     const int pol = split_policy();
+    const long xcds = device_xcds();
     p.nchunks = (N + 63) / 64;
     // Choose (column halves, sequence groups) to fill the target without exceeding it: halves cost
     // repeated score tiles but no memory traffic, groups cost one extra read of two operands.
@@ -178,7 +179,11 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
         if (h == 2 && (!can_split || pol == 0)) continue;
         if (h == 1 && can_split && pol == 1) continue;
         const long base = BH * nops * h;
-        long g = base >= tgt ? 1 : tgt / base;
+        // (head, group) units are dealt round-robin over the XCDs and the workgroups of a unit stay on one XCD:
+        // the fullest XCD gets ceil(BH * g / xcds) units and must hold them at once
+        const long units_per_xcd = tgt / xcds / (nops * h);
+        long g = units_per_xcd * xcds / BH;
+        if (g < 1) g = 1;
         if (g > p.nchunks) g = p.nchunks;
         const int cpg = (int)((p.nchunks + g - 1) / g);
         g = (p.nchunks + cpg - 1) / cpg;

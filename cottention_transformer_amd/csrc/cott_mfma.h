@@ -143,25 +143,27 @@ __device__ __forceinline__ float value_scale(float keep, float cnt, float sig, b
     return p > 1.f ? keep * __builtin_amdgcn_rcpf(p) : keep;
 }
 
-// Workgroup -> (head, problem, group).  Linear id i runs on XCD i % xcds; per XCD the ids are ordered
-// (head block, group, problem), so the workgroups of one head and group are neighbours in the
-// dispatch order of ONE XCD.
+// Workgroup -> (head, problem, group).  Linear id i runs on XCD i % xcds.  The (head, group) units, numbered
+// group-major (unit = grp * BH + bh), are dealt round-robin over the XCDs: any number of heads loads all XCDs
+// evenly, no XCD collects the units of one group (the first and last groups do less work), and with BH a
+// multiple of the XCD count a head stays on one XCD.  Per XCD the ids are ordered (unit, problem), so the
+// workgroups of one head and group are neighbours in the dispatch order of ONE XCD and share its L2.
 struct WorkItem {
     int bh, prob, grp;
 };
-__device__ __forceinline__ WorkItem decode_workgroup(int nprob, int G, int xcds) {
+__device__ __forceinline__ WorkItem decode_workgroup(int nprob, int BH, int xcds) {
     const int i = blockIdx.x;
     const int xcd = i % xcds;
-    int slot = i / xcds;
+    const int slot = i / xcds;
+    const int unit = (slot / nprob) * xcds + xcd;
     WorkItem wi;
     wi.prob = slot % nprob;
-    slot /= nprob;
-    wi.grp = slot % G;
-    wi.bh = (slot / G) * xcds + xcd;
+    wi.grp = unit / BH;  // >= G past the last unit: the caller returns
+    wi.bh = unit % BH;
     return wi;
 }
 inline unsigned grid_for(int BH, int nprob, int G, int xcds) {
-    return (unsigned)(((BH + xcds - 1) / xcds) * xcds * nprob * G);
+    return (unsigned)((((long)BH * G + xcds - 1) / xcds) * xcds * nprob);
 }
 
 // [64][D] tile, global -> registers, through a buffer descriptor of the head.  Thread t of NT owns 16-byte
@@ -282,10 +284,11 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int sub = set.sub;
-    const WorkItem wi = decode_workgroup(set.count, ngroups * sub, set.xcds);
-    if (wi.bh >= BH) return;
-    const Problem &pr = set.p[wi.prob];
-    const int grp = wi.grp / sub, piece = wi.grp % sub;
+    // same (head, group) -> XCD map as the scan that follows: what this pass leaves in an XCD's L2 is found there
+    const WorkItem wi = decode_workgroup(set.count * sub, BH, set.xcds);
+    if (wi.grp >= ngroups) return;
+    const Problem &pr = set.p[wi.prob / sub];
+    const int grp = wi.grp, piece = wi.prob % sub;
     // `ngroups` == G is launched when some op of the set is in complement form; the others skip their last group
     if (grp == G - 1 && ngroups == G && !pr.comp && !all_groups) return;
     if (pr.seed_from >= 0) return;
@@ -299,7 +302,7 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     f32x4 S[TL::TPW];
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-    f32x4 *slot = reinterpret_cast<f32x4 *>(pr.gstate + ((size_t)wi.bh * G * sub + wi.grp) * TL::STATE_FLOATS);
+    f32x4 *slot = reinterpret_cast<f32x4 *>(pr.gstate + (((size_t)wi.bh * G + grp) * sub + piece) * TL::STATE_FLOATS);
     if (p1 <= p0) {  // a piece past the end of its group: its slot is zero
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) slot[(w * TL::TPW + u) * 64 + l] = S[u];
@@ -875,8 +878,8 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     __shared__ __attribute__((aligned(16))) u16 sA[PREP ? 2 * SB : 8];  // PREP: the prepared A rows, staged like sB
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
-    if (wi.bh >= BH) return;
+    const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
+    if (wi.grp >= G) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
     ScanRange r;
@@ -964,8 +967,8 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     __shared__ __attribute__((aligned(16))) u16 sO[2 * 2 * kChunk * TL::OS];
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
-    if (wi.bh >= BH) return;
+    const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
+    if (wi.grp >= G) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc;
     const bool pair = pr.A2 != nullptr;
@@ -1034,8 +1037,8 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
     __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
-    if (wi.bh >= BH) return;
+    const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
+    if (wi.grp >= G) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, lda = pr.lda, ldo = pr.ldo;
     const rsrc_t rA = make_rsrc(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), ((uint32_t)(N - 1) * lda + di) * 2u);
@@ -1101,8 +1104,8 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
     __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, 1, set.xcds);
-    if (wi.bh >= BH) return;
+    const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
+    if (wi.grp >= 1) return;
     const Problem &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, lda = pr.lda, ldb = pr.ldb, ldc = pr.ldc, ldo = pr.ldo;
     const rsrc_t rA = make_rsrc(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), ((uint32_t)(N - 1) * lda + di) * 2u);

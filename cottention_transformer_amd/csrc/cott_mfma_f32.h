@@ -143,8 +143,8 @@ __global__ __launch_bounds__(kThreads) void group_state_f32_kernel(ProblemSetF32
     __shared__ __attribute__((aligned(16))) float sC[CH * TL::CS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, ngroups, set.xcds);
-    if (wi.bh >= BH) return;
+    const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);  // the (head, group) -> XCD map of the scan
+    if (wi.grp >= ngroups) return;
     const ProblemF32 &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = pr.reversed;
     const rsrc_t rB = make_rsrc(pr.B + (size_t)wi.bh * N * di, (uint32_t)N * di * 4u);
@@ -198,8 +198,8 @@ __global__ __launch_bounds__(kThreads) void scan_f32_kernel(ProblemSetF32 set, i
     __shared__ __attribute__((aligned(16))) float sP[APPLY ? 4 : CH * TL::PS];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.count, G, set.xcds);
-    if (wi.bh >= BH) return;
+    const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
+    if (wi.grp >= G) return;
     const ProblemF32 &pr = set.p[wi.prob];
     const int di = pr.di, dj = pr.dj, ldc = pr.ldc, reversed = APPLY ? 0 : pr.reversed;
     const rsrc_t rA = make_rsrc(pr.A + (size_t)wi.bh * N * di, (uint32_t)N * di * 4u);

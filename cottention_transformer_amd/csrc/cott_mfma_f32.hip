@@ -12,7 +12,7 @@ hipError_t run_causal_f32(const SetArgs &a) {
     if (a.G > 1) {
         {
             ProfScope prof(K_GROUP_STATE, a.stream);
-            group_state_f32_kernel<DI, DJ><<<dim3(grid_for(a.BH, a.count, a.G - 1, a.xcds)), dim3(kThreads), 0, a.stream>>>(
+            group_state_f32_kernel<DI, DJ><<<dim3(grid_for(a.BH, a.count, a.G, a.xcds)), dim3(kThreads), 0, a.stream>>>(
                 ps, a.BH, a.N, a.nchunks, a.cpg, a.G, a.G - 1);
         }
         const int bps = (TL::STATE_FLOATS / 4 + kThreads - 1) / kThreads;
