@@ -330,7 +330,9 @@ int check_common(const char *fn, int B, int H, int N, int di, int dj, int dtype)
     if (dj < 1) return fail(COTT_ERR_INVALID, "%s: D_value must be positive (got %d)", fn, dj);
     if ((long)B * H > (1L << 22)) return fail(COTT_ERR_UNSUPPORTED, "%s: B*H = %ld exceeds 2^22", fn, (long)B * H);
     const long dmax = di > dj ? di : dj;
-    if ((long)N * dmax > (1L << 30)) return fail(COTT_ERR_UNSUPPORTED, "%s: N*D = %ld exceeds 2^30", fn, (long)N * dmax);
+    // one head is addressed through a 32-bit byte offset: its bytes must stay below 2^32 (fp32: N*D < 2^30)
+    if ((long)N * dmax > (1L << 30) - (dtype == COTT_F32 ? 1 : 0))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: N*D = %ld exceeds 2^30", fn, (long)N * dmax);
     return COTT_OK;
 }
 

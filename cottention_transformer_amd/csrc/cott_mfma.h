@@ -15,6 +15,7 @@
 // per-group sums into exclusive prefixes, scan_kernel runs the recurrence seeded with its prefix.
 #pragma once
 #include "cott_common.h"
+#include <type_traits>
 
 namespace cott {
 
@@ -697,6 +698,8 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
 // score-times-C products remain for either wavefront.  SKIP = 1, 2: the scores of keys at or after the query are the
 // ones that count (ops that sum over the future, or over the past in complement form); SKIP = 3, 4: those of keys
 // at or before it.  The caller picks the variant that matches the problem's mask.
+// SKIP = 5 + b / 9 + b (one block per wavefront): the wavefront owns block b = 0..3 and leaves out the score tiles
+// of keys before (5 + b) / after (9 + b) its block in the same way.
 // TRS: sS holds the 16-bit copy of the TRANSPOSE of this problem's state (the copy published for a twin problem whose
 // B and C are this problem's C and B); it is then read with transposing LDS reads.
 template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false, int SKIP = 0, bool TRS = false>
@@ -706,11 +709,24 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
-    static_assert(SKIP == 0 || IB == 2, "block pairing needs two blocks per wavefront");
+    static_assert(SKIP == 0 || (SKIP <= 4 ? IB == 2 : (IB == 1 && SKIP <= 12)), "block pairing needs two blocks per wavefront");
     // block (16 positions of the chunk) number `ib` of this wavefront; whether its score tile against key tile jt
     // can hold anything (SKIP: keys >= queries are kept)
-    auto blk = [&](int ib) { return SKIP == 0 ? blk0 + ib : ((SKIP & 1) ? (ib == 0 ? 0 : 3) : (ib == 0 ? 1 : 2)); };
-    auto live = [&](int ib, int jt) { return SKIP == 0 || (SKIP <= 2 ? jt >= blk(ib) : jt <= blk(ib)); };
+    auto blk = [&](int ib) {
+        if constexpr (SKIP >= 5) return (SKIP - 5) & 3;
+        else return SKIP == 0 ? blk0 + ib : ((SKIP & 1) ? (ib == 0 ? 0 : 3) : (ib == 0 ? 1 : 2));
+    };
+    auto live = [&](int ib, int jt) {
+        if constexpr (SKIP == 0) return true;
+        else if constexpr (SKIP <= 4) return SKIP <= 2 ? jt >= blk(ib) : jt <= blk(ib);
+        else return SKIP <= 8 ? jt >= SKIP - 5 : jt <= SKIP - 9;
+    };
+    auto live_step = [&](int kb) {  // whether any block of this wavefront uses keys 32 kb .. 32 kb + 31
+        bool any = false;
+#pragma unroll
+        for (int ib = 0; ib < IB; ++ib) any = any || live(ib, 2 * kb) || live(ib, 2 * kb + 1);
+        return any;
+    };
     const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
     const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     const int reversed = r.reversed;
@@ -765,8 +781,9 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                     const int jt = j0 + jj;
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb)
-                        vf[slot][jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
-                                               lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
+                        if (live_step(kb))
+                            vf[slot][jj][kb] = cat(lds_col4(cC, TL::CS, 32 * kb + 4 * g, 16 * jt, m),
+                                                   lds_col4(cC, TL::CS, 32 * kb + 16 + 4 * g, 16 * jt, m));
 #pragma unroll
                     for (int ks = 0; ks < TL::KS; ++ks)
                         sf[slot][jj][ks] =
@@ -857,6 +874,22 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     });
 }
 
+// Calls f(integral_constant<int, v>) with v = block (0..3) + (future ? 0 : 4), i.e. SKIP - 5 of output_role, for an
+// output wavefront that owns one block of 16 positions.
+template <class F>
+__device__ __forceinline__ void one_block_variant(int block, bool future, F &&f) {
+    switch (block + (future ? 0 : 4)) {
+        case 0: f(std::integral_constant<int, 0>{}); break;
+        case 1: f(std::integral_constant<int, 1>{}); break;
+        case 2: f(std::integral_constant<int, 2>{}); break;
+        case 3: f(std::integral_constant<int, 3>{}); break;
+        case 4: f(std::integral_constant<int, 4>{}); break;
+        case 5: f(std::integral_constant<int, 5>{}); break;
+        case 6: f(std::integral_constant<int, 6>{}); break;
+        default: f(std::integral_constant<int, 7>{}); break;
+    }
+}
+
 // One problem per workgroup: OW output wavefronts (IB = 4/OW blocks each), 4 state, LW loader.
 // PREP: q, k, v are the raw projections and are prepared inside the kernel (PrepSide; forward direction, G = 1).
 template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false, bool STREAM = false, bool PREP = false>
@@ -936,8 +969,11 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
                                                                     STAGED ? sO : nullptr, sA);
             }
         } else {
-            output_role<TR, DI, DJ, PF, IB, STREAM, PREP>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, IB * wv, l, sB, sC, sS,
-                                                          STAGED ? sO : nullptr, sA);
+            // one block per wavefront: the variant that knows its block and the side of the diagonal that counts
+            one_block_variant(wv, (pr.mask_rev != 0) != (pr.comp != 0), [&](auto tag) {
+                output_role<TR, DI, DJ, PF, 1, STREAM, PREP, 5 + decltype(tag)::value>(
+                    A_head, O_head, di, dj, pr.lda, pr.ldo, r, wv, l, sB, sC, sS, STAGED ? sO : nullptr, sA);
+            });
         }
     }
 }
@@ -998,8 +1034,10 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
         state_role<TR, D, D>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS);
     } else if (!pair) {
         if (wv < 4) {
-            output_role<TR, D, D, PF, 1>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r,
-                                         wv, l, sB, sC, sS, sO);
+            one_block_variant(wv, (pr.mask_rev != 0) != (pr.comp != 0), [&](auto tag) {
+                output_role<TR, D, D, PF, 1, false, false, 5 + decltype(tag)::value>(
+                    pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r, wv, l, sB, sC, sS, sO);
+            });
         } else {
             for (int p = r.p0 - 1; p < r.p1; ++p) __syncthreads();  // idle: keep the barrier count
         }
