@@ -29,6 +29,9 @@ SIGNATURES = {
     "cott_prep_ex_bwd": (_i, [_vp] * 15 + [_i] * 10 + [_vp]),
     "cott_causal_bwd_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
+    "cott_causal_saved_plan": (_i, [_i] * 6 + [ctypes.POINTER(_i)] * 3 + [ctypes.POINTER(_sz)]),
+    "cott_causal_fwd_save": (_i, [_vp] * 5 + [_i] * 8 + [_vp, _sz, _vp]),
+    "cott_causal_bwd_saved": (_i, [_vp] * 8 + [_i] * 8 + [_vp, _sz, _vp]),
     "cott_causal_fwd_bnhd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_causal_bwd_bnhd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_workspace_bytes": (_sz, [_i] * 6),

@@ -28,19 +28,25 @@ class CustomAttention(torch.autograd.Function):
         if Q.dtype not in _SUPPORTED:
             raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
         Q, K, V = Q.contiguous(), K.contiguous(), V.contiguous()
-        ctx.save_for_backward(Q, K, V)  # saved before any autocast conversion (Custom_Kernel.py:16)
         dt = _autocast_target(Q, half_entry=(Q.dtype == torch.float16))
+        if dt == Q.dtype == K.dtype == V.dtype and dt in (torch.float16, torch.bfloat16):
+            # 16-bit tensors, forward and backward in the same type: on sequences long enough to be cut into groups
+            # the forward pass also leaves the states the backward pass starts dQ from (None otherwise)
+            out, states = ops.causal_dot_product_saving(Q, K, V)
+            ctx.save_for_backward(Q, K, V, *(() if states is None else (states,)))
+            return out
+        ctx.save_for_backward(Q, K, V)  # saved before any autocast conversion (Custom_Kernel.py:16)
         return ops.causal_dot_product(Q.to(dt), K.to(dt), V.to(dt), False)
 
     @staticmethod
     def backward(ctx, grad_output):
-        Q, K, V = ctx.saved_tensors
+        Q, K, V, *states = ctx.saved_tensors
         if Q.dtype not in _SUPPORTED:
             raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
         # One fused call in the saved tensors' dtype replaces the three launches of
         # Custom_Kernel.py:106-108 (same operand permutations inside the library).
         g = grad_output.contiguous().to(Q.dtype)
-        return ops.causal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g)
+        return ops.causal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g, saved=states[0] if states else None)
 
 
 class CustomAttentionMergedHeads(torch.autograd.Function):

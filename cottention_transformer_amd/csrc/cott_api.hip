@@ -132,6 +132,10 @@ struct Op {
     void *sout = nullptr;
     unsigned char lay[4] = {0, 0, 0, 0};  // A, B, C, O given as (B,N,H,width) instead of (BH,N,width)
     int H = 1;
+    // states handed from a forward to a backward pass (cott_causal_fwd_save / cott_causal_bwd_saved)
+    void *save = nullptr;       // (BH, save_n, pad(di) * pad(dj)) fp32 in 16 x 16 tiles: written by a forward op
+    const void *ext = nullptr;  // the same array, read by the backward op that sums over the past (dQ)
+    int save_cpg = 0, save_n = 0;
 };
 
 // How a set of `nops` ops with the same padded head dims is laid on the chip.
@@ -275,7 +279,7 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
             wgs = 2L * (p.G - 1);
         else
             for (int c = 0; c < cnt; ++c) {
-                if (L.twin_of[c] >= 0) continue;
+                if (L.twin_of[c] >= 0 || ops[members[c]].ext != nullptr) continue;
                 const bool comp = L.complement && !ops[members[c]].reversed && !ops[members[c]].sin && !ops[members[c]].sout;
                 wgs += (long)p.halves * (causal && !comp ? p.G - 1 : p.G);
             }
@@ -419,6 +423,25 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
                 d.lds = o.dj;
                 for (int x = 0; x < 4; ++x) d.lay[x] = o.lay[x];
                 d.H = o.H;
+                if (o.save != nullptr) {
+                    if (!causal || o.reversed || dtype == COTT_F32)
+                        return fail(COTT_ERR_UNSUPPORTED, "%s: states are saved by a forward-direction 16-bit causal op", fn);
+                    d.save = o.save;  // (the column half is found from c0)
+                    d.save_njt = cott::mfma_pad(o.dj) / 16;
+                    d.save_slot = cott::mfma_pad(o.di) * cott::mfma_pad(o.dj);
+                    d.save_cpg = o.save_cpg;
+                    d.save_n = o.save_n;
+                }
+                if (o.ext != nullptr) {
+                    if (!d.comp || p.G != o.save_n || p.cpg != o.save_cpg)
+                        return fail(COTT_ERR_INVALID, "%s: the saved states were cut for another plan (%d cuts of %d chunks; "
+                                    "this launch needs %d of %d, complement form %d)", fn, o.save_n, o.save_cpg, p.G, p.cpg, d.comp);
+                    d.ext = o.ext;  // saved by an op with this op's dims swapped
+                    d.save_njt = cott::mfma_pad(o.di) / 16;
+                    d.save_slot = cott::mfma_pad(o.di) * cott::mfma_pad(o.dj);
+                    d.save_cpg = o.save_cpg;
+                    d.save_n = o.save_n;
+                }
             }
         }
         a.ws = p.ws_bytes ? reinterpret_cast<float *>(ws_cursor) : nullptr;
@@ -681,6 +704,97 @@ int cott_causal_bwd(const void *q, const void *k, const void *v, const void *d_o
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
     Op ops[3];
     grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
+    return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+// Whether the backward pass of this shape takes states saved by the forward pass, and how they are cut: dQ must run
+// in complement form in a set cut into G > 1 groups (16-bit MFMA kernels, no pair workgroups).
+bool saved_states_plan(long BH, int N, int Dk, int Dv, int dtype, int *cpg, int *ncuts, size_t *bwd_ws) {
+    *cpg = 0;
+    *ncuts = 0;
+    if (bwd_ws) *bwd_ws = 0;
+    if ((dtype != COTT_BF16 && dtype != COTT_F16) || BH * N == 0) return false;
+    if (!use_mfma(dtype, Dk, Dv, N) || !use_mfma(dtype, Dv, Dk, N)) return false;
+    Op ops[3];
+    char tag[8];  // distinct stand-in addresses: the layout only compares operands
+    grad_ops(ops, tag + 0, tag + 1, tag + 2, tag + 3, tag + 4, tag + 5, tag + 6, Dk, Dv, true);
+    int members[8], cnt = 0;
+    for (int j = 0; j < 3; ++j)
+        if (pad_key(ops[j]) == pad_key(ops[0])) members[cnt++] = j;
+    const SetLayout L = layout_set(ops, 3, members, cnt, BH, N, dtype, true);
+    if (!L.complement || L.pair || L.p.G <= 1) return false;
+    *cpg = L.p.cpg;
+    *ncuts = L.p.G;
+    if (bwd_ws) {
+        ops[0].ext = tag + 7;
+        ops[0].save_cpg = L.p.cpg;
+        ops[0].save_n = L.p.G;
+        *bwd_ws = ops_workspace(ops, 3, BH, N, dtype, true);
+    }
+    return true;
+}
+}  // namespace
+
+int cott_causal_saved_plan(int B, int H, int N, int Dk, int Dv, int dtype, int *chunks_per_cut, int *ncuts,
+                           int *slot_floats, size_t *bwd_workspace_bytes) {
+    const char *fn = "cott_causal_saved_plan";
+    if (!chunks_per_cut || !ncuts || !slot_floats) return fail(COTT_ERR_INVALID, "%s: null result pointer", fn);
+    *chunks_per_cut = 0;
+    *ncuts = 0;
+    *slot_floats = 0;
+    if (bwd_workspace_bytes) *bwd_workspace_bytes = 0;
+    if (elem_size(dtype) == 0 || B < 0 || H < 0 || N < 0 || Dk < 1 || Dv < 1)
+        return fail(COTT_ERR_INVALID, "%s: bad shape or dtype", fn);
+    if (saved_states_plan((long)B * H, N, Dk, Dv, dtype, chunks_per_cut, ncuts, bwd_workspace_bytes))
+        *slot_floats = cott::mfma_pad(Dk) * cott::mfma_pad(Dv);
+    return COTT_OK;
+}
+
+int cott_causal_fwd_save(const void *q, const void *k, const void *v, void *o, float *saved, int chunks_per_cut,
+                         int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    const char *fn = "cott_causal_fwd_save";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if ((dtype != COTT_BF16 && dtype != COTT_F16) || !use_mfma(dtype, Dk, Dv, N))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: needs bf16 / fp16 tensors and head dims 32..128 in steps of 16", fn);
+    if (chunks_per_cut < 1 || ncuts < 1 || (long)(ncuts - 1) * chunks_per_cut > (N + 63) / 64 - 1)
+        return fail(COTT_ERR_INVALID, "%s: %d cuts of %d chunks do not fit %d positions (ask cott_causal_saved_plan)", fn,
+                    ncuts, chunks_per_cut, N);
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (!q || !k || !v || !o || !saved) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(saved))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op op{q, k, v, o, Dk, Dv, 0};
+    op.save = saved;
+    op.save_cpg = chunks_per_cut;
+    op.save_n = ncuts;
+    return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int cott_causal_bwd_saved(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
+                          const float *saved, int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv,
+                          int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+    const char *fn = "cott_causal_bwd_saved";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if (int rc = check_common(fn, B, H, N, Dv, Dk, dtype)) return rc;
+    if ((long)B * H * N == 0) return COTT_OK;
+    int cpg = 0, cuts = 0;
+    if (!saved_states_plan((long)B * H, N, Dk, Dv, dtype, &cpg, &cuts, nullptr))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: the backward pass of this shape takes no saved states "
+                    "(cott_causal_saved_plan gives 0 cuts); call cott_causal_bwd", fn);
+    if (cpg != chunks_per_cut || cuts != ncuts)
+        return fail(COTT_ERR_INVALID, "%s: states saved as %d cuts of %d chunks, this shape needs %d of %d", fn, ncuts,
+                    chunks_per_cut, cuts, cpg);
+    if (!q || !k || !v || !d_o || !dq || !dk || !dv || !saved) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
+        !aligned16(dv) || !aligned16(saved))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op ops[3];
+    grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
+    ops[0].ext = saved;
+    ops[0].save_cpg = chunks_per_cut;
+    ops[0].save_n = ncuts;
     return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 

@@ -26,6 +26,11 @@ struct OpDesc {
     int c0 = 0;  // first column of the C / O slice within the full rows (column halves)
     // >= 0: index (within the set) of the op whose state, transposed, is this op's state (see ProblemT::seed_from)
     int seed_from = -1;
+    // States handed from a forward to a backward pass (16-bit causal MFMA kernels only; see ProblemT::save / ext):
+    // (BH, save_n, save_slot) fp32 in 16 x 16 tiles, save_njt tiles per tile row.
+    void *save = nullptr;
+    const void *ext = nullptr;
+    int save_njt = 0, save_slot = 0, save_cpg = 0, save_n = 0;
 };
 
 // A set of ops launched together over the same (BH, N); MFMA path: all share padded head dims.

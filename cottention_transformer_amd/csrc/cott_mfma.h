@@ -49,6 +49,20 @@ struct ProblemT {
     // it and its scan reads the other problem's slots transposed.
     int seed_from;
     int c0;  // first column of this problem's C / O slice within the full rows (column halves)
+    // States handed from a forward to a backward pass.  save != null (an op that walks forwards over the past, not
+    // in complement form): the state after every chunk p with (nchunks - 1 - p) % save_cpg == 0 goes to slot
+    // (nchunks - 1 - p) / save_cpg (if < save_n) of this head, so slot g holds the sum over the chunks before
+    // nchunks - g * save_cpg (slot 0: the whole sequence).  A slot holds the padded state as 16 x 16 tiles in the
+    // accumulator layout: element [16 it + 4 g + q][16 jt + m] at ((it * save_njt + jt) * 64 + 16 g + m) * 4 + q,
+    // save_njt tiles per tile row, save_slot floats per slot; a column-half problem writes its own tile columns
+    // (c0 / 16 onwards).  One 16-byte store per lane and tile: a memory-bound scan has no vector-memory issue slots
+    // to spare for narrower ones.
+    // ext != null (an op in complement form cut into G groups of save_cpg chunks whose state is the TRANSPOSE of
+    // the saved one): slot `group` of this head is the op's state at the first chunk it walks; the group-state and
+    // prefix passes skip the op.
+    float *save;
+    const float *ext;
+    int save_njt, save_slot, save_cpg, save_n;
     // Row strides of A, B and O in elements (C's is ldc) and, for each operand, where a head
     // starts: head bh is at (bh / H) * bs + (bh % H) * hs elements.  (BH,N,w) tensors have ld = w, hs = N * w,
     // bs = H * hs; (B,N,H,w) tensors, whose heads are interleaved inside a position, ld = H * w, hs = w,
@@ -292,7 +306,7 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     const int grp = wi.grp, piece = wi.prob % sub;
     // `ngroups` == G is launched when some op of the set is in complement form; the others skip their last group
     if (grp == G - 1 && ngroups == G && !pr.comp && !all_groups) return;
-    if (pr.seed_from >= 0) return;
+    if (pr.seed_from >= 0 || pr.ext != nullptr) return;
     const int di = pr.di, dj = pr.dj, ldb = pr.ldb, ldc = pr.ldc, reversed = pr.reversed;
     const rsrc_t rB = make_rsrc(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), ((uint32_t)(N - 1) * ldb + di) * 2u);
     const rsrc_t rC = make_rsrc(pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), ((uint32_t)(N - 1) * ldc + dj) * 2u);
@@ -352,7 +366,7 @@ __global__ __launch_bounds__(kThreads) void state_prefix_kernel(ProblemSetT<E> s
     const int e = (blockIdx.x % blocks_per_state) * kThreads + threadIdx.x;
     const int rest = blockIdx.x / blocks_per_state;
     const int prob = rest % set.count, bh = rest / set.count;
-    if (e >= sf4 || bh >= BH || set.p[prob].seed_from >= 0) return;
+    if (e >= sf4 || bh >= BH || set.p[prob].seed_from >= 0 || set.p[prob].ext != nullptr) return;
     const int nslots = G * sub;
     const bool comp = mode == 0 && set.p[prob].comp;
     const int nread = (mode == 1 || comp) ? nslots : ncomputed * sub;
@@ -614,10 +628,18 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
 // fp32 hand-over states or null (sout only written when `last_group`).  sS: 16-bit copy transposed to
 // [j][i] for the A_blk S product (a twin problem whose B and C are this problem's C and B reads the same copy
 // transposed, see output_role).
+// Forward-to-backward state hand-over of one workgroup (see ProblemT::save / ext): ext points at the slot of this
+// head and group, save at the first slot of this head.
+struct StateIO {
+    const float *ext = nullptr;
+    float *save = nullptr;
+    int njt = 0, jt0 = 0, slot = 0, save_cpg = 1, save_n = 0;  // njt, slot: ProblemT::save_njt, save_slot; jt0 = c0 / 16
+};
+
 template <class TR, int DI, int DJ>
 __device__ __forceinline__ void state_role(const float *seed, bool seed_transposed, const float *sin, float *sout, int lds, bool last_group,
                                            int di, int dj, const ScanRange &r, int w, int l, const u16 *sB,
-                                           const u16 *sC, u16 *sS) {
+                                           const u16 *sC, u16 *sS, const StateIO &io = StateIO()) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
@@ -654,6 +676,19 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
                 if (i0 + q < di && j < dj) S[u][q] += sin[(size_t)(i0 + q) * lds + j];
         }
     }
+    if (io.ext != nullptr) {
+        // element [16it + 4g + q][16jt + m] of this state is element [16jt + m][16it + 4g + q] of the saved one:
+        // its tile (jt, it), lane (g' = m / 4, m' = 4g + q), component m % 4
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) {
+            const int t = w * TL::TPW + u;
+            const int it = t / TL::NJT, jt = t % TL::NJT;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (16 * it + 4 * g + q < di && 16 * jt + m < dj)  // (tiles outside the real dims are never written)
+                    S[u][q] += io.ext[((size_t)(jt * io.njt + it) * 64 + ((m >> 2) * 16 + 4 * g + q)) * 4 + (m & 3)];
+        }
+    }
     auto put_state = [&](u16 *dst) {
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) {
@@ -669,6 +704,18 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
         const int buf = (p - r.p0) & 1;
         state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m, r.comp ? 0x80008000u : 0u);
         put_state(sS + (buf ^ 1) * SSZ);
+        if (io.save != nullptr) {  // (this op walks forwards: p is the chunk's place in the sequence)
+            const int back = r.nchunks - 1 - p;
+            if (back % io.save_cpg == 0 && back / io.save_cpg < io.save_n) {
+                f32x4 *dst = reinterpret_cast<f32x4 *>(io.save + (size_t)(back / io.save_cpg) * io.slot);
+#pragma unroll
+                for (int u = 0; u < TL::TPW; ++u) {
+                    const int t = w * TL::TPW + u;
+                    // (tile columns past this problem's width belong to the other column half, or to nobody)
+                    if (16 * (t % TL::NJT) < dj) dst[((t / TL::NJT) * io.njt + io.jt0 + t % TL::NJT) * 64 + l] = S[u];
+                }
+            }
+        }
         __syncthreads();
     }
     if (sout != nullptr && last_group) {
@@ -942,11 +989,21 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
             loader_role<DI, DJ, PF, LT, STREAM>(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
                                                 di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (OW + 4), sB, sC, STAGED ? &so : nullptr);
     } else if (wv >= OW) {
-        const float *slots = pr.seed_from >= 0 ? set.p[pr.seed_from].gstate : pr.gstate;
+        const float *slots = pr.ext ? nullptr : (pr.seed_from >= 0 ? set.p[pr.seed_from].gstate : pr.gstate);
+        StateIO io;
+        io.njt = pr.save_njt;
+        io.slot = pr.save_slot;
+        if (pr.ext != nullptr) io.ext = pr.ext + ((size_t)wi.bh * G + wi.grp) * pr.save_slot;
+        if (pr.save != nullptr) {
+            io.save = pr.save + (size_t)wi.bh * pr.save_n * pr.save_slot;
+            io.jt0 = pr.c0 / 16;
+            io.save_cpg = pr.save_cpg;
+            io.save_n = pr.save_n;
+        }
         state_role<TR, DI, DJ>(
             slots ? slots + ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS : nullptr, pr.seed_from >= 0,
             pr.sin ? pr.sin + (size_t)wi.bh * di * pr.lds : nullptr, pr.sout ? pr.sout + (size_t)wi.bh * di * pr.lds : nullptr,
-            pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS);
+            pr.lds, wi.grp == G - 1, di, dj, r, wv - OW, l, sB, sC, sS, io);
     } else {
         const u16 *A_head = pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh);
         u16 *O_head = pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh);

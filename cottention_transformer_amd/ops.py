@@ -4,6 +4,8 @@ workspace with torch, and enqueue the HIP kernels on torch's current stream thro
 Tensor contract is the reference's: (B, H, N, D) for q/k/v/o (Cuda_Kernel/combined_kernel_general.cu
 :360-369), state (B, H, Dk, Dv) for decode.  Nothing here computes on the CPU.
 """
+import ctypes
+
 import torch
 
 from . import _loader
@@ -133,6 +135,52 @@ def causal_dot_product(q, k, v, reversed=False, merged_heads=False):
     return o
 
 
+_saved_plan_cache = {}
+
+
+def saved_states_plan(dtype, b, h, n, dk, dv):
+    """(chunks_per_cut, ncuts, floats per slot, backward workspace bytes) of the states the forward pass can leave for the backward
+    pass of this shape, or None when that backward pass takes none (it only does on sequences long enough, for the
+    number of heads, to be cut into groups; bf16 / fp16).  cott_causal_saved_plan, remembered per shape."""
+    if dtype not in (torch.bfloat16, torch.float16):
+        return None
+    key = (dtype, b, h, n, dk, dv)
+    plan = _saved_plan_cache.get(key, False)
+    if plan is False:
+        cpc, cuts, slot, ws = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
+        rc = _loader.lib().cott_causal_saved_plan(b, h, n, dk, dv, _DTYPES[dtype], ctypes.byref(cpc),
+                                                  ctypes.byref(cuts), ctypes.byref(slot), ctypes.byref(ws))
+        _check(rc, "cott_causal_saved_plan")
+        plan = _saved_plan_cache[key] = (cpc.value, cuts.value, slot.value, ws.value) if cuts.value > 0 else None
+    return plan
+
+
+def causal_dot_product_saving(q, k, v):
+    """(o, saved): causal_dot_product(q, k, v) that also leaves, where saved_states_plan() has cuts for the shape,
+    the (B,H,ncuts,slot) fp32 states (in the kernels' tile layout, see include/cottention.h) that causal_backward(..., saved=saved) starts dQ from instead of passing over
+    k and v once more (what CustomAttention.forward keeps for backward, Cuda_Kernel/Custom_Kernel.py:16, plus this
+    one small tensor).  saved is None where the plan has no cuts."""
+    _require_gpu(Q=q, K=k, V=v)
+    b, h, n, dk, dv = _shapes(q, k, v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("Q, K and V must have the same dtype")
+    plan = saved_states_plan(q.dtype, b, h, n, dk, dv)
+    if plan is None:
+        return causal_dot_product(q, k, v), None
+    cpc, cuts, slot, _ = plan
+    code = _dtype_code(q)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
+    saved = torch.empty((b, h, cuts, slot), dtype=torch.float32, device=q.device)
+    L = _loader.lib()
+    with _on(q.device):
+        ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
+        rc = L.cott_causal_fwd_save(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), saved.data_ptr(), cpc, cuts,
+                                    b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
+    _check(rc, "cott_causal_fwd_save")
+    return o, saved
+
+
 _prep_supported_cache = {}
 
 
@@ -218,8 +266,9 @@ def causal_prefill(q, k, v, state=None, return_state=True):
     return o, s_out
 
 
-def causal_backward(q, k, v, grad_out, merged_heads=False):
-    """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out ((B,N,H,Dv) with merged_heads)."""
+def causal_backward(q, k, v, grad_out, merged_heads=False, saved=None):
+    """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out ((B,N,H,Dv) with merged_heads).
+    saved: the states causal_dot_product_saving() returned for the same q, k, v (not with merged_heads)."""
     _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)
     b, h, n, dk, dv = _shapes(q, k, v)
     want = (b, n, h, dv) if merged_heads else tuple(v.shape)
@@ -231,6 +280,21 @@ def causal_backward(q, k, v, grad_out, merged_heads=False):
     q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), grad_out.contiguous()
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     L = _loader.lib()
+    if saved is not None:
+        plan = saved_states_plan(q.dtype, b, h, n, dk, dv)
+        if merged_heads or plan is None:
+            raise RuntimeError("causal_backward: this call takes no saved states")
+        cpc, cuts, slot, ws_bytes = plan
+        _require_gpu(saved=saved)
+        if tuple(saved.shape) != (b, h, cuts, slot) or saved.dtype != torch.float32 or not saved.is_contiguous():
+            raise RuntimeError(f"causal_backward: saved must be a contiguous fp32 tensor of shape {(b, h, cuts, slot)}")
+        with _on(q.device):
+            ws, ws_ptr = _workspace(ws_bytes, q.device)
+            rc = L.cott_causal_bwd_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(),
+                                         dk_.data_ptr(), dv_.data_ptr(), saved.data_ptr(), cpc, cuts, b, h, n, dk, dv, code,
+                                         ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
+        _check(rc, "cott_causal_bwd_saved")
+        return dq, dk_, dv_
     with _on(q.device):
         ws, ws_ptr = _workspace(_ws_bytes("cott_causal_bwd_workspace_bytes", b, h, n, dk, dv, code), q.device)
         fn = L.cott_causal_bwd_bnhd if merged_heads else L.cott_causal_bwd

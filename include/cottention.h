@@ -96,6 +96,37 @@ COTT_API int cott_causal_bwd(const void *q, const void *k, const void *v, const 
                     int B, int H, int N, int Dk, int Dv, int dtype,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- causal forward / backward with states saved for the backward pass -----------------------
+ * On long sequences of few heads the backward pass cuts every head into groups and needs the state
+ * sum_{s' in the groups before} k[s']^T v[s'] at each cut to compute dq; cott_causal_bwd gets it from an extra pass
+ * over k and v.  The forward pass carries exactly that state past every cut, so a training step can have it written
+ * there (a few MiB) and skip the extra pass: what CustomAttention.forward saves for backward
+ * (Cuda_Kernel/Custom_Kernel.py:16, ctx.save_for_backward) grows by one small tensor.
+ *   cott_causal_saved_plan   chunks_per_cut, ncuts (0 = this shape's backward pass takes no saved states: use the
+ *                            plain entry points), the floats per saved slot and the workspace
+ *                            cott_causal_bwd_saved needs.
+ *   cott_causal_fwd_save     cott_causal_fwd (not reversed; same o, bit for bit) that also writes
+ *                            saved: (B,H,ncuts,slot_floats) fp32, slot g = sum over the positions before
+ *                            64 * (ceil(N/64) - g * chunks_per_cut) of k^T v  (slot 0: the whole sequence).
+ *                            Workspace: cott_causal_workspace_bytes().
+ *   cott_causal_bwd_saved    cott_causal_bwd with dq seeded from `saved` (same results to rounding).
+ * A slot holds the (Dk,Dv) state padded to (P(Dk),P(Dv)), P(d) = 32, 64 or 128, as 16 x 16 tiles in the MFMA
+ * accumulator layout, so that the forward pass writes it with one 16-byte store per lane and tile: element
+ * [16 it + 4 g + c][16 jt + m] is float ((it * P(Dv)/16 + jt) * 64 + 16 g + m) * 4 + c of the slot; tiles outside
+ * (Dk,Dv) are not written.  The array only has a meaning for the shape and dtype it was made for.
+ * bf16 / fp16, head dims 32..128 in steps of 16; other cases return COTT_ERR_UNSUPPORTED. */
+COTT_API int cott_causal_saved_plan(int B, int H, int N, int Dk, int Dv, int dtype,
+                           int *chunks_per_cut, int *ncuts, int *slot_floats, size_t *bwd_workspace_bytes);
+COTT_API int cott_causal_fwd_save(const void *q, const void *k, const void *v, void *o,
+                         float *saved, int chunks_per_cut, int ncuts,
+                         int B, int H, int N, int Dk, int Dv, int dtype,
+                         void *workspace, size_t workspace_bytes, void *stream);
+COTT_API int cott_causal_bwd_saved(const void *q, const void *k, const void *v, const void *d_o,
+                          void *dq, void *dk, void *dv,
+                          const float *saved, int chunks_per_cut, int ncuts,
+                          int B, int H, int N, int Dk, int Dv, int dtype,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- causal forward / backward with the head merge folded in --------------------------------
  * The same two operations with the attention output o (forward) and its gradient d_o (backward) laid out
  * (B,N,H,Dv), i.e. as the rows of the (B,N,H*Dv) tensor that the output projection reads and

@@ -1,0 +1,113 @@
+"""GPU parity of the forward pass that saves states for the backward pass (cott_causal_fwd_save /
+cott_causal_bwd_saved) against the plain entry points and the CPU oracle."""
+import os
+
+import pytest
+import torch
+
+from util import TOL, inputs, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+
+
+@pytest.fixture(scope="module")
+def ct():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    import cottention_transformer_amd as ct_
+    from cottention_transformer_amd import _loader
+    assert os.path.exists(_loader.lib_path()), "libcottention_hip.so must be prebuilt in-tree"
+    _loader.lib()
+    return ct_
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+SAVED_CASES = [
+    (1, 16, 6000, 96, 96, BF),      # padded head dims (the forward pass runs column halves of 48)
+    # shapes whose backward pass is cut into groups with dQ in complement form
+    (1, 16, 4096, 128, 128, BF),    # forward in column halves (two workgroups write each slot)
+    (2, 8, 10000, 128, 128, HF),    # ragged tail, fp16
+    (1, 16, 7777, 128, 64, BF),     # Dk != Dv: dQ and dK form the set, dV runs apart
+    (1, 16, 30000, 64, 128, BF),
+    (1, 5, 30000, 128, 128, BF),    # 16 cuts; forward and backward cut the sequence differently
+]
+
+
+@pytest.mark.parametrize("case", SAVED_CASES, ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_states_saved_by_the_forward_pass_feed_the_backward_pass(ct, oracle, case):
+    b, h, n, dk, dv, dt = case
+    say("saved states", case)
+    plan = ct.saved_states_plan(dt, b, h, n, dk, dv)
+    assert plan is not None, "the case is meant to have cuts"
+    cpc, cuts, slot, _ = plan
+    q, k, v, do = inputs(b, h, n, dk, dv, dt, seed=n + 1)
+    qd, kd, vd, gd = (x.to(DEV) for x in (q, k, v, do))
+    o, saved = ct.causal_dot_product_saving(qd, kd, vd)
+    assert torch.equal(o, ct.causal_dot_product(qd, kd, vd)), "the saving forward must not change o"
+    assert saved.shape == (b, h, cuts, slot) and saved.dtype == torch.float32
+    # a slot is the padded state in 16 x 16 tiles: [tile row][tile column][g][m][c] holds element [16it+4g+c][16jt+m]
+    pk, pv = (32 if d <= 32 else 64 if d <= 64 else 128 for d in (dk, dv))
+    assert slot == pk * pv
+    states = saved.view(b, h, cuts, pk // 16, pv // 16, 4, 16, 4).permute(0, 1, 2, 3, 5, 7, 4, 6).reshape(b, h, cuts, pk, pv)
+    states = states[..., :dk, :dv]
+    # slot g = sum over the positions before 64 * (nchunks - g * cpc) of k^T v, in fp64 from the same rounded inputs
+    nchunks = (n + 63) // 64
+    for g_ in range(cuts):
+        end = min(n, 64 * (nchunks - g_ * cpc))
+        ref = torch.einsum("bhsi,bhsj->bhij", kd[:, :, :end].double(), vd[:, :, :end].double())
+        err = float((states[:, :, g_].double() - ref).norm() / ref.norm())
+        assert err <= 1e-5, (g_, err)
+    got = ct.causal_backward(qd, kd, vd, gd, saved=saved)
+    plain = ct.causal_backward(qd, kd, vd, gd)
+    for name, a, p_, r in zip(("dQ", "dK", "dV"), got, plain, oracle.causal_bwd(q, k, v, do)):
+        e_ref, e_plain = rel_l2(a, r), rel_l2(a, p_.double().cpu().numpy())
+        say(f"  {name}: vs oracle {e_ref:.2e}, vs the plain backward {e_plain:.2e}")
+        assert e_ref <= TOL[dt], name
+        assert e_plain <= 5e-3, name
+
+
+def test_saved_states_are_refused_where_the_backward_pass_takes_none(ct):
+    # enough heads that nothing is cut into groups: no plan, the saving forward returns None and the backward refuses
+    b, h, n, d = 8, 16, 512, 64
+    assert ct.saved_states_plan(BF, b, h, n, d, d) is None
+    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=3))
+    o, saved = ct.causal_dot_product_saving(q, k, v)
+    assert saved is None and torch.equal(o, ct.causal_dot_product(q, k, v))
+    with pytest.raises(RuntimeError, match="takes no saved states"):
+        ct.causal_backward(q, k, v, do, saved=torch.zeros(b, h, 1, d * d, device=DEV))
+    # a plan exists, but the states were cut differently
+    b, h, n, d = 1, 16, 4096, 128
+    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=4))
+    _, saved = ct.causal_dot_product_saving(q, k, v)
+    with pytest.raises(RuntimeError, match="saved must be"):
+        ct.causal_backward(q, k, v, do, saved=saved[:, :, :-1].contiguous())
+
+
+def test_custom_attention_saves_the_states_on_long_16_bit_sequences(ct, oracle):
+    """CustomAttention.apply on bf16 tensors long enough to be cut into groups: the forward pass keeps the states and
+    the backward pass uses them (spied on); gradients against the oracle."""
+    from unittest import mock
+    from cottention_transformer_amd import ops
+    from cottention_transformer_amd.autograd import CustomAttention
+    b, h, n, d = 1, 16, 4096, 128
+    q, k, v, do = inputs(b, h, n, d, d, BF, seed=11)
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    with mock.patch.object(ops, "causal_backward", wraps=ops.causal_backward) as spy:
+        out = CustomAttention.apply(qd, kd, vd)
+        out.backward(do.to(DEV))
+        assert spy.call_count == 1 and spy.call_args.kwargs.get("saved") is not None
+    assert rel_l2(out, oracle.causal(q, k, v)) <= TOL[BF]
+    for name, a, r in zip(("dQ", "dK", "dV"), (qd.grad, kd.grad, vd.grad), oracle.causal_bwd(q, k, v, do)):
+        assert rel_l2(a, r) <= TOL[BF], name
+    # fp32 tensors under autocast compute the forward in bf16 and the backward in fp32: nothing is saved
+    q32, k32, v32 = (x.float().to(DEV).requires_grad_(True) for x in (q, k, v))
+    with mock.patch.object(ops, "causal_backward", wraps=ops.causal_backward) as spy:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = CustomAttention.apply(q32, k32, v32)
+        out.backward(do.to(DEV))
+        assert spy.call_count == 1 and spy.call_args.kwargs.get("saved") is None
+    assert out.dtype == BF and q32.grad.dtype == torch.float32

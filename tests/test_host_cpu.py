@@ -164,6 +164,41 @@ def test_no_alloc_entry_point_checks_and_its_scratch_symbol(tmp_path):
     assert all("GLOBAL" in l and str(32 << 20) in l for l in rows), rows
 
 
+def test_saved_states_plan_and_argument_checks():
+    """cott_causal_saved_plan answers without a GPU (256 CUs in 8 XCDs assumed); the two entry points that use the
+    plan check their arguments before anything is launched."""
+    import ctypes
+    from cottention_transformer_amd import _loader
+    L = _loader.lib()
+
+    def plan(*shape_and_dtype):
+        cpc, cuts, slot, ws = ctypes.c_int(-1), ctypes.c_int(-1), ctypes.c_int(-1), ctypes.c_size_t(1)
+        rc = L.cott_causal_saved_plan(*shape_and_dtype, ctypes.byref(cpc), ctypes.byref(cuts), ctypes.byref(slot),
+                                      ctypes.byref(ws))
+        return rc, cpc.value, cuts.value, slot.value, ws.value
+    # long-context benchmark configuration: the backward pass runs 5 groups of 205 chunks per head
+    rc, cpc, cuts, slot, ws = plan(1, 16, 65536, 128, 128, _loader.BF16)
+    assert (rc, cpc, cuts, slot) == (_loader.OK, 205, 5, 128 * 128) and ws > 0
+    assert cuts * cpc >= 1024 > (cuts - 1) * cpc
+    # enough heads for one group each, pair workgroups (D = 64), fp32: no saved states
+    for shape in ((8, 16, 2048, 64, 64, _loader.BF16), (1, 16, 65536, 64, 64, _loader.BF16), (1, 16, 65536, 128, 128, _loader.F32)):
+        assert plan(*shape)[:4] == (_loader.OK, 0, 0, 0)
+    assert L.cott_causal_saved_plan(1, 16, 65536, 128, 128, _loader.BF16, None, None, None, None) == _loader.ERR_INVALID
+    # the saving forward refuses cuts that do not fit the sequence, other dtypes and null pointers
+    fwd, bwd = L.cott_causal_fwd_save, L.cott_causal_bwd_saved
+    assert fwd(16, 16, 16, 16, 16, 205, 6, 1, 16, 65536, 128, 128, _loader.BF16, None, 0, None) == _loader.ERR_INVALID
+    assert "do not fit" in _loader.last_error()
+    assert fwd(16, 16, 16, 16, 16, 205, 5, 1, 16, 65536, 128, 128, _loader.F32, None, 0, None) == _loader.ERR_UNSUPPORTED
+    assert fwd(16, 16, 16, 16, None, 205, 5, 1, 16, 65536, 128, 128, _loader.BF16, None, 0, None) == _loader.ERR_INVALID
+    assert fwd(None, None, None, None, None, 1, 1, 0, 16, 64, 128, 128, _loader.BF16, None, 0, None) == _loader.OK
+    # the backward pass refuses shapes without a plan and states cut for another plan
+    assert bwd(*[16] * 8, 1, 1, 8, 16, 2048, 64, 64, _loader.BF16, None, 0, None) == _loader.ERR_UNSUPPORTED
+    assert "takes no saved states" in _loader.last_error()
+    assert bwd(*[16] * 8, 200, 5, 1, 16, 65536, 128, 128, _loader.BF16, None, 0, None) == _loader.ERR_INVALID
+    assert "this shape needs 5 of 205" in _loader.last_error()
+    assert bwd(*[16] * 7, None, 205, 5, 1, 16, 65536, 128, 128, _loader.BF16, None, 0, None) == _loader.ERR_INVALID
+
+
 # ---- host layer mirrors the reference's checks ----------------------------------------------------
 
 def test_host_rejects_cpu_tensors_like_the_reference():
