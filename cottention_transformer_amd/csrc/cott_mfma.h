@@ -22,6 +22,7 @@ namespace cott {
 constexpr int kChunk = 64;     // positions per chunk
 constexpr int kThreads = 256;  // 4 wavefronts per workgroup
 constexpr int kMaxProblems = 6;
+constexpr int kWaveStageStride = 64 + 8;  // elements per row of an output wavefront's own staging tile [16 IB][64]
 
 // One generic op.  A, B: rows of `di` elements, contiguous.  C, O: `dj` columns taken from rows of
 // `ldc` elements (the pointers already include the first column), so a problem can own a column
@@ -82,6 +83,10 @@ struct ProblemSetT {
     // 16-bit kernels: the group-state pass cuts every group of the scan into `sub` pieces, one workgroup and one
     // slot each (slot (bh * G + grp) * sub + piece); the prefix pass leaves the scan's seed in the first of them
     int sub;
+    // problems the group-state pass computes sums for (the others take their states from a twin problem or from
+    // the forward pass): act[0 .. nact), so that its grid holds no workgroups that leave at once
+    int act[kMaxProblems];
+    int nact;
 };
 typedef ProblemT<u16> Problem;  // 16-bit storage (bf16 / fp16)
 typedef ProblemSetT<u16> ProblemSet;
@@ -299,10 +304,12 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int sub = set.sub;
-    // same (head, group) -> XCD map as the scan that follows: what this pass leaves in an XCD's L2 is found there
-    const WorkItem wi = decode_workgroup(set.count * sub, BH, set.xcds);
+    // (head, group) units dealt over the XCDs like those of the scan that follows; only the problems that need sums
+    // take part (workgroups that leave at once would still take dispatch slots, and the ones that stay then pile up
+    // two to a CU beside idle CUs)
+    const WorkItem wi = decode_workgroup(set.nact * sub, BH, set.xcds);
     if (wi.grp >= ngroups) return;
-    const Problem &pr = set.p[wi.prob / sub];
+    const Problem &pr = set.p[set.act[wi.prob / sub]];
     const int grp = wi.grp, piece = wi.prob % sub;
     // `ngroups` == G is launched when some op of the set is in complement form; the others skip their last group
     if (grp == G - 1 && ngroups == G && !pr.comp && !all_groups) return;
@@ -749,10 +756,11 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
 // of keys before (5 + b) / after (9 + b) its block in the same way.
 // TRS: sS holds the 16-bit copy of the TRANSPOSE of this problem's state (the copy published for a twin problem whose
 // B and C are this problem's C and B); it is then read with transposing LDS reads.
-template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false, int SKIP = 0, bool TRS = false>
+template <class TR, int DI, int DJ, int PF, int IB, bool STREAM = false, bool PREP = false, int SKIP = 0, bool TRS = false,
+          bool WST = false>
 __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int di, int dj, int lda, int ldc,
                                             const ScanRange &r, int blk0, int l, const u16 *sB, const u16 *sC,
-                                            const u16 *sS, u16 *sOt = nullptr, const u16 *sA = nullptr) {
+                                            const u16 *sS, u16 *sOt = nullptr, const u16 *sA = nullptr, u16 *sW = nullptr) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS, SSZ = DJ * TL::SS;
     const int g = l >> 4, m = l & 15;
@@ -907,7 +915,9 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                         }
                         const int col = 16 * jt + 4 * g;
                         const u32x2 val = {TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
-                        if (sOt != nullptr) {
+                        if constexpr (WST) {
+                            *reinterpret_cast<u32x2 *>(sW + (16 * ib + m) * kWaveStageStride + (col & 63)) = val;
+                        } else if (sOt != nullptr) {
                             *reinterpret_cast<u32x2 *>(sOt + buf * (2 * kChunk * TL::OS) +
                                                        (16 * blk(ib) + m) * TL::OS + col) = val;
                         } else {
@@ -915,6 +925,22 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
                             buf_store8(rO, off, val);
                         }
                     }
+                if constexpr (WST) {
+                    // 64 finished columns of this wavefront's rows: back out of its staging tile as 16-byte pieces,
+                    // eight lanes to a 128-byte row segment, and to memory as whole cache lines
+                    static_assert(!WST || (JB == 1 || JB == 2 || JB == 4), "a flush covers four column tiles");
+                    if (((bt + 1) * JB) % 4 == 0) {
+                        const int c0 = 16 * ((bt + 1) * JB - 4);
+#pragma unroll
+                        for (int u = 0; u < 2 * IB; ++u) {
+                            const int lrow = (l >> 3) + 8 * u, col = c0 + 8 * (l & 7);
+                            const u32x4 val = *reinterpret_cast<const u32x4 *>(sW + lrow * kWaveStageStride + 8 * (l & 7));
+                            const int prow = row0 + 16 * blk(u / 2) + (lrow & 15);
+                            const uint32_t off = (col < dj) ? (uint32_t)(prow * ldc + col) * 2u : kOobOffset;
+                            __builtin_amdgcn_raw_buffer_store_b128(val, rO, (int)off, 0, 0);
+                        }
+                    }
+                }
             }
             chunk_barrier();
         }
@@ -939,7 +965,10 @@ __device__ __forceinline__ void one_block_variant(int block, bool future, F &&f)
 
 // One problem per workgroup: OW output wavefronts (IB = 4/OW blocks each), 4 state, LW loader.
 // PREP: q, k, v are the raw projections and are prepared inside the kernel (PrepSide; forward direction, G = 1).
-template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false, bool STREAM = false, bool PREP = false>
+// WST: every output wavefront passes its tiles through a small staging tile of its own in LDS and stores them as
+// 16-byte pieces that make up whole 128-byte row segments (where a workgroup-wide staged tile, STAGED, has no room).
+template <class TR, int DI, int DJ, int PF, int OW, int LW, bool STAGED = false, bool STREAM = false, bool PREP = false,
+          bool WST = false>
 __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set, int BH, int N, int nchunks,
                                                                   int cpg, int G, PrepSide prep) {
     using TL = Tiling<DI, DJ>;
@@ -956,6 +985,8 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
     // the layout has room for two tiles per buffer, this kernel uses the first)
     __shared__ __attribute__((aligned(16))) u16 sO[STAGED ? 2 * 2 * kChunk * TL::OS : 8];
     __shared__ __attribute__((aligned(16))) u16 sA[PREP ? 2 * SB : 8];  // PREP: the prepared A rows, staged like sB
+    static_assert(!WST || (!STAGED && 4 / OW == 2 && DJ % 64 == 0), "wave-staged stores: two blocks per wavefront");
+    __shared__ __attribute__((aligned(16))) u16 sWst[WST ? OW * 32 * kWaveStageStride : 8];
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
@@ -1010,20 +1041,21 @@ __global__ __launch_bounds__(64 * (OW + 4 + LW)) void scan_kernel(ProblemSet set
         if constexpr (IB == 2) {
             // two wavefronts of two blocks: blocks {0,3} and {1,2}, dead score tiles left out (see output_role)
             const bool future = (pr.mask_rev != 0) != (pr.comp != 0);
+            u16 *sW = sWst + (WST ? wv * 32 * kWaveStageStride : 0);
             if (future) {
                 if (wv == 0)
-                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 1>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
-                                                                    STAGED ? sO : nullptr, sA);
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 1, false, WST>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l,
+                                                                                      sB, sC, sS, STAGED ? sO : nullptr, sA, sW);
                 else
-                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 2>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
-                                                                    STAGED ? sO : nullptr, sA);
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 2, false, WST>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l,
+                                                                                      sB, sC, sS, STAGED ? sO : nullptr, sA, sW);
             } else {
                 if (wv == 0)
-                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 3>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
-                                                                    STAGED ? sO : nullptr, sA);
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 3, false, WST>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l,
+                                                                                      sB, sC, sS, STAGED ? sO : nullptr, sA, sW);
                 else
-                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 4>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS,
-                                                                    STAGED ? sO : nullptr, sA);
+                    output_role<TR, DI, DJ, PF, 2, STREAM, PREP, 4, false, WST>(A_head, O_head, di, dj, pr.lda, pr.ldo, r, 0, l,
+                                                                                      sB, sC, sS, STAGED ? sO : nullptr, sA, sW);
             }
         } else {
             // one block per wavefront: the variant that knows its block and the side of the diagonal that counts
