@@ -30,14 +30,15 @@ def _entry(half_entry):
                                                             torch.bfloat16):
             raise RuntimeError("Unsupported data type")                                  # :387
         dt = _autocast_target(Q, half_entry=half_entry)                                  # :377-389
+        if inplace:
+            # the reference makes V the output tensor (:403-404); here the kernels write into V's memory where
+            # the library allows the alias (ops.causal_dot_product(into_v=True))
+            if V.dtype != dt or not V.is_contiguous():
+                raise RuntimeError("inplace=True needs a contiguous V of the compute dtype")
+            return ops.causal_dot_product(Q.contiguous().to(dt), K.contiguous().to(dt), V, bool(reversed),
+                                          into_v=True)
         out = ops.causal_dot_product(Q.contiguous().to(dt), K.contiguous().to(dt), V.contiguous().to(dt),
                                      bool(reversed))                                     # :397-421
-        if inplace:
-            # the reference aliases the output onto V (:403-404); same observable effect: V holds O
-            if V.dtype != out.dtype or not V.is_contiguous():
-                raise RuntimeError("inplace=True needs a contiguous V of the compute dtype")
-            V.copy_(out)
-            return V
         return out
     return call
 

@@ -27,6 +27,7 @@ SIGNATURES = {
     "cott_prep_bwd": (_i, [_vp] * 13 + [_i] * 7 + [_vp]),
     "cott_prep_ex_fwd": (_i, [_vp] * 11 + [_i] * 10 + [_vp]),
     "cott_prep_ex_bwd": (_i, [_vp] * 15 + [_i] * 10 + [_vp]),
+    "cott_causal_fwd_may_alias_v": (_i, [_i] * 6),
     "cott_causal_bwd_workspace_bytes": (_sz, [_i] * 6),
     "cott_causal_bwd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_causal_saved_plan": (_i, [_i] * 6 + [ctypes.POINTER(_i)] * 3 + [ctypes.POINTER(_sz)]),

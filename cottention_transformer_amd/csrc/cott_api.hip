@@ -537,6 +537,14 @@ int cott_causal_fwd(const void *q, const void *k, const void *v, void *o, int B,
     return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+int cott_causal_fwd_may_alias_v(int B, int H, int N, int Dk, int Dv, int dtype) {
+    // The MFMA scan kernels load the v rows of a chunk before they store its outputs, every workgroup reads only the
+    // rows (sequence group) and columns (column half) it writes, and the group-state pass has finished with v
+    // before the scan starts.  The plain-FMA kernels declare their operands __restrict__.
+    if (check_common("cott_causal_fwd_may_alias_v", B, H, N, Dk, Dv, dtype) != COTT_OK) return 0;
+    return use_mfma(dtype, Dk, Dv, N) ? 1 : 0;
+}
+
 int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim) {
     if (B < 0 || H < 0 || N < 0 || (dtype != COTT_BF16 && dtype != COTT_F16) || Dk % 16 != 0 || Dk < 32) return 0;
     if (!use_mfma(dtype, Dk, Dv, N)) return 0;

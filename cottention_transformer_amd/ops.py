@@ -97,25 +97,45 @@ def _stream(device=None):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+def _overlaps(a, b):
+    """Whether the storage ranges spanned by two tensors intersect."""
+    if a.numel() == 0 or b.numel() == 0 or a.untyped_storage().data_ptr() != b.untyped_storage().data_ptr():
+        return False
+    span = lambda t: (t.data_ptr(), t.data_ptr() + (sum((s - 1) * st for s, st in zip(t.shape, t.stride())) + 1) * t.element_size())
+    (a0, a1), (b0, b1) = span(a), span(b)
+    return a0 < b1 and b0 < a1
+
+
 def merged_heads_supported(dtype, n, h, dk, dv):
     """Whether the causal ops can write o / read grad_out as (B,N,H,Dv) (see causal_dot_product)."""
     ok = lambda d: 32 <= d <= 128 and d % 16 == 0
     return dtype in (torch.bfloat16, torch.float16) and ok(dk) and ok(dv) and n * h * max(dk, dv) <= 1 << 30
 
 
-def causal_dot_product(q, k, v, reversed=False, merged_heads=False):
+def causal_dot_product(q, k, v, reversed=False, merged_heads=False, into_v=False):
     """o[s,j] = sum_i q[s,i] sum_{s'<=s (>=s if reversed)} k[s',i] v[s',j]; all of one dtype.
 
     merged_heads: return o as (B,N,H,Dv), the rows of the (B,N,H*Dv) tensor an output projection reads, instead
     of (B,H,N,Dv): the head merge of GPT_Trainer/GPTCosAttention.py:500 without its copy (bf16 / fp16 only, see
-    merged_heads_supported)."""
+    merged_heads_supported).
+    into_v: the result overwrites v and v is returned (inplace=True of Cuda_Kernel/combined_kernel_general.cu
+    :403-404).  Where the library allows it (cott_causal_fwd_may_alias_v: the MFMA kernels) the kernels write
+    straight into v's memory; otherwise the result is computed beside it and copied.  v must be contiguous."""
     _require_gpu(Q=q, K=k, V=v)
     b, h, n, dk, dv = _shapes(q, k, v)
     if not (q.dtype == k.dtype == v.dtype):
         raise RuntimeError("Q, K and V must have the same dtype")
     code = _dtype_code(q)
+    if into_v:
+        if merged_heads or not v.is_contiguous():
+            raise RuntimeError("into_v needs a contiguous (B,H,N,Dv) v")
+        if _overlaps(q, v) or _overlaps(k, v):
+            raise RuntimeError("into_v: Q and K must not share memory with V")
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     L = _loader.lib()
+    if into_v and not L.cott_causal_fwd_may_alias_v(b, h, n, dk, dv, code):
+        v.copy_(causal_dot_product(q, k, v, reversed))
+        return v
     if merged_heads:
         if reversed:
             raise RuntimeError("merged_heads is only available for the forward direction")
@@ -126,7 +146,7 @@ def causal_dot_product(q, k, v, reversed=False, merged_heads=False):
                                         ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
         _check(rc, "cott_causal_fwd_bnhd")
         return o
-    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
+    o = v if into_v else torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
     with _on(q.device):
         ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
         rc = L.cott_causal_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, h, n, dk, dv, code,

@@ -56,6 +56,12 @@ COTT_API size_t cott_causal_workspace_bytes(int B, int H, int N, int Dk, int Dv,
 COTT_API int cott_causal_fwd(const void *q, const void *k, const void *v, void *o,
                     int B, int H, int N, int Dk, int Dv, int dtype, int reversed,
                     void *workspace, size_t workspace_bytes, void *stream);
+/* inplace=True of forward_<T> (combined_kernel_general.cu:403-404: the output tensor IS V).  Returns 1 when
+ * cott_causal_fwd may be called with o == v for this shape and dtype (every workgroup has read the rows and
+ * columns of v it needs before it, or any other workgroup, writes them as o): the MFMA kernels, i.e. bf16 / fp16 /
+ * fp32 with head dims 32..128 in steps of 16.  0: the caller computes into a temporary and copies.  Only the exact
+ * alias o == v is covered; q and k must not overlap o. */
+COTT_API int cott_causal_fwd_may_alias_v(int B, int H, int N, int Dk, int Dv, int dtype);
 
 /* ---- causal forward that takes no workspace and allocates nothing ------------------------------
  * cott_causal_fwd with the group-state slots (its workspace) kept in a device array built into the library

@@ -372,6 +372,49 @@ def test_custom_attention_autograd_and_dropin_names(ct, oracle):
         kernel.float32(qd[..., :16].contiguous(), kd[..., :16].contiguous(), vd, 1, False, False)
 
 
+INPLACE_CASES = [
+    # (b, h, n, dk, dv, dtype, reversed): what each case runs through
+    (8, 16, 512, 64, 64, BF, False),     # two column halves per head: both workgroups of a head write rows the other reads
+    (1, 2, 5000, 64, 64, BF, False),     # sequence groups: the group-state pass reads v before the scan overwrites it
+    (1, 2, 5000, 128, 128, HF, True),    # reversed, widest tiles (outputs staged per wavefront)
+    (2, 3, 1000, 48, 80, BF, False),     # padded head dims
+    (1, 2, 3000, 64, 64, F32, False),    # fp32 MFMA kernels
+    (1, 2, 300, 64, 64, F64, False),     # plain-FMA kernels: no alias allowed, computed beside v and copied
+    (1, 2, 300, 64, 20, F32, True),      # output dim outside the MFMA kernels' range: likewise
+]
+
+
+@pytest.mark.parametrize("case", INPLACE_CASES, ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_output_written_over_v(ct, oracle, case):
+    """inplace=True of forward_<T> (combined_kernel_general.cu:403-404): V holds the output afterwards, bit for bit what
+    the out-of-place call returns, and where the library allows the alias no second tensor of V's size is allocated."""
+    from cottention_transformer_amd import _loader, ops
+    b, h, n, dk, dv, dt, rev = case
+    say("inplace", case)
+    q, k, v, _ = inputs(b, h, n, dk, dv, dt, seed=n + dv)
+    qd, kd, vd = (x.to(DEV) for x in (q, k, v))
+    ref = ct.causal_dot_product(qd, kd, vd, rev)
+    assert rel_l2(ref, oracle.causal(q, k, v, rev)) <= TOL[dt]
+    v2 = vd.clone()
+    alias = bool(_loader.lib().cott_causal_fwd_may_alias_v(b, h, n, dk, dv, ops._DTYPES[dt]))
+    assert alias == (dt != F64 and dv % 16 == 0 and 32 <= dv <= 128)
+    ct.causal_dot_product(qd, kd, vd.clone(), rev, into_v=True)  # (warm-up: workspace and caches allocated)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    r = ct.causal_dot_product(qd, kd, v2, rev, into_v=True)
+    torch.cuda.synchronize()
+    grown = torch.cuda.max_memory_allocated() - before
+    assert r.data_ptr() == v2.data_ptr()
+    assert torch.equal(v2, ref), "the in-place result must equal the out-of-place one bit for bit"
+    if alias:  # nothing but the call's workspace (group-state slots) is allocated
+        ws = _loader.lib().cott_causal_workspace_bytes(b, h, n, dk, dv, ops._DTYPES[dt])
+        assert grown <= ws + 4096, "an aliased call must not allocate a second output"
+    if dk == dv:
+        with pytest.raises(RuntimeError, match="must not share memory"):
+            ct.causal_dot_product(v2, kd, v2, rev, into_v=True)
+
+
 def test_autocast_rule(ct, oracle):
     # fp32 inputs under autocast run the forward in bf16 (combined_kernel_general.cu:377-389); backward
     # runs outside autocast on the saved fp32 tensors (Custom_Kernel.py:16,38)

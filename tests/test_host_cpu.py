@@ -59,6 +59,18 @@ def test_library_exports_every_declared_symbol():
     assert lib.cott_version() >= 100
 
 
+def test_alias_query_follows_the_kernel_family():
+    """cott_causal_fwd_may_alias_v: the MFMA kernels (16-bit and fp32, head dims 32..128 in steps of 16) may write o
+    over v; fp64 and other head dims (plain-FMA kernels, operands declared __restrict__) may not."""
+    from cottention_transformer_amd import _loader
+    f = _loader.lib().cott_causal_fwd_may_alias_v
+    assert f(8, 16, 2048, 64, 64, _loader.BF16) == 1 and f(1, 16, 65536, 128, 128, _loader.F16) == 1
+    assert f(1, 2, 300, 64, 64, _loader.F32) == 1 and f(1, 2, 300, 48, 80, _loader.BF16) == 1
+    assert f(1, 2, 300, 64, 64, _loader.F64) == 0
+    assert f(1, 2, 300, 64, 20, _loader.F32) == 0 and f(1, 2, 300, 256, 256, _loader.BF16) == 0
+    assert f(1, 2, 300, 40, 64, _loader.BF16) == 0  # (a shape cott_causal_fwd refuses)
+
+
 def test_workspace_queries_are_pure_host_functions():
     from cottention_transformer_amd import _loader
     L = _loader.lib()
