@@ -24,7 +24,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # `bench.py --calibration-copy` (counters scaled by their reading for the 256 MiB copy in the same run).
 # A counter run cannot be made from inside this script; the figures and commands are in
 # profiles/headline_kernels_hbm_traffic_pmc.txt.
-MEASURED_TRAFFIC_BYTES = {"scan": 125.22 * 2**20, "scan_grad": 300.69 * 2**20}
+MEASURED_TRAFFIC_BYTES = {"scan": 125.46 * 2**20, "scan_grad": 301.06 * 2**20}
 
 
 def parse():
@@ -123,7 +123,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if args.long_only:
-        print(json.dumps(long_context(torch, ct, dev, args.long_only, args.steps, args.warmup)))
+        # (only the step as CustomAttention runs it, so that a kernel trace of this command holds one plan per kernel)
+        print(json.dumps(long_context(torch, ct, dev, args.long_only, args.steps, args.warmup, compare_plain=False)))
         return
     B, H, N, D = 8, 16, 2048, 64
     q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
@@ -231,7 +232,7 @@ def cold_cache_kernel_times(torch, ct, dev, q, k, v, do):
     return out
 
 
-def long_context(torch, ct, dev, n, steps, warmup, kernels=True):
+def long_context(torch, ct, dev, n, steps, warmup, kernels=True, compare_plain=True):
     """Long-context configuration B=1 H=16 D=128 bf16 at sequence length n: forward, backward and both, with the
     per-kernel durations the library records (HIP events around each launch)."""
     from cottention_transformer_amd import _loader
@@ -262,7 +263,7 @@ def long_context(torch, ct, dev, n, steps, warmup, kernels=True):
         bwd = lambda: ct.causal_backward(q, k, v, do)
     out = {"N": n, "states_saved_for_backward": saving}
     out.update(measure(fwd, bwd))
-    if saving:
+    if saving and compare_plain:
         plain = measure(lambda: ct.causal_dot_product(q, k, v), lambda: ct.causal_backward(q, k, v, do))
         out["plain_entry_points"] = {k_: plain[k_] for k_ in ("us", "fwd_us", "bwd_us", "frac_hbm")}
     if kernels:
