@@ -21,7 +21,16 @@ def _autocast_target(q, half_entry=False):
 
 
 class CustomAttention(torch.autograd.Function):
-    """O = causal cosine-attention core of (Q, K, V), tensors (N, H, S, D); apply(Q, K, V) -> O."""
+    """O = causal cosine-attention core of (Q, K, V), tensors (N, H, S, D); apply(Q, K, V) -> O.
+
+    backward_in_forward_dtype (class attribute, default False = the reference's behaviour): under autocast the
+    reference computes the forward in bf16 but saves the fp32 tensors (Custom_Kernel.py:16) and runs the backward on
+    them in fp32 (:38, :106-108).  Set to True, the tensors are saved as the forward pass rounded them and the
+    backward runs in that 16-bit type too (gradients returned in the inputs' types): the gradients of the function
+    that was actually evaluated, from the 16-bit kernels (several times faster than the fp32 ones) and from half
+    the saved bytes."""
+
+    backward_in_forward_dtype = False
 
     @staticmethod
     def forward(ctx, Q, K, V):
@@ -29,6 +38,10 @@ class CustomAttention(torch.autograd.Function):
             raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
         Q, K, V = Q.contiguous(), K.contiguous(), V.contiguous()
         dt = _autocast_target(Q, half_entry=(Q.dtype == torch.float16))
+        ctx.grad_dtypes = None
+        if dt in (torch.float16, torch.bfloat16) and CustomAttention.backward_in_forward_dtype:
+            ctx.grad_dtypes = (Q.dtype, K.dtype, V.dtype)
+            Q, K, V = Q.to(dt), K.to(dt), V.to(dt)
         if dt == Q.dtype == K.dtype == V.dtype and dt in (torch.float16, torch.bfloat16):
             # 16-bit tensors, forward and backward in the same type: on sequences long enough to be cut into groups
             # the forward pass also leaves the states the backward pass starts dQ from (None otherwise)
@@ -46,7 +59,10 @@ class CustomAttention(torch.autograd.Function):
         # One fused call in the saved tensors' dtype replaces the three launches of
         # Custom_Kernel.py:106-108 (same operand permutations inside the library).
         g = grad_output.contiguous().to(Q.dtype)
-        return ops.causal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g, saved=states[0] if states else None)
+        grads = ops.causal_backward(Q, K.to(Q.dtype), V.to(Q.dtype), g, saved=states[0] if states else None)
+        if ctx.grad_dtypes is not None:
+            grads = tuple(x.to(t) for x, t in zip(grads, ctx.grad_dtypes))
+        return grads
 
 
 class CustomAttentionMergedHeads(torch.autograd.Function):

@@ -372,6 +372,32 @@ def test_custom_attention_autograd_and_dropin_names(ct, oracle):
         kernel.float32(qd[..., :16].contiguous(), kd[..., :16].contiguous(), vd, 1, False, False)
 
 
+def test_autocast_backward_in_the_forward_type_is_an_option(ct, oracle):
+    """CustomAttention.backward_in_forward_dtype: fp32 tensors under autocast, forward AND backward in bf16, gradients
+    handed back in fp32; off by default (the reference's fp32 backward on the saved fp32 tensors, test_autocast_rule)."""
+    from unittest import mock
+    from cottention_transformer_amd import ops
+    from cottention_transformer_amd.autograd import CustomAttention
+    assert CustomAttention.backward_in_forward_dtype is False
+    b, h, n, d = 2, 3, 700, 64
+    q, k, v, do = inputs(b, h, n, d, d, F32, seed=6)
+    qg, kg, vg = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    try:
+        CustomAttention.backward_in_forward_dtype = True
+        with mock.patch.object(ops, "causal_backward", wraps=ops.causal_backward) as spy:
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                out = CustomAttention.apply(qg, kg, vg)
+            out.backward(do.to(DEV).bfloat16())
+            assert spy.call_count == 1 and all(t.dtype == BF for t in spy.call_args.args[:4])
+    finally:
+        CustomAttention.backward_in_forward_dtype = False
+    assert out.dtype == BF and all(t.grad.dtype == F32 for t in (qg, kg, vg))
+    qb, kb, vb, gb = (x.bfloat16() for x in (q, k, v, do))
+    assert rel_l2(out, oracle.causal(qb, kb, vb)) <= 2e-2
+    for got, ref in zip((qg.grad, kg.grad, vg.grad), oracle.causal_bwd(qb, kb, vb, gb)):
+        assert rel_l2(got, ref) <= 2e-2
+
+
 INPLACE_CASES = [
     # (b, h, n, dk, dv, dtype, reversed): what each case runs through
     (8, 16, 512, 64, 64, BF, False),     # two column halves per head: both workgroups of a head write rows the other reads
