@@ -129,10 +129,25 @@ def main():
     B, H, N, D = 8, 16, 2048, 64
     q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
 
-    def step():
-        o = ct.causal_dot_product(q, k, v)
-        grads = ct.causal_backward(q, k, v, do)
-        return o, grads
+    # The step as CustomAttention runs it on 16-bit tensors: the forward pass leaves the state dQ starts from (here one
+    # 16 KiB slot per head, the sum over the whole sequence) and the backward pass takes it, so that dQ walks the
+    # sequence from the end together with dK and dV.  The plain entry points are timed beside it (extras).
+    saving = ct.saved_states_plan(torch.bfloat16, B, H, N, D, D) is not None
+    if saving:
+        saved0 = ct.causal_dot_product_saving(q, k, v)[1]
+        fwd = lambda: ct.causal_dot_product_saving(q, k, v)
+        bwd = lambda: ct.causal_backward(q, k, v, do, saved=saved0)
+
+        def step():
+            o, saved = ct.causal_dot_product_saving(q, k, v)
+            grads = ct.causal_backward(q, k, v, do, saved=saved)
+            return o, grads
+    else:
+        fwd = lambda: ct.causal_dot_product(q, k, v)
+        bwd = lambda: ct.causal_backward(q, k, v, do)
+
+        def step():
+            return fwd(), bwd()
 
     # untimed spin-up so that the clocks have settled before the W warm-up steps (a cold process measures ~8 % low)
     t_end = time.perf_counter() + SPINUP_S
@@ -145,8 +160,14 @@ def main():
     tokens_per_s = B * N / sec
 
     # forward-only / backward-only split (same buffers)
-    sec_f = time_region(torch, lambda: ct.causal_dot_product(q, k, v), args.steps, 5)
-    sec_b = time_region(torch, lambda: ct.causal_backward(q, k, v, do), args.steps, 5)
+    sec_f = time_region(torch, fwd, args.steps, 5)
+    sec_b = time_region(torch, bwd, args.steps, 5)
+    if saving:
+        def plain_step():
+            ct.causal_dot_product(q, k, v)
+            ct.causal_backward(q, k, v, do)
+        sec_plain = time_region(torch, plain_step, args.steps, args.warmup)
+        sec_plain_b = time_region(torch, lambda: ct.causal_backward(q, k, v, do), args.steps, 5)
 
     # Per-kernel durations: the library brackets each launch with HIP events on the launch stream.
     _loader.profile_enable(True)
@@ -168,7 +189,7 @@ def main():
     alg_bytes = passes.get(dominant, 4) * tensor_bytes
     achieved = alg_bytes / (kern[dominant]["avg_us"] * 1e-6) / 1e9
     # the same kernels with cold caches: what a training step sees (other kernels run between forward and backward)
-    cold = cold_cache_kernel_times(torch, ct, dev, q, k, v, do)
+    cold = cold_cache_kernel_times(torch, fwd, bwd, dev)
     cold_dom = cold["bwd_kernel_us"] if dominant == "scan_grad" else cold["fwd_kernel_us"]
     cold_step_us = cold["fwd_kernel_us"] + cold["bwd_kernel_us"]
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -186,7 +207,10 @@ def main():
                                "algorithmic_tflops": 14.0 * B * H * N * D * D / sec / 1e12,
                                "frac_mfma_bf16": 14.0 * B * H * N * D * D / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS}}
 
-    extras = {"fwd_us": sec_f * 1e6, "bwd_us": sec_b * 1e6, "kernels": kern}
+    extras = {"fwd_us": sec_f * 1e6, "bwd_us": sec_b * 1e6, "kernels": kern, "states_saved_for_backward": saving}
+    if saving:
+        extras["plain_entry_points"] = {"us_per_step": sec_plain * 1e6, "bwd_us": sec_plain_b * 1e6,
+                                        "tokens_per_s": B * N / sec_plain}
     extras["cold_cache_headline"] = cold
     if not args.no_extras:
         extras.update(run_extras(torch, ct, dev))
@@ -197,7 +221,8 @@ def main():
         "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[2]: GPT-300M-shape causal cosine attention fwd+bwd (dQ,dK,dV), "
-                               "B=8 H=16 N=2048 D=64 bf16, fp32 state carry", "B": B, "H": H, "N": N, "D": D,
+                               "B=8 H=16 N=2048 D=64 bf16, fp32 state carry; forward keeps a 16 KiB state per head "
+                               "for the backward pass, as CustomAttention does", "B": B, "H": H, "N": N, "D": D,
                    "spinup_s": SPINUP_S},
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(torch),
@@ -224,10 +249,10 @@ def cold_kernel_us(torch, fn, kernel, big):
     return 1e3 * ms / n
 
 
-def cold_cache_kernel_times(torch, ct, dev, q, k, v, do):
+def cold_cache_kernel_times(torch, fwd, bwd, dev):
     big = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
-    out = {"fwd_kernel_us": cold_kernel_us(torch, lambda: ct.causal_dot_product(q, k, v), "scan", big),
-           "bwd_kernel_us": cold_kernel_us(torch, lambda: ct.causal_backward(q, k, v, do), "scan_grad", big)}
+    out = {"fwd_kernel_us": cold_kernel_us(torch, fwd, "scan", big),
+           "bwd_kernel_us": cold_kernel_us(torch, bwd, "scan_grad", big)}
     del big
     return out
 

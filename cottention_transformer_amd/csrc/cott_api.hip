@@ -258,9 +258,14 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
     // Gradient sets cut into sequence groups: the op that sums over the past (dQ) is put in complement form and
     // walks the sequence from the end like the two that sum over the future, so the three workgroups of a head
     // and group read the same tiles at the same time and the second and third reader find them in L2.
-    bool any_rev = false;
-    for (int c = 0; c < cnt; ++c) any_rev = any_rev || ops[members[c]].reversed;
-    L.complement = causal && !L.pair && p.G > 1 && cnt > 1 && any_rev && p.halves == 1 && half;
+    // With states saved by the forward pass (Op::ext) this also pays when a head is ONE group: the state dQ starts
+    // from is then the sum over the whole sequence, which only the forward pass has for free.
+    bool any_rev = false, any_ext = false;
+    for (int c = 0; c < cnt; ++c) {
+        any_rev = any_rev || ops[members[c]].reversed;
+        any_ext = any_ext || ops[members[c]].ext != nullptr;
+    }
+    L.complement = causal && !L.pair && (p.G > 1 || any_ext) && cnt > 1 && any_rev && p.halves == 1 && half;
     // ... and when two of them are X = G(.,B,C), Y = G(.,C,B) with square padded head dims (dK and dV), their
     // states are transposes of each other: the group-state pass computes X's only.
     for (int c = 0; c < 8; ++c) L.twin_of[c] = -1;
@@ -280,7 +285,7 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
     if (p.G > 1 && half) {
         long wgs = 0;
         if (L.pair)
-            wgs = 2L * (p.G - 1);
+            wgs = (ops[members[0]].ext != nullptr ? 1L : 2L) * (p.G - 1);
         else
             for (int c = 0; c < cnt; ++c) {
                 if (L.twin_of[c] >= 0 || ops[members[c]].ext != nullptr) continue;
@@ -418,7 +423,8 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
                 d.dj = djh;
                 d.ldc = o.dj;
                 d.reversed = o.reversed;
-                d.comp = (complement && !o.reversed && !o.sin && !o.sout) ? 1 : 0;
+                // (... and so does dQ beside a (dK, dV) pair when the forward pass has left its states)
+                d.comp = ((complement || (pair && o.ext != nullptr)) && !o.reversed && !o.sin && !o.sout) ? 1 : 0;
                 d.seed_from = twin_of[c];  // (halves == 1 here: set index == member index)
                 d.c0 = h * djh;
                 const size_t ssz = dtype == COTT_F64 ? 8 : 4;
@@ -731,15 +737,17 @@ bool saved_states_plan(long BH, int N, int Dk, int Dv, int dtype, int *cpg, int 
     Op ops[3];
     char tag[8];  // distinct stand-in addresses: the layout only compares operands
     grad_ops(ops, tag + 0, tag + 1, tag + 2, tag + 3, tag + 4, tag + 5, tag + 6, Dk, Dv, true);
+    ops[0].ext = tag + 7;  // plan as the backward pass would with the states at hand
     int members[8], cnt = 0;
     for (int j = 0; j < 3; ++j)
         if (pad_key(ops[j]) == pad_key(ops[0])) members[cnt++] = j;
     const SetLayout L = layout_set(ops, 3, members, cnt, BH, N, dtype, true);
-    if (!L.complement || L.pair || L.p.G <= 1) return false;
+    // dQ takes the states where it runs in complement form: in sets cut into groups, and -- a head being one group,
+    // the one slot then holding the sum over the whole sequence -- beside a (dK, dV) pair or two more problems
+    if (!L.pair && !L.complement) return false;
     *cpg = L.p.cpg;
     *ncuts = L.p.G;
     if (bwd_ws) {
-        ops[0].ext = tag + 7;
         ops[0].save_cpg = L.p.cpg;
         ops[0].save_n = L.p.G;
         *bwd_ws = ops_workspace(ops, 3, BH, N, dtype, true);

@@ -87,6 +87,7 @@ struct ProblemSetT {
     // the forward pass): act[0 .. nact), so that its grid holds no workgroups that leave at once
     int act[kMaxProblems];
     int nact;
+    int plain_two;  // scan_pair_kernel: the plain problem's workgroup runs two output wavefronts of two blocks
 };
 typedef ProblemT<u16> Problem;  // 16-bit storage (bf16 / fp16)
 typedef ProblemSetT<u16> ProblemSet;
@@ -1105,8 +1106,12 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
     r.p1 = min(r.p0 + cpg, nchunks);
     r.reversed = pr.reversed;
     r.mask_rev = pr.mask_rev;
-    r.comp = 0;  // (the pair workgroups never run in complement form)
-    const float *seed = pr.gstate ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS : nullptr;
+    // The plain problem (dQ) runs in complement form when the forward pass has left its states (ProblemT::ext): it
+    // then walks the sequence from the end like the pair and reads the tiles the pair's workgroup reads, at about
+    // the same time.  The pair itself never does.
+    r.comp = pair ? 0 : pr.comp;
+    const float *seed = (pr.gstate && pr.ext == nullptr)
+                            ? pr.gstate + ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS : nullptr;
     if (wv >= NOUT + 4) {
         StagedOut so;
         so.O[0] = pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh);
@@ -1120,12 +1125,29 @@ __global__ __launch_bounds__(64 * (2 * OWP + 4 + LW)) void scan_pair_kernel(Prob
                                   di, dj, pr.ldb, ldc, r, (int)threadIdx.x - 64 * (NOUT + 4), sB, sC, &so);
     } else if (wv >= NOUT) {
         // one 16-bit copy of the state serves both problems of a pair: the second reads it transposed
-        state_role<TR, D, D>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS);
+        StateIO io;
+        if (!pair && pr.ext != nullptr) {
+            io.ext = pr.ext + ((size_t)wi.bh * G + wi.grp) * pr.save_slot;
+            io.njt = pr.save_njt;
+            io.slot = pr.save_slot;
+        }
+        state_role<TR, D, D>(seed, false, nullptr, nullptr, 0, false, di, dj, r, wv - NOUT, l, sB, sC, sS, io);
     } else if (!pair) {
-        if (wv < 4) {
-            one_block_variant(wv, (pr.mask_rev != 0) != (pr.comp != 0), [&](auto tag) {
-                output_role<TR, D, D, PF, 1, false, false, 5 + decltype(tag)::value>(
-                    pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh), nullptr, di, dj, pr.lda, pr.ldo, r, wv, l, sB, sC, sS, sO);
+        const u16 *A_head = pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh);
+        const bool future = (pr.mask_rev != 0) != (r.comp != 0);
+        if (set.plain_two && wv < 2) {
+            // two output wavefronts of two blocks, the pace of the pair's workgroup next door
+            if (future) {
+                if (wv == 0) output_role<TR, D, D, PF, 2, false, false, 1>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS, sO);
+                else output_role<TR, D, D, PF, 2, false, false, 2>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS, sO);
+            } else {
+                if (wv == 0) output_role<TR, D, D, PF, 2, false, false, 3>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS, sO);
+                else output_role<TR, D, D, PF, 2, false, false, 4>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, 0, l, sB, sC, sS, sO);
+            }
+        } else if (!set.plain_two && wv < 4) {
+            one_block_variant(wv, future, [&](auto tag) {
+                output_role<TR, D, D, PF, 1, false, false, 5 + decltype(tag)::value>(A_head, nullptr, di, dj, pr.lda, pr.ldo, r, wv,
+                                                                                     l, sB, sC, sS, sO);
             });
         } else {
             for (int p = r.p0 - 1; p < r.p1; ++p) __syncthreads();  // idle: keep the barrier count

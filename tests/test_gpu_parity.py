@@ -435,7 +435,8 @@ def test_output_written_over_v(ct, oracle, case):
     assert torch.equal(v2, ref), "the in-place result must equal the out-of-place one bit for bit"
     if alias:  # nothing but the call's workspace (group-state slots) is allocated
         ws = _loader.lib().cott_causal_workspace_bytes(b, h, n, dk, dv, ops._DTYPES[dt])
-        assert grown <= ws + 4096, "an aliased call must not allocate a second output"
+        ws_alloc = -(-ws // (2 << 20)) * (2 << 20)  # (the caching allocator hands out large blocks in 2 MiB steps)
+        assert grown <= ws_alloc + 4096, "an aliased call must not allocate a second output"
     if dk == dv:
         with pytest.raises(RuntimeError, match="must not share memory"):
             ct.causal_dot_product(v2, kd, v2, rev, into_v=True)

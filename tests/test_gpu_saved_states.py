@@ -27,6 +27,15 @@ def say(*a):
 
 
 SAVED_CASES = [
+    # a head is one group: the one slot is the sum over the whole sequence
+    (8, 16, 2048, 64, 64, BF),      # headline shape: dQ in complement form beside the (dK, dV) pair workgroups
+    (3, 43, 1000, 48, 48, HF),      # the same with a ragged tail and padded head dims
+    (8, 16, 2048, 32, 32, BF),
+    (8, 16, 1024, 128, 128, BF),    # three separate problems per head walking backwards together
+    (6, 16, 700, 128, 64, BF),      # Dk != Dv: dQ and dK form the set
+    # pair workgroups in sequence groups
+    (2, 16, 8192, 64, 64, BF),
+    (1, 16, 10000, 64, 64, HF),
     (1, 16, 6000, 96, 96, BF),      # padded head dims (the forward pass runs column halves of 48)
     # shapes whose backward pass is cut into groups with dQ in complement form
     (1, 16, 4096, 128, 128, BF),    # forward in column halves (two workgroups write each slot)
@@ -71,14 +80,14 @@ def test_states_saved_by_the_forward_pass_feed_the_backward_pass(ct, oracle, cas
 
 
 def test_saved_states_are_refused_where_the_backward_pass_takes_none(ct):
-    # enough heads that nothing is cut into groups: no plan, the saving forward returns None and the backward refuses
-    b, h, n, d = 8, 16, 512, 64
-    assert ct.saved_states_plan(BF, b, h, n, d, d) is None
-    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=3))
+    # problems split into column halves: no plan, the saving forward returns None and the backward refuses
+    b, h, n, dk, dv = 4, 16, 2048, 128, 64
+    assert ct.saved_states_plan(BF, b, h, n, dk, dv) is None
+    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, dk, dv, BF, seed=3))
     o, saved = ct.causal_dot_product_saving(q, k, v)
     assert saved is None and torch.equal(o, ct.causal_dot_product(q, k, v))
     with pytest.raises(RuntimeError, match="takes no saved states"):
-        ct.causal_backward(q, k, v, do, saved=torch.zeros(b, h, 1, d * d, device=DEV))
+        ct.causal_backward(q, k, v, do, saved=torch.zeros(b, h, 1, 128 * 64, device=DEV))
     # a plan exists, but the states were cut differently
     b, h, n, d = 1, 16, 4096, 128
     q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=4))

@@ -192,8 +192,13 @@ def test_saved_states_plan_and_argument_checks():
     rc, cpc, cuts, slot, ws = plan(1, 16, 65536, 128, 128, _loader.BF16)
     assert (rc, cpc, cuts, slot) == (_loader.OK, 205, 5, 128 * 128) and ws > 0
     assert cuts * cpc >= 1024 > (cuts - 1) * cpc
-    # enough heads for one group each, pair workgroups (D = 64), fp32: no saved states
-    for shape in ((8, 16, 2048, 64, 64, _loader.BF16), (1, 16, 65536, 64, 64, _loader.BF16), (1, 16, 65536, 128, 128, _loader.F32)):
+    # headline shape: dQ beside the (dK, dV) pair workgroups starts from the sum over the whole sequence, one slot
+    assert plan(8, 16, 2048, 64, 64, _loader.BF16) == (_loader.OK, 32, 1, 64 * 64, 0)
+    # ... likewise three separate problems of one group each (128-wide heads); pairs cut into groups
+    assert plan(8, 16, 2048, 128, 128, _loader.BF16)[:4] == (_loader.OK, 32, 1, 128 * 128)
+    assert plan(1, 16, 65536, 64, 64, _loader.BF16)[:4] == (_loader.OK, 128, 8, 64 * 64)
+    # problems split into column halves, fp32: no saved states
+    for shape in ((4, 16, 2048, 128, 64, _loader.BF16), (1, 16, 65536, 128, 128, _loader.F32)):
         assert plan(*shape)[:4] == (_loader.OK, 0, 0, 0)
     assert L.cott_causal_saved_plan(1, 16, 65536, 128, 128, _loader.BF16, None, None, None, None) == _loader.ERR_INVALID
     # the saving forward refuses cuts that do not fit the sequence, other dtypes and null pointers
@@ -204,7 +209,7 @@ def test_saved_states_plan_and_argument_checks():
     assert fwd(16, 16, 16, 16, None, 205, 5, 1, 16, 65536, 128, 128, _loader.BF16, None, 0, None) == _loader.ERR_INVALID
     assert fwd(None, None, None, None, None, 1, 1, 0, 16, 64, 128, 128, _loader.BF16, None, 0, None) == _loader.OK
     # the backward pass refuses shapes without a plan and states cut for another plan
-    assert bwd(*[16] * 8, 1, 1, 8, 16, 2048, 64, 64, _loader.BF16, None, 0, None) == _loader.ERR_UNSUPPORTED
+    assert bwd(*[16] * 8, 1, 1, 4, 16, 2048, 128, 64, _loader.BF16, None, 0, None) == _loader.ERR_UNSUPPORTED
     assert "takes no saved states" in _loader.last_error()
     assert bwd(*[16] * 8, 200, 5, 1, 16, 65536, 128, 128, _loader.BF16, None, 0, None) == _loader.ERR_INVALID
     assert "this shape needs 5 of 205" in _loader.last_error()
