@@ -258,14 +258,12 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
     // Gradient sets cut into sequence groups: the op that sums over the past (dQ) is put in complement form and
     // walks the sequence from the end like the two that sum over the future, so the three workgroups of a head
     // and group read the same tiles at the same time and the second and third reader find them in L2.
-    // With states saved by the forward pass (Op::ext) this also pays when a head is ONE group: the state dQ starts
-    // from is then the sum over the whole sequence, which only the forward pass has for free.
-    bool any_rev = false, any_ext = false;
-    for (int c = 0; c < cnt; ++c) {
-        any_rev = any_rev || ops[members[c]].reversed;
-        any_ext = any_ext || ops[members[c]].ext != nullptr;
-    }
-    L.complement = causal && !L.pair && (p.G > 1 || any_ext) && cnt > 1 && any_rev && p.halves == 1 && half;
+    // (Beside a (dK, dV) pair dQ does the same whenever the forward pass has left its states, also when a head is one
+    // group: see run_ops.  Three separate problems of one group each gain nothing from it: 142 -> 157 us at B8 H16
+    // N2048 D128, where the 384 workgroups do not run at the same time anyway.)
+    bool any_rev = false;
+    for (int c = 0; c < cnt; ++c) any_rev = any_rev || ops[members[c]].reversed;
+    L.complement = causal && !L.pair && p.G > 1 && cnt > 1 && any_rev && p.halves == 1 && half;
     // ... and when two of them are X = G(.,B,C), Y = G(.,C,B) with square padded head dims (dK and dV), their
     // states are transposes of each other: the group-state pass computes X's only.
     for (int c = 0; c < 8; ++c) L.twin_of[c] = -1;
@@ -742,8 +740,8 @@ bool saved_states_plan(long BH, int N, int Dk, int Dv, int dtype, int *cpg, int 
     for (int j = 0; j < 3; ++j)
         if (pad_key(ops[j]) == pad_key(ops[0])) members[cnt++] = j;
     const SetLayout L = layout_set(ops, 3, members, cnt, BH, N, dtype, true);
-    // dQ takes the states where it runs in complement form: in sets cut into groups, and -- a head being one group,
-    // the one slot then holding the sum over the whole sequence -- beside a (dK, dV) pair or two more problems
+    // dQ takes the states where it runs in complement form: in sets cut into groups, and beside a (dK, dV) pair
+    // (there also when a head is one group: the one slot is then the sum over the whole sequence)
     if (!L.pair && !L.complement) return false;
     *cpg = L.p.cpg;
     *ncuts = L.p.G;

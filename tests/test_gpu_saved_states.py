@@ -31,8 +31,6 @@ SAVED_CASES = [
     (8, 16, 2048, 64, 64, BF),      # headline shape: dQ in complement form beside the (dK, dV) pair workgroups
     (3, 43, 1000, 48, 48, HF),      # the same with a ragged tail and padded head dims
     (8, 16, 2048, 32, 32, BF),
-    (8, 16, 1024, 128, 128, BF),    # three separate problems per head walking backwards together
-    (6, 16, 700, 128, 64, BF),      # Dk != Dv: dQ and dK form the set
     # pair workgroups in sequence groups
     (2, 16, 8192, 64, 64, BF),
     (1, 16, 10000, 64, 64, HF),

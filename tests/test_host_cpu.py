@@ -194,11 +194,11 @@ def test_saved_states_plan_and_argument_checks():
     assert cuts * cpc >= 1024 > (cuts - 1) * cpc
     # headline shape: dQ beside the (dK, dV) pair workgroups starts from the sum over the whole sequence, one slot
     assert plan(8, 16, 2048, 64, 64, _loader.BF16) == (_loader.OK, 32, 1, 64 * 64, 0)
-    # ... likewise three separate problems of one group each (128-wide heads); pairs cut into groups
-    assert plan(8, 16, 2048, 128, 128, _loader.BF16)[:4] == (_loader.OK, 32, 1, 128 * 128)
+    # ... likewise pairs cut into groups
     assert plan(1, 16, 65536, 64, 64, _loader.BF16)[:4] == (_loader.OK, 128, 8, 64 * 64)
-    # problems split into column halves, fp32: no saved states
-    for shape in ((4, 16, 2048, 128, 64, _loader.BF16), (1, 16, 65536, 128, 128, _loader.F32)):
+    # three separate problems of one group each (128-wide heads), column halves, fp32: no saved states
+    for shape in ((8, 16, 2048, 128, 128, _loader.BF16), (4, 16, 2048, 128, 64, _loader.BF16),
+                  (1, 16, 65536, 128, 128, _loader.F32)):
         assert plan(*shape)[:4] == (_loader.OK, 0, 0, 0)
     assert L.cott_causal_saved_plan(1, 16, 65536, 128, 128, _loader.BF16, None, None, None, None) == _loader.ERR_INVALID
     # the saving forward refuses cuts that do not fit the sequence, other dtypes and null pointers
