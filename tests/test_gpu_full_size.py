@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import TOL, inputs, rel_l2
+from util import TOL, inputs, rel_l2, worst_block
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -28,21 +28,6 @@ def ct():
 
 def say(*a):
     print(*a, flush=True)
-
-
-def worst_block(x, ref, rows=64):
-    """Largest rel-L2 over blocks of `rows` consecutive positions of any head; x, ref: (..., N, D)."""
-    x = x.detach().double().cpu().numpy() if hasattr(x, "detach") else np.asarray(x, dtype=np.float64)
-    ref = np.asarray(ref, dtype=np.float64)
-    n, d = ref.shape[-2:]
-    pad = (-n) % rows
-    if pad:
-        widths = [(0, 0)] * (ref.ndim - 2) + [(0, pad), (0, 0)]
-        x, ref = np.pad(x, widths), np.pad(ref, widths)
-    shape = ref.shape[:-2] + ((n + pad) // rows, rows * d)
-    num = np.linalg.norm((x - ref).reshape(shape), axis=-1)
-    den = np.linalg.norm(ref.reshape(shape), axis=-1)
-    return float(np.max(num / np.maximum(den, 1e-300)))
 
 
 def check(name, got, ref, tol):

@@ -5,7 +5,7 @@ import os
 import pytest
 import torch
 
-from util import TOL, inputs, rel_l2
+from util import TOL, inputs, rel_l2, worst_block
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -72,8 +72,9 @@ def test_states_saved_by_the_forward_pass_feed_the_backward_pass(ct, oracle, cas
     plain = ct.causal_backward(qd, kd, vd, gd)
     for name, a, p_, r in zip(("dQ", "dK", "dV"), got, plain, oracle.causal_bwd(q, k, v, do)):
         e_ref, e_plain = rel_l2(a, r), rel_l2(a, p_.double().cpu().numpy())
-        say(f"  {name}: vs oracle {e_ref:.2e}, vs the plain backward {e_plain:.2e}")
-        assert e_ref <= TOL[dt], name
+        e_blk = worst_block(a, r)  # (dQ in complement form: no stretch of the sequence may carry the error of the rest)
+        say(f"  {name}: vs oracle {e_ref:.2e} (worst 64-row block {e_blk:.2e}), vs the plain backward {e_plain:.2e}")
+        assert e_ref <= TOL[dt] and e_blk <= TOL[dt], name
         assert e_plain <= 5e-3, name
 
 

@@ -17,6 +17,21 @@ def rel_l2(x, ref):
     return float(np.linalg.norm(x - ref) / max(np.linalg.norm(ref), 1e-300))
 
 
+def worst_block(x, ref, rows=64):
+    """Largest rel-L2 over blocks of `rows` consecutive positions of any head; x, ref: (..., N, D)."""
+    x = x.detach().double().cpu().numpy() if hasattr(x, "detach") else np.asarray(x, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    n, d = ref.shape[-2:]
+    pad = (-n) % rows
+    if pad:
+        widths = [(0, 0)] * (ref.ndim - 2) + [(0, pad), (0, 0)]
+        x, ref = np.pad(x, widths), np.pad(ref, widths)
+    shape = ref.shape[:-2] + ((n + pad) // rows, rows * d)
+    num = np.linalg.norm((x - ref).reshape(shape), axis=-1)
+    den = np.linalg.norm(ref.reshape(shape), axis=-1)
+    return float(np.max(num / np.maximum(den, 1e-300)))
+
+
 def inputs(b, h, n, dk, dv, dtype, seed=0):
     """Seeded Q,K,V,dO ~ N(0,1); Q,K L2-normalised along D (GPTCosAttention.py:229-230); cast to dtype."""
     g = torch.Generator().manual_seed(seed)
