@@ -43,6 +43,8 @@ CAUSAL_CASES = [
     (2, 2, 257, 48, 80, BF),      # head dims that are multiples of 16 but not of 32
     (1, 2, 1023, 64, 64, BF),     # speeds.py:5 length; one chunk per group
     (2, 4, 19217, 64, 64, BF),    # several chunks per group and several groups per head
+    (6, 16, 300, 128, 128, BF),   # 96 heads of one group each, widest tiles: gradients as two launches (dK, dV | dQ in halves)
+    (7, 16, 200, 96, 80, HF),     # ... with padded head dims (all three problems share padded dims 128 x 128)
     (1, 2, 100, 64, 32, F32),
     (1, 1, 70, 256, 48, F32),     # D beyond the MFMA range -> generic path
     (1, 2, 77, 256, 256, BF),     # 16-bit storage on the generic path
