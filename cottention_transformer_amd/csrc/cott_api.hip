@@ -771,6 +771,9 @@ bool saved_states_plan(long BH, int N, int Dk, int Dv, int dtype, int *cpg, int 
     // dQ takes the states where it runs in complement form: in sets cut into groups, and beside a (dK, dV) pair
     // (there also when a head is one group: the one slot is then the sum over the whole sequence)
     if (!L.pair && !L.complement) return false;
+    // Sequences of a few chunks gain nothing from it, and their rows would lose precision: in complement form the
+    // rows of the first chunk are a difference of two sums rounded to 16 bits instead of one short sum.
+    if (L.p.nchunks < 8) return false;
     *cpg = L.p.cpg;
     *ncuts = L.p.G;
     if (bwd_ws) {

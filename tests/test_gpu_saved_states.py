@@ -119,3 +119,47 @@ def test_custom_attention_saves_the_states_on_long_16_bit_sequences(ct, oracle):
         out.backward(do.to(DEV))
         assert spy.call_count == 1 and spy.call_args.kwargs.get("saved") is None
     assert out.dtype == BF and q32.grad.dtype == torch.float32
+
+
+def test_random_shapes_every_16_bit_path_against_the_fp32_kernels(ct):
+    """30 seeded random shapes (head dims 32..128, 2..300 heads, 1..65536 positions, bf16 / fp16): the plain, the
+    saved-state and the merged-heads backward, the saving forward and the forward written over V, all against the
+    fp32 kernels of this library (themselves checked against the oracle in test_gpu_parity.py) on the same rounded
+    inputs: whole tensor and worst 64-row block within the 16-bit bar.  Launch plans differ from shape to shape
+    (column halves, sequence groups, pair workgroups, two launches, saved states or none)."""
+    import random
+    rnd = random.Random(5)
+
+    def err(a, r):
+        return max(rel_l2(a, r.double().cpu().numpy()), worst_block(a, r.double().cpu().numpy()))
+
+    worst = 0.0
+    for it in range(30):
+        dk = rnd.choice([32, 48, 64, 64, 64, 96, 128, 128])
+        dv = rnd.choice([dk, dk, dk, 32, 64, 128, 80])
+        h = rnd.choice([1, 2, 4, 8, 16])
+        b = max(1, rnd.choice([2, 8, 16, 40, 48, 90, 96, 128, 129, 200, 300]) // h)
+        n = min(rnd.choice([1, 63, 64, 65, 300, 1000, 2048, 4096, 10000, 30000, 65536]),
+                max(64, (1 << 26) // (b * h * max(dk, dv))))
+        dt = rnd.choice([BF, BF, HF])
+        q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, dk, dv, dt, seed=it))
+        say(f"random case {it}: B{b} H{h} N{n} Dk{dk} Dv{dv} {dt} plan {ct.saved_states_plan(dt, b, h, n, dk, dv)}")
+        ref_o = ct.causal_dot_product(q.float(), k.float(), v.float())
+        ref = ct.causal_backward(q.float(), k.float(), v.float(), do.float())
+        o = ct.causal_dot_product(q, k, v)
+        o2, saved = ct.causal_dot_product_saving(q, k, v)
+        assert torch.equal(o, o2)
+        v2 = v.clone()
+        assert ct.causal_dot_product(q, k, v2, into_v=True) is v2 and torch.equal(v2, o)
+        errs = [err(o, ref_o)]
+        outs = [ct.causal_backward(q, k, v, do)]
+        if saved is not None:
+            outs.append(ct.causal_backward(q, k, v, do, saved=saved))
+        if ct.merged_heads_supported(dt, n, h, dk, dv):
+            assert torch.equal(ct.causal_dot_product(q, k, v, merged_heads=True).permute(0, 2, 1, 3), o)
+            outs.append(ct.causal_backward(q, k, v, do.permute(0, 2, 1, 3).contiguous(), merged_heads=True))
+        for grads in outs:
+            errs += [err(a, r) for a, r in zip(grads, ref)]
+        assert max(errs) <= TOL[dt], (it, errs)
+        worst = max(worst, max(errs))
+    say(f"worst error over all cases and paths: {worst:.2e}")
