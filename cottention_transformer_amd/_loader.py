@@ -22,6 +22,7 @@ SIGNATURES = {
     "cott_causal_fwd_noalloc": (_i, [_vp] * 4 + [_i] * 7 + [_vp]),
     "cott_causal_fwd_prep_supported": (_i, [_i] * 7),
     "cott_causal_fwd_prep": (_i, [_vp] * 11 + [ctypes.c_longlong] + [_i] * 10 + [_vp]),
+    "cott_causal_fwd_prep_save": (_i, [_vp] * 11 + [ctypes.c_longlong] + [_i] * 4 + [_vp] + [_i] * 8 + [_vp]),
     "cott_causal_fwd_state": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_prep_fwd": (_i, [_vp] * 9 + [_i] * 7 + [_vp]),
     "cott_prep_bwd": (_i, [_vp] * 13 + [_i] * 7 + [_vp]),
@@ -33,6 +34,8 @@ SIGNATURES = {
     "cott_causal_saved_plan": (_i, [_i] * 6 + [ctypes.POINTER(_i)] * 3 + [ctypes.POINTER(_sz)]),
     "cott_causal_fwd_save": (_i, [_vp] * 5 + [_i] * 8 + [_vp, _sz, _vp]),
     "cott_causal_bwd_saved": (_i, [_vp] * 8 + [_i] * 8 + [_vp, _sz, _vp]),
+    "cott_causal_fwd_save_bnhd": (_i, [_vp] * 5 + [_i] * 8 + [_vp, _sz, _vp]),
+    "cott_causal_bwd_saved_bnhd": (_i, [_vp] * 8 + [_i] * 8 + [_vp, _sz, _vp]),
     "cott_causal_fwd_bnhd": (_i, [_vp] * 4 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_causal_bwd_bnhd": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _sz, _vp]),
     "cott_noncausal_workspace_bytes": (_sz, [_i] * 6),

@@ -77,13 +77,16 @@ class CustomAttentionMergedHeads(torch.autograd.Function):
             raise ValueError("Only float32, float64, float16, and bfloat16 are supported")
         dt = _autocast_target(Q, half_entry=(Q.dtype == torch.float16))
         Q, K, V = Q.contiguous().to(dt), K.contiguous().to(dt), V.contiguous().to(dt)
-        ctx.save_for_backward(Q, K, V)  # in the computed (16-bit) type: the backward reads the merged layout too
-        return ops.causal_dot_product(Q, K, V, False, merged_heads=True)
+        # in the computed (16-bit) type: the backward reads the merged layout too; with the states for its dQ
+        out, states = ops.causal_dot_product_saving(Q, K, V, merged_heads=True)
+        ctx.save_for_backward(Q, K, V, *(() if states is None else (states,)))
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        Q, K, V = ctx.saved_tensors
-        return ops.causal_backward(Q, K, V, grad_output.contiguous().to(Q.dtype), merged_heads=True)
+        Q, K, V, *states = ctx.saved_tensors
+        return ops.causal_backward(Q, K, V, grad_output.contiguous().to(Q.dtype), merged_heads=True,
+                                   saved=states[0] if states else None)
 
 
 class NonCausalAttention(torch.autograd.Function):
@@ -163,16 +166,18 @@ class PreparedCausalAttention(torch.autograd.Function):
     def forward(ctx, q, k, v, keep, cnt, sig, rot_table=None, first_position=0, bnhd=False, merged_heads=False):
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         rotary = (rot_table, int(first_position)) if rot_table is not None else None
-        out, prepared = ops.causal_dot_product_prepared(q, k, v, keep, cnt, sig, rotary=rotary, bnhd=bnhd,
-                                                        merged_heads=merged_heads, want_prepared=True)
-        ctx.save_for_backward(q, k, v, keep, cnt, sig, rot_table, *prepared)
+        out, prepared, states = ops.causal_dot_product_prepared(q, k, v, keep, cnt, sig, rotary=rotary, bnhd=bnhd,
+                                                                merged_heads=merged_heads, want_prepared=True,
+                                                                save_states=True)
+        ctx.save_for_backward(q, k, v, keep, cnt, sig, rot_table, *prepared, *(() if states is None else (states,)))
         ctx.first_position, ctx.bnhd, ctx.merged = int(first_position), bool(bnhd), bool(merged_heads)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        q, k, v, keep, cnt, sig, rot_table, qh, kh, vh = ctx.saved_tensors
-        gq, gk, gv = ops.causal_backward(qh, kh, vh, grad_output.contiguous().to(qh.dtype), merged_heads=ctx.merged)
+        q, k, v, keep, cnt, sig, rot_table, qh, kh, vh, *states = ctx.saved_tensors
+        gq, gk, gv = ops.causal_backward(qh, kh, vh, grad_output.contiguous().to(qh.dtype), merged_heads=ctx.merged,
+                                         saved=states[0] if states else None)
         rotary = None
         if rot_table is not None:
             b, n = (q.shape[0], q.shape[1]) if ctx.bnhd else (q.shape[0], q.shape[2])

@@ -593,11 +593,11 @@ int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtyp
     return p.G == 1 && cott::mfma_pad(Dk) * cott::mfma_pad(Dv / p.halves) <= 128 * 64;
 }
 
-int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
-                         const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
-                         long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, int B, int H, int N, int Dk,
-                         int Dv, int dtype, void *stream) {
-    const char *fn = "cott_causal_fwd_prep";
+namespace {
+int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out,
+                  void *v_out, const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
+                  long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved, int chunks_per_cut,
+                  int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *stream) {
     if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
     if (dtype != COTT_BF16 && dtype != COTT_F16)
         return fail(COTT_ERR_UNSUPPORTED, "%s: needs bf16 / fp16 tensors", fn);
@@ -626,6 +626,15 @@ int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o, v
     op.H = H;
     if (in_bnhd) op.lay[0] = op.lay[1] = op.lay[2] = 1;
     if (o_bnhd) op.lay[3] = 1;
+    if (saved != nullptr) {
+        if (chunks_per_cut < 1 || ncuts < 1 || (long)(ncuts - 1) * chunks_per_cut > (N + 63) / 64 - 1)
+            return fail(COTT_ERR_INVALID, "%s: %d cuts of %d chunks do not fit %d positions (ask cott_causal_saved_plan)", fn,
+                        ncuts, chunks_per_cut, N);
+        if (!aligned16(saved)) return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+        op.save = saved;
+        op.save_cpg = chunks_per_cut;
+        op.save_n = ncuts;
+    }
     cott::SetArgs::Prep prep;
     prep.on = true;
     prep.keep = keep;
@@ -641,6 +650,25 @@ int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o, v
     prep.ko = k_out;
     prep.vo = v_out;
     return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, nullptr, 0, static_cast<hipStream_t>(stream), &prep);
+}
+}  // namespace
+
+int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
+                         const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
+                         long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, int B, int H, int N, int Dk,
+                         int Dv, int dtype, void *stream) {
+    return fwd_prep_impl("cott_causal_fwd_prep", q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos0, rotary_dim,
+                         table_rows, in_bnhd, o_bnhd, nullptr, 0, 0, B, H, N, Dk, Dv, dtype, stream);
+}
+
+int cott_causal_fwd_prep_save(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
+                              const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
+                              long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved,
+                              int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *stream) {
+    const char *fn = "cott_causal_fwd_prep_save";
+    if ((long)B * H * N != 0 && saved == nullptr) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    return fwd_prep_impl(fn, q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos0, rotary_dim, table_rows,
+                         in_bnhd, o_bnhd, saved, chunks_per_cut, ncuts, B, H, N, Dk, Dv, dtype, stream);
 }
 
 namespace {
@@ -800,10 +828,12 @@ int cott_causal_saved_plan(int B, int H, int N, int Dk, int Dv, int dtype, int *
     return COTT_OK;
 }
 
-int cott_causal_fwd_save(const void *q, const void *k, const void *v, void *o, float *saved, int chunks_per_cut,
-                         int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace,
-                         size_t workspace_bytes, void *stream) {
-    const char *fn = "cott_causal_fwd_save";
+namespace {
+int check_interleaved(const char *fn, int H, int N, int Dk, int Dv, int dtype);
+
+int fwd_save_impl(const char *fn, bool o_bnhd, const void *q, const void *k, const void *v, void *o, float *saved,
+                  int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace,
+                  size_t workspace_bytes, void *stream) {
     if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
     if ((dtype != COTT_BF16 && dtype != COTT_F16) || !use_mfma(dtype, Dk, Dv, N))
         return fail(COTT_ERR_UNSUPPORTED, "%s: needs bf16 / fp16 tensors and head dims 32..128 in steps of 16", fn);
@@ -814,17 +844,20 @@ int cott_causal_fwd_save(const void *q, const void *k, const void *v, void *o, f
     if (!q || !k || !v || !o || !saved) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(saved))
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    if (o_bnhd)
+        if (int rc = check_interleaved(fn, H, N, Dk, Dv, dtype)) return rc;
     Op op{q, k, v, o, Dk, Dv, 0};
     op.save = saved;
     op.save_cpg = chunks_per_cut;
     op.save_n = ncuts;
+    if (o_bnhd) op.lay[3] = 1;
+    op.H = H;
     return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
-int cott_causal_bwd_saved(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
-                          const float *saved, int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv,
-                          int dtype, void *workspace, size_t workspace_bytes, void *stream) {
-    const char *fn = "cott_causal_bwd_saved";
+int bwd_saved_impl(const char *fn, bool do_bnhd, const void *q, const void *k, const void *v, const void *d_o, void *dq,
+                   void *dk, void *dv, const float *saved, int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv,
+                   int dtype, void *workspace, size_t workspace_bytes, void *stream) {
     if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
     if (int rc = check_common(fn, B, H, N, Dv, Dk, dtype)) return rc;
     if ((long)B * H * N == 0) return COTT_OK;
@@ -839,12 +872,46 @@ int cott_causal_bwd_saved(const void *q, const void *k, const void *v, const voi
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
         !aligned16(dv) || !aligned16(saved))
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    if (do_bnhd)
+        if (int rc = check_interleaved(fn, H, N, Dk, Dv, dtype)) return rc;
     Op ops[3];
     grad_ops(ops, q, k, v, d_o, dq, dk, dv, Dk, Dv, true);
     ops[0].ext = saved;
     ops[0].save_cpg = chunks_per_cut;
     ops[0].save_n = ncuts;
+    if (do_bnhd) {
+        ops[0].lay[0] = 1;  // d_o is A of dq, B of dk, C of dv (see cott_causal_bwd_bnhd)
+        ops[1].lay[1] = 1;
+        ops[2].lay[2] = 1;
+    }
+    for (int i = 0; i < 3; ++i) ops[i].H = H;
     return run_ops(fn, true, ops, 3, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+int cott_causal_fwd_save(const void *q, const void *k, const void *v, void *o, float *saved, int chunks_per_cut,
+                         int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    return fwd_save_impl("cott_causal_fwd_save", false, q, k, v, o, saved, chunks_per_cut, ncuts, B, H, N, Dk, Dv, dtype,
+                         workspace, workspace_bytes, stream);
+}
+int cott_causal_fwd_save_bnhd(const void *q, const void *k, const void *v, void *o, float *saved, int chunks_per_cut,
+                              int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+    return fwd_save_impl("cott_causal_fwd_save_bnhd", true, q, k, v, o, saved, chunks_per_cut, ncuts, B, H, N, Dk, Dv, dtype,
+                         workspace, workspace_bytes, stream);
+}
+int cott_causal_bwd_saved(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
+                          const float *saved, int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv,
+                          int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+    return bwd_saved_impl("cott_causal_bwd_saved", false, q, k, v, d_o, dq, dk, dv, saved, chunks_per_cut, ncuts, B, H, N, Dk,
+                          Dv, dtype, workspace, workspace_bytes, stream);
+}
+int cott_causal_bwd_saved_bnhd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
+                               const float *saved, int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv,
+                               int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+    return bwd_saved_impl("cott_causal_bwd_saved_bnhd", true, q, k, v, d_o, dq, dk, dv, saved, chunks_per_cut, ncuts, B, H, N,
+                          Dk, Dv, dtype, workspace, workspace_bytes, stream);
 }
 
 namespace {

@@ -175,28 +175,29 @@ def saved_states_plan(dtype, b, h, n, dk, dv):
     return plan
 
 
-def causal_dot_product_saving(q, k, v):
+def causal_dot_product_saving(q, k, v, merged_heads=False):
     """(o, saved): causal_dot_product(q, k, v) that also leaves, where saved_states_plan() has cuts for the shape,
     the (B,H,ncuts,slot) fp32 states (in the kernels' tile layout, see include/cottention.h) that causal_backward(..., saved=saved) starts dQ from instead of passing over
     k and v once more (what CustomAttention.forward keeps for backward, Cuda_Kernel/Custom_Kernel.py:16, plus this
-    one small tensor).  saved is None where the plan has no cuts."""
+    one small tensor).  saved is None where the plan has no cuts.  merged_heads: o as (B,N,H,Dv), see causal_dot_product."""
     _require_gpu(Q=q, K=k, V=v)
     b, h, n, dk, dv = _shapes(q, k, v)
     if not (q.dtype == k.dtype == v.dtype):
         raise RuntimeError("Q, K and V must have the same dtype")
     plan = saved_states_plan(q.dtype, b, h, n, dk, dv)
     if plan is None:
-        return causal_dot_product(q, k, v), None
+        return causal_dot_product(q, k, v, merged_heads=merged_heads), None
     cpc, cuts, slot, _ = plan
     code = _dtype_code(q)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    o = torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device)
+    o = torch.empty((b, n, h, dv) if merged_heads else (b, h, n, dv), dtype=q.dtype, device=q.device)
     saved = torch.empty((b, h, cuts, slot), dtype=torch.float32, device=q.device)
     L = _loader.lib()
+    fn = L.cott_causal_fwd_save_bnhd if merged_heads else L.cott_causal_fwd_save
     with _on(q.device):
         ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
-        rc = L.cott_causal_fwd_save(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), saved.data_ptr(), cpc, cuts,
-                                    b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), saved.data_ptr(), cpc, cuts,
+                b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
     _check(rc, "cott_causal_fwd_save")
     return o, saved
 
@@ -219,13 +220,15 @@ def fused_preparation_supported(dtype, b, h, n, dk, dv, rotary_dim=0):
 
 
 def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=None, bnhd=False, merged_heads=False,
-                                want_prepared=True):
+                                want_prepared=True, save_states=False):
     """Causal forward on the RAW projections q, k, v: rotation, normalisation, value scaling and masking
     (prepare_inputs) happen inside the attention kernel (GPT_Trainer/GPTCosAttention.py:229-248, 462-476 in front
     of :282 as one launch).  rotary = (table (P,R) fp32, first position): the table row of position s is
     first position + s.  bnhd: q, k, v are (B,N,H,D); merged_heads: o is returned as (B,N,H,Dv).
     Returns (o, (q_hat, k_hat, v_hat)) with the prepared tensors (B,H,N,D) that the backward pass needs, or
-    (o, None) when want_prepared is false.  Raises where fused_preparation_supported() is false."""
+    (o, None) when want_prepared is false.  Raises where fused_preparation_supported() is false.
+    save_states: returns (o, prepared, saved) with the states causal_backward(q_hat, k_hat, v_hat, ..., saved=saved)
+    takes (None where saved_states_plan() has none for the shape)."""
     _require_gpu(Q=q, K=k, V=v)
     b, h, n, dk, dv = _prep_shapes(q, k, v, bnhd)
     if not (q.dtype == k.dtype == v.dtype):
@@ -247,13 +250,20 @@ def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=N
                     torch.empty((b, h, n, dk), dtype=q.dtype, device=q.device),
                     torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device))
     L = _loader.lib()
+    plan = saved_states_plan(q.dtype, b, h, n, dk, dv) if save_states else None
+    saved = None
     with _on(q.device):
-        rc = L.cott_causal_fwd_prep(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                    *((t.data_ptr() for t in prepared) if prepared else (None, None, None)),
-                                    _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), int(pos0), rdim, rows, int(bool(bnhd)),
-                                    int(bool(merged_heads)), b, h, n, dk, dv, code, _stream(q.device))
+        head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                *((t.data_ptr() for t in prepared) if prepared else (None, None, None)),
+                _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), int(pos0), rdim, rows, int(bool(bnhd)), int(bool(merged_heads)))
+        if plan is not None:
+            cpc, cuts, slot, _ = plan
+            saved = torch.empty((b, h, cuts, slot), dtype=torch.float32, device=q.device)
+            rc = L.cott_causal_fwd_prep_save(*head, saved.data_ptr(), cpc, cuts, b, h, n, dk, dv, code, _stream(q.device))
+        else:
+            rc = L.cott_causal_fwd_prep(*head, b, h, n, dk, dv, code, _stream(q.device))
     _check(rc, "cott_causal_fwd_prep")
-    return o, prepared
+    return (o, prepared, saved) if save_states else (o, prepared)
 
 
 def causal_prefill(q, k, v, state=None, return_state=True):
@@ -288,7 +298,8 @@ def causal_prefill(q, k, v, state=None, return_state=True):
 
 def causal_backward(q, k, v, grad_out, merged_heads=False, saved=None):
     """(dQ, dK, dV) of causal_dot_product(q, k, v) for upstream gradient grad_out ((B,N,H,Dv) with merged_heads).
-    saved: the states causal_dot_product_saving() returned for the same q, k, v (not with merged_heads)."""
+    saved: the states causal_dot_product_saving() (or causal_dot_product_prepared(save_states=True)) returned for
+    the same q, k, v."""
     _require_gpu(Q=q, K=k, V=v, prev_grad=grad_out)
     b, h, n, dk, dv = _shapes(q, k, v)
     want = (b, n, h, dv) if merged_heads else tuple(v.shape)
@@ -302,7 +313,7 @@ def causal_backward(q, k, v, grad_out, merged_heads=False, saved=None):
     L = _loader.lib()
     if saved is not None:
         plan = saved_states_plan(q.dtype, b, h, n, dk, dv)
-        if merged_heads or plan is None:
+        if plan is None:
             raise RuntimeError("causal_backward: this call takes no saved states")
         cpc, cuts, slot, ws_bytes = plan
         _require_gpu(saved=saved)
@@ -310,9 +321,10 @@ def causal_backward(q, k, v, grad_out, merged_heads=False, saved=None):
             raise RuntimeError(f"causal_backward: saved must be a contiguous fp32 tensor of shape {(b, h, cuts, slot)}")
         with _on(q.device):
             ws, ws_ptr = _workspace(ws_bytes, q.device)
-            rc = L.cott_causal_bwd_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(),
-                                         dk_.data_ptr(), dv_.data_ptr(), saved.data_ptr(), cpc, cuts, b, h, n, dk, dv, code,
-                                         ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
+            fn = L.cott_causal_bwd_saved_bnhd if merged_heads else L.cott_causal_bwd_saved
+            rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), dq.data_ptr(),
+                    dk_.data_ptr(), dv_.data_ptr(), saved.data_ptr(), cpc, cuts, b, h, n, dk, dv, code,
+                    ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
         _check(rc, "cott_causal_bwd_saved")
         return dq, dk_, dv_
     with _on(q.device):

@@ -132,6 +132,17 @@ COTT_API int cott_causal_bwd_saved(const void *q, const void *k, const void *v, 
                           const float *saved, int chunks_per_cut, int ncuts,
                           int B, int H, int N, int Dk, int Dv, int dtype,
                           void *workspace, size_t workspace_bytes, void *stream);
+/* The same pair with o (forward) / d_o (backward) laid out (B,N,H,Dv), as cott_causal_fwd_bnhd / cott_causal_bwd_bnhd
+ * (the head merge of GPT_Trainer/GPTCosAttention.py:106-113 without its copy); `saved` is the same array. */
+COTT_API int cott_causal_fwd_save_bnhd(const void *q, const void *k, const void *v, void *o,
+                              float *saved, int chunks_per_cut, int ncuts,
+                              int B, int H, int N, int Dk, int Dv, int dtype,
+                              void *workspace, size_t workspace_bytes, void *stream);
+COTT_API int cott_causal_bwd_saved_bnhd(const void *q, const void *k, const void *v, const void *d_o,
+                               void *dq, void *dk, void *dv,
+                               const float *saved, int chunks_per_cut, int ncuts,
+                               int B, int H, int N, int Dk, int Dv, int dtype,
+                               void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- causal forward / backward with the head merge folded in --------------------------------
  * The same two operations with the attention output o (forward) and its gradient d_o (backward) laid out
@@ -253,6 +264,16 @@ COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, v
                          const float *rot_table, long long pos0, int rotary_dim, int table_rows,
                          int in_bnhd, int o_bnhd,
                          int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
+/* ... that also writes the states the backward pass takes (cott_causal_saved_plan for the same shape gives
+ * chunks_per_cut and ncuts; saved as in cott_causal_fwd_save, holding sums of k_hat^T v_hat): the backward of the
+ * block is then cott_causal_bwd_saved(_bnhd) on q_hat, k_hat, v_hat followed by cott_prep_ex_bwd. */
+COTT_API int cott_causal_fwd_prep_save(const void *q, const void *k, const void *v, void *o,
+                              void *q_out, void *k_out, void *v_out,
+                              const unsigned char *keep, const float *cnt, const float *sig,
+                              const float *rot_table, long long pos0, int rotary_dim, int table_rows,
+                              int in_bnhd, int o_bnhd,
+                              float *saved, int chunks_per_cut, int ncuts,
+                              int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
 
 /* ---- per-kernel timing -----------------------------------------------------------------------
  * While enabled, every kernel launch made by the entry points above is bracketed by a pair of HIP

@@ -121,6 +121,58 @@ def test_custom_attention_saves_the_states_on_long_16_bit_sequences(ct, oracle):
     assert out.dtype == BF and q32.grad.dtype == torch.float32
 
 
+@pytest.mark.parametrize("case", [(8, 16, 2048, 64, 64, BF), (2, 16, 8192, 64, 64, HF), (1, 16, 6000, 128, 128, BF)],
+                         ids=lambda c: "x".join(map(str, c[:5])))
+def test_saved_states_with_merged_heads(ct, oracle, case):
+    """cott_causal_fwd_save_bnhd / cott_causal_bwd_saved_bnhd: o written and d_o read as (B,N,H,Dv); same numbers as the
+    (B,H,N,D) pair, bit for bit."""
+    b, h, n, dk, dv, dt = case
+    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, dk, dv, dt, seed=n + 3))
+    o, saved = ct.causal_dot_product_saving(q, k, v)
+    om, saved_m = ct.causal_dot_product_saving(q, k, v, merged_heads=True)
+    assert saved is not None and torch.equal(saved, saved_m)
+    assert om.shape == (b, n, h, dv) and torch.equal(om.permute(0, 2, 1, 3), o)
+    plain = ct.causal_backward(q, k, v, do, saved=saved)
+    merged = ct.causal_backward(q, k, v, do.permute(0, 2, 1, 3).contiguous(), merged_heads=True, saved=saved_m)
+    for name, a, p_ in zip(("dQ", "dK", "dV"), merged, plain):
+        assert torch.equal(a, p_), name
+
+
+def test_block_level_functions_hand_the_states_to_their_backward(ct):
+    """CustomAttentionMergedHeads and PreparedCausalAttention (what modules.GPTCosAttention runs) keep the states of
+    their forward pass and their backward takes them; gradients equal to those of the plain composition within the
+    16-bit bar (the blocks' own parity tests are in test_gpu_modules.py)."""
+    from unittest import mock
+    from cottention_transformer_amd import ops
+    from cottention_transformer_amd.autograd import CustomAttention, CustomAttentionMergedHeads, PreparedCausalAttention
+    b, h, n, d = 8, 16, 1024, 64
+    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=21))
+    ref = ct.causal_backward(q, k, v, do)
+    qg, kg, vg = (x.clone().requires_grad_(True) for x in (q, k, v))
+    with mock.patch.object(ops, "causal_backward", wraps=ops.causal_backward) as spy:
+        CustomAttentionMergedHeads.apply(qg, kg, vg).backward(do.permute(0, 2, 1, 3).contiguous())
+        assert spy.call_count == 1 and spy.call_args.kwargs.get("saved") is not None
+    for a, r in zip((qg.grad, kg.grad, vg.grad), ref):
+        assert rel_l2(a, r.double().cpu().numpy()) <= 5e-3
+    # the preparation inside the forward kernel: raw projections in (B,N,H,D), no mask, no value scaling, no rotation
+    raw = [torch.randn(b, n, h, d, generator=torch.Generator().manual_seed(s)).to(BF).to(DEV).requires_grad_(True)
+           for s in (1, 2, 3)]
+    if not ct.fused_preparation_supported(BF, b, h, n, d, d, 0):
+        pytest.skip("the fused preparation is not built for this shape")
+    with mock.patch.object(ops, "causal_backward", wraps=ops.causal_backward) as spy:
+        out = PreparedCausalAttention.apply(*raw, None, None, None, None, 0, True, True)
+        out.backward(do.permute(0, 2, 1, 3).contiguous())
+        assert spy.call_count == 1 and spy.call_args.kwargs.get("saved") is not None
+    # the same through the separate pieces: prepare, then the plain attention function
+    raw2 = [x.detach().clone().requires_grad_(True) for x in raw]
+    qh, kh, vh = ct.PrepareInputs.apply(*raw2, None, None, None, BF, None, None, True)
+    out2 = CustomAttention.apply(qh, kh, vh)
+    out2.backward(do)
+    assert rel_l2(out.permute(0, 2, 1, 3), out2.detach().double().cpu().numpy()) <= 5e-3
+    for a, r in zip(raw, raw2):
+        assert rel_l2(a.grad, r.grad.double().cpu().numpy()) <= 2e-2
+
+
 def test_random_shapes_every_16_bit_path_against_the_fp32_kernels(ct):
     """30 seeded random shapes (head dims 32..128, 2..300 heads, 1..65536 positions, bf16 / fp16): the plain, the
     saved-state and the merged-heads backward, the saving forward and the forward written over V, all against the
