@@ -103,14 +103,19 @@ COTT_API int cott_causal_bwd(const void *q, const void *k, const void *v, const 
                     void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- causal forward / backward with states saved for the backward pass -----------------------
- * On long sequences of few heads the backward pass cuts every head into groups and needs the state
- * sum_{s' in the groups before} k[s']^T v[s'] at each cut to compute dq; cott_causal_bwd gets it from an extra pass
- * over k and v.  The forward pass carries exactly that state past every cut, so a training step can have it written
- * there (a few MiB) and skip the extra pass: what CustomAttention.forward saves for backward
- * (Cuda_Kernel/Custom_Kernel.py:16, ctx.save_for_backward) grows by one small tensor.
+ * dq sums over the past, dk and dv over the future.  Started from the sum of k^T v over the whole sequence (or, when
+ * heads are cut into sequence groups, over everything before a group's end) dq can be computed walking the sequence
+ * from its end like the other two, so that the three read the same rows of q, k, v and d_o at the same time and the
+ * gradient launch fetches each tensor once instead of nearly twice.  cott_causal_bwd has to get those sums from an
+ * extra pass over k and v (and only does for heads cut into groups); the forward pass carries exactly these states,
+ * so a training step can have them written there (16 KiB per head at the headline shape, a few MiB on long
+ * sequences): what CustomAttention.forward saves for backward (Cuda_Kernel/Custom_Kernel.py:16,
+ * ctx.save_for_backward) grows by one small tensor.
  *   cott_causal_saved_plan   chunks_per_cut, ncuts (0 = this shape's backward pass takes no saved states: use the
  *                            plain entry points), the floats per saved slot and the workspace
- *                            cott_causal_bwd_saved needs.
+ *                            cott_causal_bwd_saved needs.  Plans exist for sequences of 8 chunks or more whose
+ *                            gradients run as dq beside a (dk, dv) pair of workgroups (square head dims up to 64)
+ *                            or as three problems cut into sequence groups.
  *   cott_causal_fwd_save     cott_causal_fwd (not reversed; same o, bit for bit) that also writes
  *                            saved: (B,H,ncuts,slot_floats) fp32, slot g = sum over the positions before
  *                            64 * (ceil(N/64) - g * chunks_per_cut) of k^T v  (slot 0: the whole sequence).
