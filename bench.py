@@ -5,7 +5,8 @@
 
 A step is one causal forward + backward (dQ, dK, dV) over one synthetic batch at the headline
 shape B=8 H=16 N=2048 D=64 bf16, called through the C ABI on torch's current stream with every
-input already resident in HBM.  Prints ONE JSON line: whole-job tokens/s, the roofline object of
+input already resident in HBM, the way CustomAttention runs it: the forward also leaves one 16 KiB
+state per head that the backward starts dQ from (the plain entry points are timed beside it).  Prints ONE JSON line: whole-job tokens/s, the roofline object of
 the dominant kernel (HIP events recorded by the library around each of its launches), and the CPU
 baseline (the reference's PyTorch cumsum formulation timed on the host cores of this box).
 """
