@@ -659,19 +659,36 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) S[u] = gs[(w * TL::TPW + u) * 64 + l];
     }
-    if constexpr (DI == DJ) {
-        if (seed != nullptr && seed_transposed) {
-            // element [16it + 4g + q][16jt + m] of this state is element [16jt + m][16it + 4g + q] of the other one:
-            // its tile (jt, it), lane (m' = 4g + q, g' = m / 4), component m % 4
+    // A state held as 16 x 16 tiles in the accumulator layout (float4 index tile * 64 + lane), read TRANSPOSED: element
+    // [16it + 4g + q][16jt + m] of this state is element [16jt + m][16it + 4g + q] of the other one, i.e. its tile
+    // (jt, it), lane (g' = m / 4, m' = 4g + q), component m % 4.  Each source tile is loaded as it lies (one coalesced
+    // 16-byte load per lane) and turned through a 1 KiB piece of LDS of this wavefront's own: 64 scattered 4-byte
+    // loads per lane took several microseconds per workgroup.  The piece lies in the second buffer of the B tile,
+    // which nobody writes before the first barrier.
+    auto add_transposed = [&](const float *src, int src_njt) {
+        float *scr = reinterpret_cast<float *>(const_cast<u16 *>(sB) + SB) + w * 256;
+        f32x4 tile[TL::TPW];
 #pragma unroll
-            for (int u = 0; u < TL::TPW; ++u) {
-                const int t = w * TL::TPW + u;
-                const int it = t / TL::NJT, jt = t % TL::NJT;
+        for (int u = 0; u < TL::TPW; ++u) {
+            const int t = w * TL::TPW + u;
+            tile[u] = reinterpret_cast<const f32x4 *>(src)[(size_t)((t % TL::NJT) * src_njt + t / TL::NJT) * 64 + l];
+        }
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    S[u][q] = seed[((size_t)(jt * TL::NJT + it) * 64 + ((m >> 2) * 16 + 4 * g + q)) * 4 + (m & 3)];
+        for (int u = 0; u < TL::TPW; ++u) {
+            const int t = w * TL::TPW + u;
+            const int it = t / TL::NJT, jt = t % TL::NJT;
+            *reinterpret_cast<f32x4 *>(scr + 4 * l) = tile[u];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float x = scr[((m >> 2) * 16 + 4 * g + q) * 4 + (m & 3)];
+                // (tiles outside the real dims are never written by the pass that saved them)
+                if (16 * it + 4 * g + q < di && 16 * jt + m < dj) S[u][q] += x;
             }
         }
+    };
+    static_assert(SB * 2 >= 4 * 1024, "room for one tile per state wavefront");
+    if constexpr (DI == DJ) {
+        if (seed != nullptr && seed_transposed) add_transposed(seed, TL::NJT);
     }
     // accumulator element r of tile (it, jt) is S[16it + 4g + r][16jt + m]
     if (sin != nullptr) {
@@ -684,19 +701,7 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
                 if (i0 + q < di && j < dj) S[u][q] += sin[(size_t)(i0 + q) * lds + j];
         }
     }
-    if (io.ext != nullptr) {
-        // element [16it + 4g + q][16jt + m] of this state is element [16jt + m][16it + 4g + q] of the saved one:
-        // its tile (jt, it), lane (g' = m / 4, m' = 4g + q), component m % 4
-#pragma unroll
-        for (int u = 0; u < TL::TPW; ++u) {
-            const int t = w * TL::TPW + u;
-            const int it = t / TL::NJT, jt = t % TL::NJT;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (16 * it + 4 * g + q < di && 16 * jt + m < dj)  // (tiles outside the real dims are never written)
-                    S[u][q] += io.ext[((size_t)(jt * io.njt + it) * 64 + ((m >> 2) * 16 + 4 * g + q)) * 4 + (m & 3)];
-        }
-    }
+    if (io.ext != nullptr) add_transposed(io.ext, io.njt);  // the state the forward pass saved is this one's transpose
     auto put_state = [&](u16 *dst) {
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) {
