@@ -61,6 +61,16 @@ def _workspace(nbytes, device):
 # The host side of a call costs about as much as the kernels of a small problem run, so the fixed parts are kept
 # short: workspace sizes are remembered per shape, the device is only switched when it is not the current one, and
 # the stream handle comes from torch's raw accessor.
+_CACHE_LIMIT = 4096  # shapes remembered per cache; a caller that sweeps sequence lengths starts over, it does not grow
+
+
+def _remember(cache, key, value):
+    if len(cache) >= _CACHE_LIMIT:
+        cache.clear()
+    cache[key] = value
+    return value
+
+
 _ws_bytes_cache = {}
 
 
@@ -68,7 +78,7 @@ def _ws_bytes(query, *key):
     k = (query, key)
     n = _ws_bytes_cache.get(k)
     if n is None:
-        n = _ws_bytes_cache[k] = getattr(_loader.lib(), query)(*key)
+        n = _remember(_ws_bytes_cache, k, getattr(_loader.lib(), query)(*key))
     return n
 
 
@@ -171,7 +181,7 @@ def saved_states_plan(dtype, b, h, n, dk, dv):
         rc = _loader.lib().cott_causal_saved_plan(b, h, n, dk, dv, _DTYPES[dtype], ctypes.byref(cpc),
                                                   ctypes.byref(cuts), ctypes.byref(slot), ctypes.byref(ws))
         _check(rc, "cott_causal_saved_plan")
-        plan = _saved_plan_cache[key] = (cpc.value, cuts.value, slot.value, ws.value) if cuts.value > 0 else None
+        plan = _remember(_saved_plan_cache, key, (cpc.value, cuts.value, slot.value, ws.value) if cuts.value > 0 else None)
     return plan
 
 
@@ -214,8 +224,8 @@ def fused_preparation_supported(dtype, b, h, n, dk, dv, rotary_dim=0):
     key = (dtype, b, h, n, dk, dv, rotary_dim)
     ok = _prep_supported_cache.get(key)
     if ok is None:
-        ok = _prep_supported_cache[key] = bool(
-            _loader.lib().cott_causal_fwd_prep_supported(b, h, n, dk, dv, _DTYPES[dtype], rotary_dim))
+        ok = _remember(_prep_supported_cache, key, bool(
+            _loader.lib().cott_causal_fwd_prep_supported(b, h, n, dk, dv, _DTYPES[dtype], rotary_dim)))
     return ok
 
 
