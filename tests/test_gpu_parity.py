@@ -690,6 +690,40 @@ def test_calls_can_be_captured_in_a_hip_graph_and_replayed(ct, oracle):
         for got, want in zip((dq, dk, dv), want_g):
             assert torch.equal(got, want), f"replay {rep}"
 
+    # the same pair as a training step runs it: the forward leaves its states, the backward takes them (both a shape
+    # cut into groups and one with pair workgroups of one group each)
+    import ctypes
+    for bb, hh, n in ((1, 2, 1023), (8, 16, 512)):
+        q, k, v, do = (x.to(DEV) for x in inputs(bb, hh, n, 64, 64, BF, seed=50))
+        plan = ct.saved_states_plan(BF, bb, hh, n, 64, 64)
+        assert plan is not None
+        cpc, cuts, slot, nb = plan
+        o = torch.empty_like(v); dq = torch.empty_like(q); dk = torch.empty_like(k); dv = torch.empty_like(v)
+        saved = torch.empty(bb, hh, cuts, slot, device=DEV)
+        nf = L.cott_causal_workspace_bytes(bb, hh, n, 64, 64, _loader.BF16)
+        wsf = torch.empty(max(nf, 16), dtype=torch.uint8, device=DEV); wsb = torch.empty(max(nb, 16), dtype=torch.uint8, device=DEV)
+        sp = ctypes.cast(saved.data_ptr(), ctypes.c_void_p)
+        graph3 = torch.cuda.CUDAGraph()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.graph(graph3, stream=side):
+            st = torch.cuda.current_stream().cuda_stream
+            assert L.cott_causal_fwd_save(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), sp, cpc, cuts, bb, hh, n,
+                                          64, 64, _loader.BF16, wsf.data_ptr() if nf else None, nf, st) == 0
+            assert L.cott_causal_bwd_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), dq.data_ptr(),
+                                           dk.data_ptr(), dv.data_ptr(), sp, cpc, cuts, bb, hh, n, 64, 64, _loader.BF16,
+                                           wsb.data_ptr() if nb else None, nb, st) == 0
+        for rep in range(3):
+            new = [x.to(DEV) for x in inputs(bb, hh, n, 64, 64, BF, seed=60 + rep)]
+            for dst, src in zip((q, k, v, do), new):
+                dst.copy_(src)
+            graph3.replay()
+            want_o, want_s = ct.causal_dot_product_saving(*new[:3])
+            want_g = ct.causal_backward(*new, saved=want_s)
+            torch.cuda.synchronize()
+            assert torch.equal(o, want_o) and torch.equal(saved, want_s), f"replay {rep}"
+            for got, want in zip((dq, dk, dv), want_g):
+                assert torch.equal(got, want), f"replay {rep}"
+
 
 FUSED_PREP_CASES = [
     # b, h, n, dk, dv, dtype, rotary_dim, projections' layout, masked   launch form
