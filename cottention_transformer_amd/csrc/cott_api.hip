@@ -213,10 +213,14 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
         best_h = 1;
         best_g = (int)g_of[1];
     }
-    // Non-causal forward with more heads than CUs: the one-workgroup-per-head kernel runs its two passes over a short
-    // sequence, and twice as many half-width workgroups keep more requests in flight (B32 H12 N512 D64: 21.3 -> 20.7 us,
-    // 31.3 -> 28.6 us with cold caches; with 192 heads the whole problems are faster, 12.5 against 14.3 us).
-    if (!causal && nops == 1 && can_split && pol != 0 && BH > tgt && g_of[1] == 1 && g_of[2] == 1) best_h = 2;
+    // Non-causal forward of small heads, more heads than CUs but at most half of the workgroups that can be resident
+    // (three per CU): the one-workgroup-per-head kernel runs its two passes over a short sequence, and twice as many
+    // half-width workgroups fill the chip (B32 H12 N512 D64: 21.3 -> 20.7 us, 31.0 -> 28.1 us with cold caches; N2048:
+    // 113 -> 108 us).  Outside that range whole problems are faster (192 heads: 12.5 against 14.3 us; 768 heads: 34.3
+    // against 38.4 us; 480 heads at N1024: 41.9 against 45.6 us; 128-wide heads: 53.5 against 56.6 us).
+    if (!causal && nops == 1 && can_split && pol != 0 && BH > tgt && 2 * BH <= 3 * tgt && di <= 64 && dj <= 64 &&
+        g_of[1] == 1 && g_of[2] == 1)
+        best_h = 2;
     p.halves = best_h;
     p.cpg = (p.nchunks + best_g - 1) / best_g;
     p.G = (p.nchunks + p.cpg - 1) / p.cpg;

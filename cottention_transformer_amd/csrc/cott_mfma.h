@@ -1250,7 +1250,7 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
 // S = B^T C over the whole sequence in fp32 accumulators (the group_state loop), pass 2 applies
 // out = A S chunk by chunk with the 16-bit state held in registers.  No workspace, one launch.
 // PF2: chunks of A rows in flight in pass 2.  PF2 > PF: the first PF2 chunks are requested before pass 1 starts instead
-// of at the hand-over (short sequences, three gradient problems per head: B32 H12 N512 D64 gradients 46.6 -> 43.0 us;
+// of at the hand-over (sequences of 4 to 8 chunks, three gradient problems per head: B32 H12 N512 D64 gradients 46.6 -> 43.0 us;
 // the forward pass alone loses 0.7 us of 21.4 with it and keeps PF2 = PF; 3, 4 and 6 chunks measured alike, 8 worse).
 template <class TR, int DI, int DJ, int PF, int PF2 = PF>
 __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int BH, int N, int nchunks) {
