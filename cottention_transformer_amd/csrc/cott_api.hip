@@ -213,6 +213,15 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
         best_h = 1;
         best_g = (int)g_of[1];
     }
+    // Three gradient problems that fill the chip equally as column halves of one group or as whole problems in groups:
+    // whole problems let dQ walk with dK and dV (complement form, shared tiles, saved states), which outweighs the
+    // group-state pass once a group has 64 chunks (B2 H16 D128 gradients, N8192: 196 -> 183 us, 168 with saved states;
+    // N16384: 404 -> 340 / 308 us; N4096: 79 against 98 / 89 us, halves kept).
+    if (causal && nops == 3 && best_h == 2 && g_of[2] == 1 && g_of[1] > 1 && cpg_of[1] >= 64 &&
+        BH * nops * g_of[1] <= tgt && pol < 0) {
+        best_h = 1;
+        best_g = (int)g_of[1];
+    }
     // Non-causal forward of small heads, more heads than CUs but at most half of the workgroups that can be resident
     // (three per CU): the one-workgroup-per-head kernel runs its two passes over a short sequence, and twice as many
     // half-width workgroups fill the chip (B32 H12 N512 D64: 21.3 -> 20.7 us, 31.0 -> 28.1 us with cold caches; N2048:
@@ -803,9 +812,10 @@ bool saved_states_plan(long BH, int N, int Dk, int Dv, int dtype, int *cpg, int 
     // dQ takes the states where it runs in complement form: in sets cut into groups, and beside a (dK, dV) pair
     // (there also when a head is one group: the one slot is then the sum over the whole sequence)
     if (!L.pair && !L.complement) return false;
-    // Sequences of a few chunks gain nothing from it, and their rows would lose precision: in complement form the
-    // rows of the first chunk are a difference of two sums rounded to 16 bits instead of one short sum.
-    if (L.p.nchunks < 8) return false;
+    // Sequences of a few chunks gain nothing from it (at 8 chunks the extra tensor costs the host side of the call more
+    // than the kernels gain), and their rows would lose precision: in complement form the rows of the first chunk are
+    // a difference of two sums rounded to 16 bits instead of one short sum.
+    if (L.p.nchunks < 16) return false;
     *cpg = L.p.cpg;
     *ncuts = L.p.G;
     if (bwd_ws) {

@@ -113,7 +113,7 @@ COTT_API int cott_causal_bwd(const void *q, const void *k, const void *v, const 
  * ctx.save_for_backward) grows by one small tensor.
  *   cott_causal_saved_plan   chunks_per_cut, ncuts (0 = this shape's backward pass takes no saved states: use the
  *                            plain entry points), the floats per saved slot and the workspace
- *                            cott_causal_bwd_saved needs.  Plans exist for sequences of 8 chunks or more whose
+ *                            cott_causal_bwd_saved needs.  Plans exist for sequences of 16 chunks or more whose
  *                            gradients run as dq beside a (dk, dv) pair of workgroups (square head dims up to 64)
  *                            or as three problems cut into sequence groups.
  *   cott_causal_fwd_save     cott_causal_fwd (not reversed; same o, bit for bit) that also writes

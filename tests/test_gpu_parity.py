@@ -693,7 +693,7 @@ def test_calls_can_be_captured_in_a_hip_graph_and_replayed(ct, oracle):
     # the same pair as a training step runs it: the forward leaves its states, the backward takes them (both a shape
     # cut into groups and one with pair workgroups of one group each)
     import ctypes
-    for bb, hh, n in ((1, 2, 1023), (8, 16, 512)):
+    for bb, hh, n in ((1, 2, 1023), (8, 16, 1024)):
         q, k, v, do = (x.to(DEV) for x in inputs(bb, hh, n, 64, 64, BF, seed=50))
         plan = ct.saved_states_plan(BF, bb, hh, n, 64, 64)
         assert plan is not None
