@@ -165,7 +165,8 @@ bool pair_eligible(const Op *ops, int n, int dtype, bool causal) {
     return true;
 }
 
-SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtype, bool no_split = false) {
+SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtype, bool no_split = false,
+                 bool has_ext = false) {
     SetPlan p;
     // the fp32 kernels are MFMA-bound with four wavefronts per workgroup: two workgroups per CU overlap well
     const long tgt = target_workgroups() * (dtype == COTT_F32 ? 2 : 1);
@@ -213,14 +214,20 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
         best_h = 1;
         best_g = (int)g_of[1];
     }
-    // Three gradient problems that fill the chip equally as column halves of one group or as whole problems in groups:
-    // whole problems let dQ walk with dK and dV (complement form, shared tiles, saved states), which outweighs the
-    // group-state pass once a group has 64 chunks (B2 H16 D128 gradients, N8192: 196 -> 183 us, 168 with saved states;
-    // N16384: 404 -> 340 / 308 us; N4096: 79 against 98 / 89 us, halves kept).
-    if (causal && nops == 3 && best_h == 2 && g_of[2] == 1 && g_of[1] > 1 && cpg_of[1] >= 64 &&
-        BH * nops * g_of[1] <= tgt && pol < 0) {
-        best_h = 1;
-        best_g = (int)g_of[1];
+    // Three gradient problems of few heads that fit the chip either as column halves of ONE group or as whole
+    // problems in groups.  Whole problems let dQ walk with dK and dV (complement form, shared tiles) at the price of
+    // the group-state and prefix passes, which pays from some group length on.  Measured on 128-wide heads, with /
+    // without the states the forward pass leaves for dQ: when the groups give more workgroups than the halves
+    // (B3 H8: 216 against 144) from 16 / 32 chunks per group (N4096, groups of 22: 71 us with states, 84 without,
+    // halves 80; N8192: 124 / 146 / 171 us); when both give the same number (B4 H8, B5 H8) from 64 / 128 chunks
+    // (B4 H8 N8192, groups of 64: 167 / 184 us, halves 196; N4096: 89 / 98 us, halves 80).
+    if (causal && nops == 3 && can_split && pol < 0 && g_of[2] == 1 && g_of[1] > 1 && BH * nops * 2 <= tgt &&
+        BH * nops * g_of[1] <= tgt) {
+        const bool fuller = g_of[1] > 2;
+        const int from = fuller ? (has_ext ? 16 : 32) : (has_ext ? 64 : 128);
+        const bool groups = cpg_of[1] >= from;
+        best_h = groups ? 1 : 2;
+        best_g = groups ? (int)g_of[1] : 1;
     }
     // Non-causal forward of small heads, more heads than CUs but at most half of the workgroups that can be resident
     // (three per CU): the one-workgroup-per-head kernel runs its two passes over a short sequence, and twice as many
@@ -265,8 +272,10 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
     const Op &first = ops[members[0]];
     const bool half = dtype == COTT_BF16 || dtype == COTT_F16;
     L.pair = use_pair(ops, n, BH, N, dtype, causal);  // then all three ops are in this set
+    bool has_ext = false;
+    for (int c = 0; c < cnt; ++c) has_ext = has_ext || ops[members[c]].ext != nullptr;
     L.p = L.pair ? plan_set(BH, N, 2, first.di, first.dj, causal, dtype, true)
-                 : plan_set(BH, N, cnt, first.di, first.dj, causal, dtype);
+                 : plan_set(BH, N, cnt, first.di, first.dj, causal, dtype, false, has_ext);
     const SetPlan &p = L.p;
     // Gradient sets cut into sequence groups: the op that sums over the past (dQ) is put in complement form and
     // walks the sequence from the end like the two that sum over the future, so the three workgroups of a head
