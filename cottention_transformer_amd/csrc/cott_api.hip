@@ -250,11 +250,15 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
 
 // Whether the backward set runs as dQ + (dK, dV) pair.  The pair workgroup is heavier than a single problem, so
 // when the three separate problems already fit the chip in one round without sequence groups (more than half and at
-// most all of the CUs), they finish sooner (33 us against 41 us at B*H = 64, N = 2048, D = 64).
+// most all of the CUs), they finish sooner (33 us against 41 us at B*H = 64, N = 2048, D = 64) ...
 bool use_pair(const Op *ops, int n, long BH, int N, int dtype, bool causal) {
     if (!pair_eligible(ops, n, dtype, causal)) return false;
     const SetPlan u = plan_set(BH, N, 3, ops[0].di, ops[0].dj, causal, dtype);
-    return !(u.G == 1 && u.halves == 1 && 3 * BH <= target_workgroups());
+    if (!(u.G == 1 && u.halves == 1 && 3 * BH <= target_workgroups())) return true;
+    // ... unless the forward pass has left the states dQ starts from and the sequence is long: the pair's workgroups
+    // (in two groups) then share every tile with dQ's, which the three separate problems cannot (B6 H8 D64 N8192:
+    // 96 against 113 us, N16384: 179 against 225 us; N4096: 51 against 51 us, N2048: 34 against 28 us).
+    return ops[0].ext != nullptr && (N + 63) / 64 >= 128;
 }
 
 int pad_key(const Op &o) { return cott::mfma_pad(o.di) * 1000 + cott::mfma_pad(o.dj); }
