@@ -229,6 +229,20 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
         best_h = groups ? 1 : 2;
         best_g = groups ? (int)g_of[1] : 1;
     }
+    // A forward pass (one problem per head) of 65..128 heads, likewise: column halves of one group (twice the score
+    // products, q and k read twice through L2) against whole problems in groups (one more pass over part of k and
+    // v, two more launches).  Where the groups give more workgroups (65..85 heads: three groups) they win from 16
+    // chunks per group for 128 x 128 tiles and from 32 for smaller ones (B9 H8 D128 N4096, groups of 22: 88 against
+    // 102 us, N2048: 56 against 41 us; D64 N8192, groups of 43: 73 against 97 us, N4096: 45 against 38 us); where both
+    // give the same number they win from 64 chunks as long as the chip is not nearly full (B11 H8 D128 N16384: 361
+    // against 420 us, B13 H8: 404 against 437 us, B15 H8: 473 against 472 us).
+    if (causal && nops == 1 && can_split && pol < 0 && g_of[2] == 1 && g_of[1] > 1 && BH * 2 <= tgt &&
+        BH * g_of[1] <= tgt) {
+        const bool wide = cott::mfma_pad(di) * cott::mfma_pad(dj) >= 128 * 128;
+        const bool groups = g_of[1] > 2 ? cpg_of[1] >= (wide ? 16 : 32) : (cpg_of[1] >= 64 && 2 * BH * 20 <= tgt * 17);
+        best_h = groups ? 1 : 2;
+        best_g = groups ? (int)g_of[1] : 1;
+    }
     // Non-causal forward of small heads, more heads than CUs but at most half of the workgroups that can be resident
     // (three per CU): the one-workgroup-per-head kernel runs its two passes over a short sequence, and twice as many
     // half-width workgroups fill the chip (B32 H12 N512 D64: 21.3 -> 20.7 us, 31.0 -> 28.1 us with cold caches; N2048:
