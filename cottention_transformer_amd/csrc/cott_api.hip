@@ -210,7 +210,12 @@ SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtyp
     // the last is read twice either way) and only repeat the score tiles: whole problems in twice as many groups
     // are faster as long as a group keeps 16 or more chunks (measured on B*H = 16..96, N = 2k..64k, D = 64..128:
     // 3 to 25 % faster forward; with 4 or 8 chunks per group the halves win by 15 to 20 %).
-    if (best_h == 2 && g_of[1] > 1 && g_of[2] > 1 && cpg_of[1] >= 16) {
+    // A forward pass of 64 x 64 tiles whose whole problems would only fill the same number of workgroups as the
+    // halves (twice the groups) needs groups of 32 chunks (B8 H8 D64 N4096..6144, groups of 16..24: halves in two
+    // groups 35 / 41 / 46 us against 39 / 44 / 50 us; N8192, groups of 32: 69 against 66 us).
+    const bool small_tiles = cott::mfma_pad(di) * cott::mfma_pad(dj) <= 64 * 64;
+    const int whole_from = (nops == 1 && g_of[1] == 2 * g_of[2] && small_tiles) ? 32 : 16;
+    if (best_h == 2 && g_of[1] > 1 && g_of[2] > 1 && cpg_of[1] >= whole_from) {
         best_h = 1;
         best_g = (int)g_of[1];
     }
