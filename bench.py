@@ -319,6 +319,10 @@ def gpt_block_step(torch, dev):
     gout = torch.randn(8, 2048, 1024, device=dev, dtype=torch.bfloat16)
 
     def step(use_cache):
+        # gradients start from None, as after a training loop's zero_grad(set_to_none=True): the hidden states of a
+        # model are no leaf, so accumulating into hid.grad would add a 64 MiB pass that no training step has
+        hid.grad = None
+        blk.zero_grad(set_to_none=True)
         with torch.autocast("cuda", dtype=torch.bfloat16):
             out = blk(hid, use_cache=use_cache)[0]
         out.backward(gout)
@@ -483,6 +487,8 @@ def run_extras(torch, ct, dev):
     bg = torch.randn(32, 512, 768, device=dev, dtype=torch.bfloat16)
 
     def bert_step():
+        bh_in.grad = None
+        bert.zero_grad(set_to_none=True)
         with torch.autocast("cuda", dtype=torch.bfloat16):
             out = bert(bh_in)[0]
         out.backward(bg)

@@ -189,3 +189,69 @@ class PreparedCausalAttention(torch.autograd.Function):
         if dsig is not None:
             dsig = dsig.to(sig.dtype)
         return dq, dk, dv, None, None, dsig, None, None, None, None
+
+
+def _weight_gradient(gy, x):
+    """gy^T x for gy (R, out), x (R, in).  With many rows and a small weight the library's single GEMM fills the
+    chip with too few tiles over a long reduction (out = in = 1024, R = 16384, bf16: 109 us); the rows are cut into
+    pieces multiplied as one batched GEMM and summed in fp32 instead (8 pieces: 47 us)."""
+    r = x.shape[0]
+    pieces = 1
+    if x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and gy.shape[1] * x.shape[1] <= 1 << 20:
+        while pieces < 16 and r % (2 * pieces) == 0 and r // (2 * pieces) >= 2048:
+            pieces *= 2
+    if pieces == 1:
+        return gy.t() @ x
+    parts = torch.bmm(gy.view(pieces, r // pieces, -1).transpose(1, 2), x.view(pieces, r // pieces, -1))
+    return parts.sum(0, dtype=torch.float32)
+
+
+class InputProjections(torch.autograd.Function):
+    """(x, w_0, b_0, w_1, b_1, ...) -> (x w_0^T + b_0, x w_1^T + b_1, ...): the q / k / v projections of an attention
+    block (GPT_Trainer/GPTCosAttention.py:447-449, BERT_Trainer/BertCosAttention.py:253-255 with biases) as one
+    operator.  Under autocast x is converted once for all of them, the gradient of x is accumulated by the GEMMs
+    themselves and converted back once, and the weight gradients take `_weight_gradient`.  b_i may be None."""
+
+    @staticmethod
+    def forward(ctx, x, *wb):
+        # the type nn.Linear would compute in: the autocast type for 16- and 32-bit inputs on the GPU, else x's own
+        cd = x.dtype
+        if x.is_cuda and x.dtype != torch.float64 and torch.is_autocast_enabled("cuda"):
+            cd = torch.get_autocast_dtype("cuda")
+        x2 = x.reshape(-1, x.shape[-1]).to(cd)
+        ws = [w.to(cd) for w in wb[0::2]]
+        ctx.save_for_backward(x2, *ws)
+        ctx.x_meta = (x.shape, x.dtype)
+        ctx.wb_dtypes = [None if t is None else t.dtype for t in wb]
+        outs = []
+        for w, b in zip(ws, wb[1::2]):
+            y = torch.nn.functional.linear(x2, w, None if b is None else b.to(cd))
+            outs.append(y.view(x.shape[:-1] + (w.shape[0],)))
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *gys):
+        x2, *ws = ctx.saved_tensors
+        shape, xdt = ctx.x_meta
+        gys = [g.reshape(-1, g.shape[-1]).to(x2.dtype) for g in gys]
+        gx = None
+        if ctx.needs_input_grad[0]:
+            gx = gys[0] @ ws[0]
+            for g, w in zip(gys[1:], ws[1:]):
+                gx.addmm_(g, w)
+            gx = gx.view(shape).to(xdt)
+        grads = [gx]
+        for i, g in enumerate(gys):
+            wdt, bdt = ctx.wb_dtypes[2 * i], ctx.wb_dtypes[2 * i + 1]
+            grads.append(_weight_gradient(g, x2).to(wdt) if ctx.needs_input_grad[1 + 2 * i] else None)
+            grads.append(g.sum(0, dtype=torch.promote_types(g.dtype, torch.float32)).to(bdt)
+                         if bdt is not None and ctx.needs_input_grad[2 + 2 * i] else None)
+        return tuple(grads)
+
+
+def project(x, *linears):
+    """The outputs of the given nn.Linear layers on x, through `InputProjections`."""
+    args = []
+    for lin in linears:
+        args += [lin.weight, lin.bias]
+    return InputProjections.apply(x, *args)

@@ -16,7 +16,7 @@ from torch import nn
 
 from . import ops
 from .autograd import (CustomAttention, CustomAttentionMergedHeads, NonCausalAttention,
-                       NonCausalAttentionMergedHeads, PreparedCausalAttention, PrepareInputs, _autocast_target)
+                       NonCausalAttentionMergedHeads, PreparedCausalAttention, PrepareInputs, _autocast_target, project)
 
 
 def _autocast_on():
@@ -175,9 +175,8 @@ class GPTCosAttention(nn.Module):
 
     def forward(self, hidden_states, layer_past=None, attention_mask=None, position_ids=None, head_mask=None,
                 use_cache=False, output_attentions=False):
-        query = self._split_heads(self.q_proj(hidden_states))          # (B,S,H,D)
-        key = self._split_heads(self.k_proj(hidden_states))
-        value = self._split_heads(self.v_proj(hidden_states))
+        query, key, value = (self._split_heads(t)                       # (B,S,H,D)
+                             for t in project(hidden_states, self.q_proj, self.k_proj, self.v_proj))
         if (self.fast_inference and hidden_states.shape[1] == 1 and position_ids is None and layer_past is None
                 and use_cache is not True and not output_attentions and attention_mask is None
                 and self.head_dim in (32, 64, 128, 256) and self.rotary_dim is not None
@@ -185,7 +184,7 @@ class GPTCosAttention(nn.Module):
             attn_output = self._decode_one(query, key, value)
             if not _autocast_on():
                 attn_output = attn_output.to(hidden_states.dtype)
-            return (self.resid_dropout(self.out_proj(attn_output)), None)
+            return (self.resid_dropout(project(attn_output, self.out_proj)[0]), None)
         first_position = None
         if position_ids is None:
             start = self.cur_s - 1 if self.fast_inference else 0
@@ -214,7 +213,7 @@ class GPTCosAttention(nn.Module):
         if attn_weights is not None:  # came back (B,H,S,D): merge the heads here (:500)
             attn_output = attn_output.permute(0, 2, 1, 3).contiguous()
         attn_output = attn_output.view(attn_output.size()[:-2] + (self.embed_dim,))
-        attn_output = self.resid_dropout(self.out_proj(attn_output))
+        attn_output = self.resid_dropout(project(attn_output, self.out_proj)[0])
         outputs = (attn_output, present)
         if output_attentions:
             outputs += (attn_weights,)
@@ -250,9 +249,9 @@ class BertCosAttention(nn.Module):
         if head_mask is not None:
             raise NotImplementedError
         split = hidden_states.shape[:-1] + (self.num_attention_heads, self.attention_head_size)
-        query_layer = self.query(hidden_states).view(split)            # (B,S,H,D); the head permute of
-        key_layer = self.key(hidden_states).view(split)                # transpose_for_scores happens inside
-        value_layer = self.value(hidden_states).view(split)            # the preparation pass
+        # (B,S,H,D); the head permute of transpose_for_scores happens inside the preparation pass
+        query_layer, key_layer, value_layer = (t.view(split) for t in
+                                               project(hidden_states, self.query, self.key, self.value))
         b, s, h, _ = query_layer.shape
         # mask, normalise, divide the values by (number of real tokens) ** sigmoid(norm_const)  (:162-178)
         keep = _keep_from_additive_mask(attention_mask, b, s, query_layer.device)

@@ -168,3 +168,40 @@ def test_bert_block_forward_backward(mods, autocast):
     got = [hd.grad, m.query.weight.grad, m.key.weight.grad, m.value.weight.grad, m.norm_const.grad.reshape(-1)]
     for name, a, r in zip(("hidden", "wq", "wk", "wv", "norm_const"), got, ref_grads):
         assert rel_l2(a.float(), r.numpy()) <= tol, name
+
+
+@pytest.mark.parametrize("autocast", [False, True], ids=["bf16-input", "autocast-bf16"])
+def test_input_projections_with_the_row_split_weight_gradient(mods, autocast):
+    """`InputProjections` at a row count where the weight gradient is multiplied in pieces (8192 rows: four pieces),
+    with and without biases, against fp64 linear layers on the CPU."""
+    from cottention_transformer_amd.autograd import _weight_gradient, project
+    say("input projections", autocast)
+    torch.manual_seed(5)
+    rows, e = 8192, 128
+    lins = [torch.nn.Linear(e, 64 * (i + 1), bias=(i != 1)).to(DEV) for i in range(3)]
+    x = torch.randn(4, rows // 4, e)
+    gs = [torch.randn(4, rows // 4, 64 * (i + 1)) for i in range(3)]
+    x64 = x.double().requires_grad_(True)
+    ref_par = [[p.detach().double().cpu().requires_grad_(True) for p in lin.parameters()] for lin in lins]
+    ref_ys = [torch.nn.functional.linear(x64, *ps) for ps in ref_par]
+    ref_grads = torch.autograd.grad(ref_ys, [x64] + [p for ps in ref_par for p in ps], [g.double() for g in gs])
+    xd = x.to(DEV)
+    if not autocast:
+        xd = xd.bfloat16()
+        lins = [lin.bfloat16() for lin in lins]
+    xd.requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        ys = project(xd, *lins)
+    assert all(y.dtype == torch.bfloat16 for y in ys)
+    for y, r in zip(ys, ref_ys):
+        assert rel_l2(y.float(), r.detach().numpy()) <= 1e-2
+    torch.autograd.backward(ys, [g.to(DEV).bfloat16() for g in gs])
+    got = [xd.grad] + [p.grad for lin in lins for p in lin.parameters()]
+    assert xd.grad.dtype == xd.dtype and all(p.grad.dtype == p.dtype for lin in lins for p in lin.parameters())
+    for a, r in zip(got, ref_grads):
+        assert rel_l2(a.float(), r.numpy()) <= 1e-2
+    # the pieces are what ran: the same product as one GEMM differs in the last bits only
+    gy, x2 = gs[0].reshape(rows, -1).to(DEV).bfloat16(), x.reshape(rows, e).to(DEV).bfloat16()
+    pieces = _weight_gradient(gy, x2)
+    assert pieces.dtype == torch.float32
+    assert rel_l2(pieces, (gy.double().t() @ x2.double()).cpu().numpy()) <= 1e-2

@@ -99,3 +99,28 @@ def test_dropin_module_files_resolve_like_the_reference_imports():
         assert getattr(mod, name) is getattr(modules, name)
         pkg = importlib.import_module(f"cottention_transformer_amd.{sub}.{name}")
         assert getattr(pkg, name) is getattr(modules, name)
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_input_projections_equal_separate_linear_layers(bias):
+    """`InputProjections` (one operator for the q / k / v projections) against three nn.Linear calls: same outputs,
+    same gradients for the input, the weights and the biases."""
+    from cottention_transformer_amd.autograd import project
+    torch.manual_seed(3)
+    lins = [torch.nn.Linear(24, 16 + 8 * i, bias=bias).double() for i in range(3)]
+    x = torch.randn(2, 5, 24, dtype=torch.float64, requires_grad=True)
+    gs = [torch.randn(2, 5, 16 + 8 * i, dtype=torch.float64) for i in range(3)]
+    ys = project(x, *lins)
+    torch.autograd.backward(ys, gs)
+    got = [x.grad.clone()] + [p.grad.clone() for lin in lins for p in lin.parameters()]
+    x.grad = None
+    for lin in lins:
+        lin.zero_grad()
+    ref_ys = [lin(x) for lin in lins]
+    torch.autograd.backward(ref_ys, gs)
+    ref = [x.grad.clone()] + [p.grad.clone() for lin in lins for p in lin.parameters()]
+    for a, b in zip(ys, ref_ys):
+        assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
+    assert len(got) == len(ref)
+    for a, b in zip(got, ref):
+        assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
