@@ -215,3 +215,62 @@ def test_random_shapes_every_16_bit_path_against_the_fp32_kernels(ct):
         assert max(errs) <= TOL[dt], (it, errs)
         worst = max(worst, max(errs))
     say(f"worst error over all cases and paths: {worst:.2e}")
+
+
+# Shapes on either side of the launch planner's measured thresholds (column halves of one group against whole problems
+# in groups, by heads, tile size and group length; pair workgroups for few small heads on long sequences; the
+# non-causal column halves): every plan the rules choose between runs at a size where the rule applies.
+PLANNER_CASES = [
+    (9, 8, 1024, 128, 128, BF),    # forward of 72 wide heads, short groups: column halves of one group
+    (9, 8, 4096, 128, 128, BF),    # ... groups of 22 chunks: whole problems in three groups
+    (11, 8, 8192, 128, 128, HF),   # 88 wide heads, two groups of 64 chunks
+    (8, 8, 4096, 64, 64, BF),      # 64 small heads: column halves in two groups (whole problems would get 16 chunks)
+    (8, 8, 8192, 64, 64, BF),      # ... whole problems in four groups of 32 chunks
+    (3, 8, 4096, 128, 128, BF),    # gradients of 24 wide heads: groups of 22 chunks with saved states, halves without
+    (4, 8, 8192, 128, 128, BF),    # gradients of 32 wide heads: groups of 64 chunks with saved states
+    (4, 8, 4096, 128, 128, HF),    # ... column halves of one group
+    (6, 8, 16384, 64, 64, BF),     # 48 small heads, 256 chunks: pair workgroups once the forward has left its states
+    (5, 16, 2048, 96, 96, BF),     # 80 heads of padded width
+]
+
+
+@pytest.mark.parametrize("case", PLANNER_CASES, ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_shapes_around_the_planner_thresholds_against_the_fp32_kernels(ct, case):
+    b, h, n, dk, dv, dt = case
+    say("planner case", case, "plan", ct.saved_states_plan(dt, b, h, n, dk, dv))
+    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, dk, dv, dt, seed=11))
+
+    def err(a, r):
+        return max(rel_l2(a, r.double().cpu().numpy()), worst_block(a, r.double().cpu().numpy()))
+
+    ref_o = ct.causal_dot_product(q.float(), k.float(), v.float())
+    ref_r = ct.causal_dot_product(q.float(), k.float(), v.float(), reversed=True)
+    ref = ct.causal_backward(q.float(), k.float(), v.float(), do.float())
+    o, saved = ct.causal_dot_product_saving(q, k, v)
+    assert torch.equal(o, ct.causal_dot_product(q, k, v))
+    errs = [err(o, ref_o), err(ct.causal_dot_product(q, k, v, reversed=True), ref_r)]
+    outs = [ct.causal_backward(q, k, v, do)]
+    if saved is not None:
+        outs.append(ct.causal_backward(q, k, v, do, saved=saved))
+    for grads in outs:
+        errs += [err(a, r) for a, r in zip(grads, ref)]
+    assert max(errs) <= TOL[dt], errs
+
+
+@pytest.mark.parametrize("case", [(48, 8, 512, 64, 64, BF), (24, 8, 512, 64, 64, HF), (96, 8, 512, 64, 64, BF),
+                                  (40, 12, 384, 128, 128, BF), (48, 8, 300, 64, 32, BF)],
+                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_non_causal_shapes_around_the_planner_thresholds_against_the_fp32_kernels(ct, case):
+    """One workgroup per head with and without column halves (257..384 small heads take halves), four to eight chunks
+    (the A rows of the first chunks are requested before the first pass)."""
+    from cottention_transformer_amd import ops
+    b, h, n, dk, dv, dt = case
+    say("non-causal planner case", case)
+    q, k, v, do = (x.to(DEV) for x in inputs(b, h, n, dk, dv, dt, seed=12))
+    ref_o = ops.noncausal_dot_product(q.float(), k.float(), v.float())
+    ref = ops.noncausal_backward(q.float(), k.float(), v.float(), do.float())
+    errs = [max(rel_l2(ops.noncausal_dot_product(q, k, v), ref_o.double().cpu().numpy()),
+                worst_block(ops.noncausal_dot_product(q, k, v), ref_o.double().cpu().numpy()))]
+    for a, r in zip(ops.noncausal_backward(q, k, v, do), ref):
+        errs += [rel_l2(a, r.double().cpu().numpy()), worst_block(a, r.double().cpu().numpy())]
+    assert max(errs) <= TOL[dt], errs
