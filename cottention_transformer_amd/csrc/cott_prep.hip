@@ -159,8 +159,13 @@ __device__ __forceinline__ void split_row(long row, const PrepArgs &a, int &s, i
 // limited by instruction issue, not by bytes: the per-row work (index split, norm, division) is repeated by
 // every lane of the row, so two groups per lane (half as many wavefronts) are faster than one, while more
 // rows or groups per lane only cost registers.
-template <class ACC, bool BACKWARD, int NV, int R>
+template <class ACC, bool BACKWARD, int NV, int R, bool ALL_BF16 = false>
 __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
+    // ALL_BF16: every tensor is bf16, known at compile time: no type dispatch around the loads and stores (the block's
+    // shapes, B8 H16 N2048 D64 in the projections' layout with rotary, mask and scale: forward 48.5 -> 44.8 us,
+    // backward 97.8 -> 91.5 us per call)
+    const int x_dtype = ALL_BF16 ? (int)COTT_BF16 : a.x_dtype, y_dtype = ALL_BF16 ? (int)COTT_BF16 : a.y_dtype,
+              g_dtype = ALL_BF16 ? (int)COTT_BF16 : a.g_dtype;
     const int t = blockIdx.y;
     const int D = t < 2 ? a.dk : a.dv;
     const int lpr = a.lpr[t];
@@ -199,8 +204,8 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
         for (int c = 0; c < NV; ++c) {
             const int col = 4 * (lane + c * lpr);
             if (act[u] && col < D) {
-                x[u][c] = load4<ACC>(a.x[t], a.x_dtype, xoff[u] + col);
-                if (BACKWARD) g[u][c] = load4<ACC>(a.g[t], a.g_dtype, (size_t)rr[u] * D + col);
+                x[u][c] = load4<ACC>(a.x[t], x_dtype, xoff[u] + col);
+                if (BACKWARD) g[u][c] = load4<ACC>(a.g[t], g_dtype, (size_t)rr[u] * D + col);
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
                 for (int i = 0; i < 4; ++i)
                     y.x[i] = BACKWARD ? mul_g * g[u][c].x[i] + mul_x * x[u][c].x[i] : mul_x * x[u][c].x[i];
                 if (BACKWARD && rotary && col < a.R) rotate4(y, sn[u][c], cs[u][c], true);
-                store4<ACC>(a.y[t], BACKWARD ? a.x_dtype : a.y_dtype, (BACKWARD ? xoff[u] : (size_t)r * D) + col, y);
+                store4<ACC>(a.y[t], BACKWARD ? x_dtype : y_dtype, (BACKWARD ? xoff[u] : (size_t)r * D) + col, y);
             }
         }
     }
@@ -351,9 +356,11 @@ hipError_t launch_prep(bool backward, const void *const x[3], const void *const 
     ProfScope prof(K_PREP, stream);
     const dim3 grid((unsigned)blocks, 3), blk(kPrepThreads);
     const bool f64 = x_dtype == COTT_F64;
+    const bool all_bf16 = x_dtype == COTT_BF16 && y_dtype == COTT_BF16 && (!backward || g_dtype == COTT_BF16);
 #define COTT_PREP(ACC, BWD) \
     do { \
         if (wide) prep_kernel<ACC, BWD, kMaxVec, 1><<<grid, blk, 0, stream>>>(a); \
+        else if (nv == 2 && all_bf16) prep_kernel<ACC, BWD, 2, 2, true><<<grid, blk, 0, stream>>>(a); \
         else if (nv == 2) prep_kernel<ACC, BWD, 2, 2><<<grid, blk, 0, stream>>>(a); \
         else prep_kernel<ACC, BWD, 1, 2><<<grid, blk, 0, stream>>>(a); \
     } while (0)
