@@ -108,6 +108,16 @@ class GPTCosAttention(nn.Module):
         self.cur_s += 1
         return out.reshape(b, 1, h * value.shape[-1])
 
+    def _unmasked_side_inputs(self, b, s, device):
+        """Keep mask (all true) and running count of kept keys (1, 2, ..., s) of a batch without padding: constants,
+        made once per shape instead of with a fill and a cumulative sum in every forward."""
+        cached = getattr(self, "_unmasked_cache", None)
+        if cached is None or cached[0] != (b, s, device):
+            keep = torch.ones(b, s, dtype=torch.bool, device=device)
+            cnt = torch.arange(1, s + 1, device=device, dtype=torch.float32)[None, :].expand(b, s).contiguous()
+            cached = self._unmasked_cache = ((b, s, device), keep, cnt)
+        return cached[1], cached[2]
+
     def _split_heads(self, tensor):
         return tensor.view(tensor.size()[:-1] + (self.num_attention_heads, self.head_dim))  # (B,S,H,D)
 
@@ -140,7 +150,10 @@ class GPTCosAttention(nn.Module):
         else:
             b, h, s, _ = query.shape
         query, key, value = _common_dtype(query, key, value)
-        keep = _keep_from_additive_mask(attention_mask, b, s, query.device)
+        if attention_mask is None:
+            keep, cnt_all = self._unmasked_side_inputs(b, s, query.device)
+        else:
+            keep, cnt_all = _keep_from_additive_mask(attention_mask, b, s, query.device), None
         sig = self.norm_const.sigmoid().reshape(h)
         table, pos = rotary if rotary is not None else (None, None)
         if self.fast_inference:
@@ -158,7 +171,8 @@ class GPTCosAttention(nn.Module):
                 out, self.state = ops.causal_prefill(q, k, v, state=self.state)
             self.cur_s += s
             return out, out
-        cnt = keep.to(torch.float32).cumsum(-1)                        # kept keys at positions <= s (:241)
+        # kept keys at positions <= s (:241)
+        cnt = cnt_all if cnt_all is not None else keep.to(torch.float32).cumsum(-1)
         dt = _autocast_target(query)
         if (bnhd and first_position is not None and merge_heads and query.dtype == dt
                 and ops.fused_preparation_supported(dt, b, h, s, query.shape[-1], value.shape[-1],
@@ -188,8 +202,12 @@ class GPTCosAttention(nn.Module):
         first_position = None
         if position_ids is None:
             start = self.cur_s - 1 if self.fast_inference else 0
-            position_ids = torch.arange(start, start + hidden_states.shape[1], device=hidden_states.device)
-            position_ids = position_ids[None, :].expand(hidden_states.shape[0], -1)
+            key_ = (start, hidden_states.shape[0], hidden_states.shape[1], hidden_states.device)
+            cached = getattr(self, "_position_cache", None)
+            if cached is None or cached[0] != key_:  # the same ids every training step: made once
+                ids = torch.arange(start, start + hidden_states.shape[1], device=hidden_states.device)
+                cached = self._position_cache = (key_, ids[None, :].expand(hidden_states.shape[0], -1))
+            position_ids = cached[1]
             first_position = start
         if layer_past is None and use_cache is not True and self.rotary_dim is not None and self.rotary_dim % 4 == 0:
             # nobody needs the rotated keys themselves: rotation, head permute and preparation in one pass
@@ -254,8 +272,16 @@ class BertCosAttention(nn.Module):
                                                project(hidden_states, self.query, self.key, self.value))
         b, s, h, _ = query_layer.shape
         # mask, normalise, divide the values by (number of real tokens) ** sigmoid(norm_const)  (:162-178)
-        keep = _keep_from_additive_mask(attention_mask, b, s, query_layer.device)
-        cnt = keep.sum(-1, keepdim=True).to(torch.float32).expand(b, s)
+        if attention_mask is None:  # no padding: constants, made once per shape
+            cached = getattr(self, "_unmasked_cache", None)
+            if cached is None or cached[0] != (b, s, query_layer.device):
+                cached = self._unmasked_cache = ((b, s, query_layer.device),
+                                                 torch.ones(b, s, dtype=torch.bool, device=query_layer.device),
+                                                 torch.full((b, s), float(s), device=query_layer.device))
+            keep, cnt = cached[1], cached[2]
+        else:
+            keep = _keep_from_additive_mask(attention_mask, b, s, query_layer.device)
+            cnt = keep.sum(-1, keepdim=True).to(torch.float32).expand(b, s)
         dt = _autocast_target(query_layer)
         q, k, v = PrepareInputs.apply(query_layer, key_layer, value_layer, keep, cnt, self.norm_const.sigmoid().reshape(h),
                                       dt, None, None, True)

@@ -205,3 +205,31 @@ def test_input_projections_with_the_row_split_weight_gradient(mods, autocast):
     pieces = _weight_gradient(gy, x2)
     assert pieces.dtype == torch.float32
     assert rel_l2(pieces, (gy.double().t() @ x2.double()).cpu().numpy()) <= 1e-2
+
+
+def test_blocks_without_a_mask_reuse_their_constant_side_inputs(mods):
+    """No attention mask: the keep mask, the counts and the position ids are constants the blocks make once per
+    shape.  Two calls in a row (the second on the cached tensors) and a call at another shape, against the CPU
+    statements with an all-true mask."""
+    from oracle import torch_forms as tf
+    torch.manual_seed(0)
+    cfg = gpt_cfg()
+    gpt = mods.GPTCosAttention(cfg).to(DEV)
+    bcfg = SimpleNamespace(hidden_size=256, num_attention_heads=4, attention_probs_dropout_prob=0.0, is_decoder=False)
+    bert = mods.BertCosAttention(bcfg).to(DEV)
+    g = torch.Generator().manual_seed(3)
+    for b, s in ((2, 96), (2, 96), (3, 40)):
+        say("blocks without a mask", b, s)
+        hidden = torch.randn(b, s, 256, generator=g)
+        keep = torch.ones(b, s, dtype=torch.bool)
+        w = [getattr(gpt, n).weight.detach().double().cpu() for n in ("q_proj", "k_proj", "v_proj", "out_proj")]
+        ref = tf.gpt_attention_block(hidden.double(), *w, gpt.norm_const.detach().double().cpu().reshape(-1),
+                                     cfg.num_attention_heads, cfg.rotary_dim, cfg.max_position_embeddings, keep)
+        out = gpt(hidden.to(DEV))[0]
+        assert rel_l2(out.float(), ref.numpy()) <= 1e-4
+        wb = [getattr(bert, n).weight.detach().double().cpu() for n in ("query", "key", "value")]
+        bb = [getattr(bert, n).bias.detach().double().cpu() for n in ("query", "key", "value")]
+        ref = tf.bert_attention_block(hidden.double(), wb[0], bb[0], wb[1], bb[1], wb[2], bb[2],
+                                      bert.norm_const.detach().double().cpu().reshape(-1), 4, keep)
+        (out,) = bert(hidden.to(DEV))
+        assert rel_l2(out.float(), ref.numpy()) <= 1e-4
