@@ -191,6 +191,33 @@ class PreparedCausalAttention(torch.autograd.Function):
         return dq, dk, dv, None, None, dsig, None, None, None, None
 
 
+class PreparedNonCausalAttention(torch.autograd.Function):
+    """(q, k, v, keep, cnt, sig, bnhd, merged_heads) -> O: the preparation steps of PrepareInputs (no rotation) and
+    the non-causal op Q (K^T V) as ONE forward launch on the raw projections (ops.noncausal_dot_product_prepared;
+    BERT_Trainer/BertCosAttention.py:162-178 in front of :249).  The kernel leaves the prepared q, k, v for the
+    backward pass: the attention gradients on them, then the fused backward of the preparation.  Only where
+    ops.noncausal_fused_preparation_supported() holds."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, keep, cnt, sig, bnhd=False, merged_heads=False):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        out, prepared = ops.noncausal_dot_product_prepared(q, k, v, keep, cnt, sig, bnhd=bnhd, merged_heads=merged_heads)
+        ctx.save_for_backward(q, k, v, keep, cnt, sig, *prepared)
+        ctx.bnhd, ctx.merged = bool(bnhd), bool(merged_heads)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        q, k, v, keep, cnt, sig, qh, kh, vh = ctx.saved_tensors
+        gq, gk, gv = ops.noncausal_backward(qh, kh, vh, grad_output.contiguous().to(qh.dtype), merged_heads=ctx.merged)
+        want = sig is not None and ctx.needs_input_grad[5]
+        dq, dk, dv, dsig = ops.prepare_inputs_backward(q, k, v, gq, gk, gv, keep, cnt, sig, want_dsig=want, bnhd=ctx.bnhd,
+                                                       check_positions=False)
+        if dsig is not None:
+            dsig = dsig.to(sig.dtype)
+        return dq, dk, dv, None, None, dsig, None, None
+
+
 def _weight_gradient(gy, x):
     """gy^T x for gy (R, out), x (R, in).  With many rows and a small weight the library's single GEMM fills the
     chip with too few tiles over a long reduction (out = in = 1024, R = 16384, bf16: 109 us); the rows are cut into

@@ -716,6 +716,54 @@ int cott_causal_fwd_prep_save(const void *q, const void *k, const void *v, void 
                          in_bnhd, o_bnhd, saved, chunks_per_cut, ncuts, B, H, N, Dk, Dv, dtype, stream);
 }
 
+int cott_noncausal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype) {
+    if (B < 0 || H < 0 || N < 0 || (dtype != COTT_BF16 && dtype != COTT_F16) || Dk % 16 != 0 || Dk < 32) return 0;
+    if (!use_mfma(dtype, Dk, Dv, N)) return 0;
+    const long dmax = Dk > Dv ? Dk : Dv;
+    if ((long)N * H * dmax > (1L << 30) || (long)B * H > (1L << 22)) return 0;
+    if ((long)B * H * N == 0) return 1;
+    // one workgroup (or two column halves) per head; heads of up to 64 columns (with wider tiles the state fragments
+    // leave no registers for the preparation: B16 H16 N512 D128 176 us against 64 us for the two kernels)
+    return Dk <= 64 && Dv <= 64 && plan_set((long)B * H, N, 1, Dk, Dv, false, dtype).G == 1;
+}
+
+int cott_noncausal_fwd_prep(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
+                            const unsigned char *keep, const float *cnt, const float *sig, int in_bnhd, int o_bnhd, int B,
+                            int H, int N, int Dk, int Dv, int dtype, void *stream) {
+    const char *fn = "cott_noncausal_fwd_prep";
+    if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
+    if (dtype != COTT_BF16 && dtype != COTT_F16) return fail(COTT_ERR_UNSUPPORTED, "%s: needs bf16 / fp16 tensors", fn);
+    if (!use_mfma(dtype, Dk, Dv, N)) return fail(COTT_ERR_UNSUPPORTED, "%s: needs head dims 32..128 in steps of 16", fn);
+    if ((cnt == nullptr) != (sig == nullptr)) return fail(COTT_ERR_INVALID, "%s: cnt and sig go together", fn);
+    if ((long)B * H * N == 0) return COTT_OK;
+    if (!cott_noncausal_fwd_prep_supported(B, H, N, Dk, Dv, dtype))
+        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation needs head dims of at most 64 and a head that fits one "
+                    "workgroup (cott_noncausal_fwd_prep_supported); prepare the inputs with cott_prep_ex_fwd instead", fn);
+    if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(q_out) || !aligned16(k_out) ||
+        !aligned16(v_out))
+        return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    Op op{q, k, v, o, Dk, Dv, 0};
+    op.H = H;
+    if (in_bnhd) op.lay[0] = op.lay[1] = op.lay[2] = 1;
+    if (o_bnhd) op.lay[3] = 1;
+    cott::SetArgs::Prep prep;
+    prep.on = true;
+    prep.keep = keep;
+    prep.cnt = cnt;
+    prep.sig = sig;
+    prep.rot = nullptr;
+    prep.pos0 = 0;
+    prep.R = 0;
+    prep.table_rows = 0;
+    prep.H = H;
+    prep.dv = Dv;
+    prep.qo = q_out;
+    prep.ko = k_out;
+    prep.vo = v_out;
+    return run_ops(fn, false, &op, 1, (long)B * H, N, dtype, nullptr, 0, static_cast<hipStream_t>(stream), &prep);
+}
+
 namespace {
 // dst[i] = src ? src[i] : 0 over n 16-byte vectors: the state pass-through of an empty sequence.  A kernel rather than
 // hipMemsetAsync / hipMemcpyAsync so that the call can be recorded into a HIP graph like every other launch here.

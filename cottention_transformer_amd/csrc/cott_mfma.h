@@ -1252,10 +1252,15 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
 // PF2: chunks of A rows in flight in pass 2.  PF2 > PF: the first PF2 chunks are requested before pass 1 starts instead
 // of at the hand-over (sequences of 4 to 8 chunks, three gradient problems per head: B32 H12 N512 D64 gradients 46.6 -> 43.0 us;
 // the forward pass alone loses 0.7 us of 21.4 with it and keeps PF2 = PF; 3, 4 and 6 chunks measured alike, 8 worse).
-template <class TR, int DI, int DJ, int PF, int PF2 = PF>
-__global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int BH, int N, int nchunks) {
+// PREP: A, B, C are the raw projections; their rows are normalised (A, B), scaled (C) and masked on the way in
+// (PrepSide, no rotation) and the prepared tensors are written to qo / ko / vo for the backward pass.  A column half
+// (c0 > 0) prepares the same A and B rows as its twin and leaves writing them to the first half.
+template <class TR, int DI, int DJ, int PF, int PF2 = PF, bool PREP = false>
+__global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int BH, int N, int nchunks, PrepSide prep) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS;
+    constexpr int NB = DI / 32, NC = DJ / 32;  // 16-byte pieces per thread of a B / C tile
+    static_assert(!PREP || PF2 == PF, "the preparing variant keeps one prefetch depth");
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * SC];
     __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
@@ -1269,12 +1274,24 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
     const rsrc_t rB = make_rsrc(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), ((uint32_t)(N - 1) * ldb + di) * 2u);
     const rsrc_t rC = make_rsrc(pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), ((uint32_t)(N - 1) * ldc + dj) * 2u);
     const rsrc_t rO = make_rsrc(pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), ((uint32_t)(N - 1) * ldo + dj) * 2u);
+    // PREP: side inputs of this head's batch element and the prepared tensors, (B,H,N,width)
+    const bool first_half = pr.c0 == 0;
+    const uint32_t qk_bytes = (PREP && first_half) ? (uint32_t)N * di * 2u : 0u;
+    const rsrc_t rQo = make_rsrc(PREP && prep.qo ? prep.qo + (size_t)wi.bh * N * di : nullptr, prep.qo ? qk_bytes : 0u);
+    const rsrc_t rKo = make_rsrc(PREP && prep.ko ? prep.ko + (size_t)wi.bh * N * di : nullptr, prep.ko ? qk_bytes : 0u);
+    const rsrc_t rVo = make_rsrc(PREP && prep.vo ? prep.vo + (size_t)wi.bh * N * prep.dv + pr.c0 : nullptr,
+                                 (PREP && prep.vo) ? ((uint32_t)(N - 1) * prep.dv + dj) * 2u : 0u);
+    const size_t tok0 = PREP ? (size_t)(wi.bh / prep.H) * N : 0;
+    const bool scaled = PREP && prep.cnt != nullptr && prep.sig != nullptr;
+    const float sig = scaled ? prep.sig[wi.bh % prep.H] : 0.f;
 
     u32x4 qn[PF2][TL::KS];
+    float keep_q[PF2];
     auto load_q = [&](int s, int p) {
         const int row = min(p, nchunks - 1) * kChunk + 16 * w + m;
 #pragma unroll
         for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * lda + 32 * ks + 8 * g) * 2u);
+        if constexpr (PREP) keep_q[s] = prep.keep != nullptr ? (float)prep.keep[tok0 + min(row, N - 1)] : 1.f;
     };
 
     // ---- pass 1: S = sum over all chunks of B_c^T C_c
@@ -1282,11 +1299,71 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     {
-        u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
+        u32x4 rb[PF][NB], rc[PF][NC];
+        float keep_b[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
         auto load_chunk = [&](int s, int p) {
             const int row0 = min(p, nchunks - 1) * kChunk;
             load_tile<DI>(rb[s], rB, row0, ldb, tid);
             load_tile<DJ>(rc[s], rC, row0, ldc, tid);
+            if constexpr (PREP) {
+#pragma unroll
+                for (int u = 0; u < NB; ++u) {
+                    const int srow = min(row0 + (tid + kThreads * u) / (DI / 8), N - 1);
+                    keep_b[s][u] = prep.keep != nullptr ? (float)prep.keep[tok0 + srow] : 1.f;
+                }
+#pragma unroll
+                for (int u = 0; u < NC; ++u) {
+                    const int srow = min(row0 + (tid + kThreads * u) / (DJ / 8), N - 1);
+                    keep_c[s][u] = prep.keep != nullptr ? (float)prep.keep[tok0 + srow] : 1.f;
+                    cnt_c[s][u] = scaled ? prep.cnt[tok0 + srow] : 0.f;
+                }
+            }
+        };
+        // registers of stage s (chunk p) -> LDS tiles tb, tc; PREP: prepared on the way, and out to ko / vo
+        auto stage = [&](int s, int p, u16 *tb, u16 *tc) {
+            if constexpr (!PREP) {
+                store_tile<DI, TL::BS>(tb, rb[s], di, tid);
+                store_tile<DJ, TL::CS>(tc, rc[s], dj, tid);
+            } else {
+                const int row0 = min(p, nchunks - 1) * kChunk;
+#pragma unroll
+                for (int u = 0; u < NB; ++u) {
+                    const int v = tid + kThreads * u;
+                    const int lrow = v / (DI / 8), col = (v % (DI / 8)) * 8;
+                    float x[8];
+                    unpack8<TR>(rb[s][u], x);
+                    float ss = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (col >= di) x[e] = 0.f;
+                        ss += x[e] * x[e];
+                    }
+#pragma unroll
+                    for (int off = 1; off < DI / 8; off <<= 1) ss += __shfl_xor(ss, off, 64);
+                    const float nrm = __builtin_amdgcn_sqrtf(ss);
+                    const float mul = keep_b[s][u] * __builtin_amdgcn_rcpf(nrm > prep.eps ? nrm : prep.eps);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[e] *= mul;
+                    const u32x4 y = pack8<TR>(x);
+                    *reinterpret_cast<u32x4 *>(tb + lrow * TL::BS + col) = y;
+                    const uint32_t off = (col < di && p < nchunks) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
+                    __builtin_amdgcn_raw_buffer_store_b128(y, rKo, (int)off, 0, 0);
+                }
+#pragma unroll
+                for (int u = 0; u < NC; ++u) {
+                    const int v = tid + kThreads * u;
+                    const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+                    float x[8];
+                    unpack8<TR>(rc[s][u], x);
+                    const float mul = (col < dj) ? value_scale(keep_c[s][u], cnt_c[s][u], sig, scaled) : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[e] *= mul;
+                    const u32x4 y = (col < dj) ? pack8<TR>(x) : u32x4{0u, 0u, 0u, 0u};
+                    *reinterpret_cast<u32x4 *>(tc + lrow * TL::CS + col) = y;
+                    const uint32_t off = (col < dj && p < nchunks) ? (uint32_t)((row0 + lrow) * prep.dv + col) * 2u : kOobOffset;
+                    __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);
+                }
+            }
         };
 #pragma unroll
         for (int s = 0; s < PF; ++s) load_chunk(s, s);
@@ -1294,15 +1371,13 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
 #pragma unroll
             for (int s = 0; s < PF2; ++s) load_q(s, s);
         }
-        store_tile<DI, TL::BS>(sB, rb[0], di, tid);
-        store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
+        stage(0, 0, sB, sC);
         load_chunk(0, PF);
         __syncthreads();
         run_rounds<PF>(0, nchunks, [&](int s, int p) {
             const int s1 = (s + 1) % PF;
             const int buf = p & 1;
-            store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-            store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+            stage(s1, p + 1, sB + (buf ^ 1) * SB, sC + (buf ^ 1) * SC);
             load_chunk(s1, p + 1 + PF);
             state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
             chunk_barrier();
@@ -1335,8 +1410,32 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
             u32x4 qc[TL::KS];
 #pragma unroll
             for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
-            if (PF2 == PF || p + PF2 < nchunks) load_q(s, p + PF2);
             const int orow = p * kChunk + 16 * w + m;
+            if constexpr (PREP) {
+                // a row of A lives in the four lanes m, m + 16, m + 32, m + 48 (eight columns of every 32 each)
+                float x[TL::KS][8];
+                float ss = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < TL::KS; ++ks) {
+                    unpack8<TR>(qc[ks], x[ks]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ss += x[ks][e] * x[ks][e];
+                }
+                ss += __shfl_xor(ss, 16, 64);
+                ss += __shfl_xor(ss, 32, 64);
+                const float nrm = __builtin_amdgcn_sqrtf(ss);
+                const float mul = keep_q[s] * __builtin_amdgcn_rcpf(nrm > prep.eps ? nrm : prep.eps);
+#pragma unroll
+                for (int ks = 0; ks < TL::KS; ++ks) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[ks][e] *= mul;
+                    qc[ks] = pack8<TR>(x[ks]);
+                    const int col = 32 * ks + 8 * g;
+                    const uint32_t off = (col < di) ? (uint32_t)(orow * di + col) * 2u : kOobOffset;
+                    __builtin_amdgcn_raw_buffer_store_b128(qc[ks], rQo, (int)off, 0, 0);
+                }
+            }
+            if (PF2 == PF || p + PF2 < nchunks) load_q(s, p + PF2);
 #pragma unroll
             for (int jt = 0; jt < TL::NJT; ++jt) {
                 f32x4 o = {0.f, 0.f, 0.f, 0.f};

@@ -16,7 +16,8 @@ from torch import nn
 
 from . import ops
 from .autograd import (CustomAttention, CustomAttentionMergedHeads, NonCausalAttention,
-                       NonCausalAttentionMergedHeads, PreparedCausalAttention, PrepareInputs, _autocast_target, project)
+                       NonCausalAttentionMergedHeads, PreparedCausalAttention, PreparedNonCausalAttention, PrepareInputs,
+                       _autocast_target, project)
 
 
 def _autocast_on():
@@ -283,6 +284,19 @@ class BertCosAttention(nn.Module):
             keep = _keep_from_additive_mask(attention_mask, b, s, query_layer.device)
             cnt = keep.sum(-1, keepdim=True).to(torch.float32).expand(b, s)
         dt = _autocast_target(query_layer)
+        d = self.attention_head_size
+        if (query_layer.dtype == dt and ops.noncausal_fused_preparation_supported(dt, b, h, s, d, d)
+                and ops.merged_heads_supported(dt, s, h, d, d)):
+            # one forward launch: normalisation, value scaling, mask and the attention op
+            context_layer = PreparedNonCausalAttention.apply(query_layer, key_layer, value_layer, keep, cnt,
+                                                             self.norm_const.sigmoid().reshape(h), True, True)
+            if not _autocast_on():
+                context_layer = context_layer.to(hidden_states.dtype)
+            context_layer = context_layer.view(context_layer.size()[:-2] + (self.all_head_size,))
+            outputs = (context_layer, None) if output_attentions else (context_layer,)
+            if self.is_decoder:
+                outputs = outputs + ((key_layer.permute(0, 2, 1, 3), value_layer.permute(0, 2, 1, 3)),)
+            return outputs
         q, k, v = PrepareInputs.apply(query_layer, key_layer, value_layer, keep, cnt, self.norm_const.sigmoid().reshape(h),
                                       dt, None, None, True)
         # Q (K^T V)  (:249); (QK^T)V at :222 is the same product

@@ -276,6 +276,45 @@ def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=N
     return (o, prepared, saved) if save_states else (o, prepared)
 
 
+def noncausal_fused_preparation_supported(dtype, b, h, n, dk, dv):
+    """Whether noncausal_dot_product_prepared has a kernel for the shape: bf16 / fp16, head dims 32..64 in steps of
+    16, enough heads that a head is handled by one workgroup (cott_noncausal_fwd_prep_supported)."""
+    if dtype not in (torch.bfloat16, torch.float16):
+        return False
+    key = ("nc", dtype, b, h, n, dk, dv)
+    ok = _prep_supported_cache.get(key)
+    if ok is None:
+        ok = _remember(_prep_supported_cache, key, bool(
+            _loader.lib().cott_noncausal_fwd_prep_supported(b, h, n, dk, dv, _DTYPES[dtype])))
+    return ok
+
+
+def noncausal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, bnhd=False, merged_heads=False):
+    """Non-causal Q (K^T V) on the RAW projections: normalisation, value scaling and masking (prepare_inputs without a
+    rotation) happen inside the attention kernel (BERT_Trainer/BertCosAttention.py:162-178 in front of :249 as one
+    launch).  bnhd: q, k, v are (B,N,H,D); merged_heads: o is returned as (B,N,H,Dv).  Returns
+    (o, (q_hat, k_hat, v_hat)) with the prepared tensors (B,H,N,D) that the backward pass needs.  Raises where
+    noncausal_fused_preparation_supported() is false."""
+    _require_gpu(Q=q, K=k, V=v)
+    b, h, n, dk, dv = _prep_shapes(q, k, v, bnhd)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise RuntimeError("Q, K and V must have the same dtype")
+    code = _dtype_code(q)
+    keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    o = torch.empty((b, n, h, dv) if merged_heads else (b, h, n, dv), dtype=q.dtype, device=q.device)
+    prepared = (torch.empty((b, h, n, dk), dtype=q.dtype, device=q.device),
+                torch.empty((b, h, n, dk), dtype=q.dtype, device=q.device),
+                torch.empty((b, h, n, dv), dtype=q.dtype, device=q.device))
+    with _on(q.device):
+        rc = _loader.lib().cott_noncausal_fwd_prep(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                                   *(t.data_ptr() for t in prepared), _ptr(keep), _ptr(cnt), _ptr(sig),
+                                                   int(bool(bnhd)), int(bool(merged_heads)), b, h, n, dk, dv, code,
+                                                   _stream(q.device))
+    _check(rc, "cott_noncausal_fwd_prep")
+    return o, prepared
+
+
 def causal_prefill(q, k, v, state=None, return_state=True):
     """Causal forward over a whole prompt (or one piece of a sequence) with the recurrence state handed over:
     returns (o, state_out) with o[s] = q[s] (state + sum_{s'<=s} k[s'] v[s']^T) and

@@ -269,6 +269,19 @@ COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, v
                          const float *rot_table, long long pos0, int rotary_dim, int table_rows,
                          int in_bnhd, int o_bnhd,
                          int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
+/* The non-causal counterpart: o = q_hat (k_hat^T v_hat) on the raw projections in one launch, q_hat, k_hat, v_hat as
+ * above without a rotation (BERT_Trainer/BertCosAttention.py:162-178 mask / normalise / scale in front of :249; there
+ * cnt is the number of real tokens of the batch element at every position).  q_out, k_out, v_out receive the
+ * prepared tensors for the backward pass (cott_noncausal_bwd on them, then cott_prep_ex_bwd).  bf16 / fp16, head
+ * dims 32..64 in steps of 16, and a head must fit one workgroup (no sequence groups: B*H at least about the number
+ * of CUs): cott_noncausal_fwd_prep_supported() says whether a shape qualifies; otherwise COTT_ERR_UNSUPPORTED.
+ * Needs no workspace. */
+COTT_API int cott_noncausal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype);
+COTT_API int cott_noncausal_fwd_prep(const void *q, const void *k, const void *v, void *o,
+                            void *q_out, void *k_out, void *v_out,
+                            const unsigned char *keep, const float *cnt, const float *sig,
+                            int in_bnhd, int o_bnhd,
+                            int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
 /* ... that also writes the states the backward pass takes (cott_causal_saved_plan for the same shape gives
  * chunks_per_cut and ncuts; saved as in cott_causal_fwd_save, holding sums of k_hat^T v_hat): the backward of the
  * block is then cott_causal_bwd_saved(_bnhd) on q_hat, k_hat, v_hat followed by cott_prep_ex_bwd. */

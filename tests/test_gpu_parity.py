@@ -794,6 +794,75 @@ def test_input_preparation_inside_the_forward_kernel(ct, oracle, case):
         assert got.shape == ref.shape and rel_l2(got, ref.numpy()) <= 2e-2, name
 
 
+NC_FUSED_PREP_CASES = [
+    # b, h, n, dk, dv, dtype, projections' layout, masked      launch form
+    (32, 12, 512, 64, 64, BF, True, True),     # the BERT-base shape: two column halves per head, eight chunks
+    (40, 8, 300, 64, 64, HF, True, True),      # ragged tail
+    (16, 16, 130, 64, 32, BF, True, True),     # one workgroup per head, narrower values
+    (64, 8, 63, 32, 64, BF, False, False),     # no mask, a single partial chunk, per-head layout
+    (48, 8, 200, 48, 48, HF, False, True),     # padded head dims
+]
+
+
+@pytest.mark.parametrize("case", NC_FUSED_PREP_CASES,
+                         ids=lambda c: "x".join(map(str, c[:5])) + "-" + str(c[5]).split(".")[-1])
+def test_input_preparation_inside_the_non_causal_kernel(ct, oracle, case):
+    """cott_noncausal_fwd_prep: mask, normalisation and value scaling inside the non-causal kernel
+    (BERT_Trainer/BertCosAttention.py:162-178, 249 as one launch) against the CPU statement of those steps
+    (oracle/torch_forms.py) followed by the non-causal oracle; the prepared tensors it leaves for the backward pass;
+    the two-kernel path on the same inputs; and the autograd function against autograd through the CPU forms."""
+    from oracle import torch_forms as tf
+    b, h, n, dk, dv, dt, bnhd, masked = case
+    say("fused preparation, non-causal", case)
+    assert ct.noncausal_fused_preparation_supported(dt, b, h, n, dk, dv)
+    g = torch.Generator().manual_seed(n + dk)
+    shape = (lambda d: (b, n, h, d)) if bnhd else (lambda d: (b, h, n, d))
+    q, k, v = (torch.randn(shape(d), generator=g).to(dt) for d in (dk, dk, dv))
+    keep = None
+    if masked:  # padding at the end of every sequence, as a BERT batch has it
+        keep = torch.arange(n)[None, :] < torch.randint(1, n + 1, (b, 1), generator=g)
+    sig = torch.sigmoid(torch.randn(h, generator=g))
+    go = torch.randn(b, h, n, dv, generator=g).to(dt)
+    q64, k64, v64, s64 = (t.double().requires_grad_(True) for t in (q, k, v, sig))
+    qh, kh, vh = ((t.permute(0, 2, 1, 3) if bnhd else t) for t in (q64, k64, v64))
+    rq, rk, rv, cnt = tf.input_prep_bert(qh, kh, vh, keep, s64)
+    ref_o = oracle.noncausal(rq.detach(), rk.detach(), rv.detach())
+    args = dict(keep=None if keep is None else keep.to(DEV), cnt=cnt.float().to(DEV), sig=sig.to(DEV), bnhd=bnhd)
+    for merged in (False, True):
+        o, prepared = ct.noncausal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV), merged_heads=merged, **args)
+        assert o.shape == ((b, n, h, dv) if merged else (b, h, n, dv)) and o.dtype == dt
+        assert rel_l2(o.permute(0, 2, 1, 3) if merged else o, ref_o) <= TOL[dt], merged
+        for name, got, ref in zip("qkv", prepared, (rq, rk, rv)):
+            assert got.shape == ref.shape and rel_l2(got, ref.detach().numpy()) <= TOL[dt], name
+        if keep is not None:
+            dropped = ~keep.to(DEV)[:, None, :].expand(b, h, n)
+            assert all(torch.all(t[dropped] == 0) for t in prepared)
+    # the separate preparation pass followed by the plain op gives the same numbers to 16-bit rounding
+    p2 = ct.prepare_inputs(q.to(DEV), k.to(DEV), v.to(DEV), args["keep"], args["cnt"], args["sig"], out_dtype=dt, bnhd=bnhd)
+    for a, r in zip(prepared, p2):
+        assert rel_l2(a, r.double().cpu().numpy()) <= 1e-2
+    o2 = ct.noncausal_dot_product(*p2)
+    assert rel_l2(o2, o.permute(0, 2, 1, 3).double().cpu().numpy()) <= 1e-2
+    # gradients through the autograd function
+    ro = tf.noncausal_einsum(rq, rk, rv)
+    ref_grads = torch.autograd.grad(ro, [q64, k64, v64, s64], go.double())
+    qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sig))
+    out = ct.PreparedNonCausalAttention.apply(qd, kd, vd, args["keep"], args["cnt"], sd, bnhd, False)
+    assert rel_l2(out, ref_o) <= TOL[dt]
+    out.backward(go.to(DEV))
+    for name, got, ref in zip(("dq", "dk", "dv", "dsig"), (qd.grad, kd.grad, vd.grad, sd.grad), ref_grads):
+        assert got.shape == ref.shape and rel_l2(got, ref.numpy()) <= 2e-2, name
+
+
+def test_non_causal_fused_preparation_is_refused_where_not_built(ct):
+    assert not ct.noncausal_fused_preparation_supported(F32, 32, 12, 512, 64, 64)
+    assert not ct.noncausal_fused_preparation_supported(BF, 1, 2, 4096, 64, 64)      # few heads: sequence groups
+    q = torch.randn(1, 2, 4096, 64, device=DEV, dtype=BF)
+    assert not ct.noncausal_fused_preparation_supported(BF, 16, 16, 512, 128, 128)   # wide heads: the two kernels
+    with pytest.raises(RuntimeError, match="one workgroup"):
+        ct.noncausal_dot_product_prepared(q, q, q)
+
+
 def test_fused_preparation_is_refused_where_not_built(ct):
     assert not ct.fused_preparation_supported(F32, 8, 16, 256, 64, 64)
     assert not ct.fused_preparation_supported(BF, 1, 2, 4096, 64, 64)        # few heads: sequence groups
