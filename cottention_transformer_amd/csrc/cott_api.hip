@@ -634,8 +634,10 @@ int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtyp
     if ((long)N * H * dmax > (1L << 30) || (long)B * H > (1L << 22)) return 0;
     if ((long)B * H * N == 0) return 1;
     const SetPlan p = plan_set((long)B * H, N, 1, Dk, Dv, true, dtype);
-    // one group per head, and tiles small enough that the prepared q tile fits LDS beside them
-    return p.G == 1 && cott::mfma_pad(Dk) * cott::mfma_pad(Dv / p.halves) <= 128 * 64;
+    // one group per head, and q / k rows of at most 64 columns: with 128 the loader wavefronts hold four pieces of q and
+    // of k per chunk with their table entries, and the launch takes 400 us where the preparation pass and the plain
+    // forward take 165 (B8 H16 N2048)
+    return p.G == 1 && cott::mfma_pad(Dk) <= 64 && cott::mfma_pad(Dk) * cott::mfma_pad(Dv / p.halves) <= 128 * 64;
 }
 
 namespace {
@@ -656,8 +658,8 @@ int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, v
     }
     if ((long)B * H * N == 0) return COTT_OK;
     if (!cott_causal_fwd_prep_supported(B, H, N, Dk, Dv, dtype, rot_table ? rotary_dim : 0))
-        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation needs one group per head and tiles of at most 128 x 64 "
-                    "(cott_causal_fwd_prep_supported); prepare the inputs with cott_prep_ex_fwd instead", fn);
+        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation needs one group per head and q / k rows of at most 64 "
+                    "columns (cott_causal_fwd_prep_supported); prepare the inputs with cott_prep_ex_fwd instead", fn);
     if (in_bnhd || o_bnhd) {
         const long dmax = Dk > Dv ? Dk : Dv;
         if ((long)N * H * dmax > (1L << 30))

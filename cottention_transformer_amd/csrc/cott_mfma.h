@@ -157,6 +157,23 @@ __device__ __forceinline__ int table_row(const PrepSide &ps, int s) {
     long long t = ps.pos0 + s;
     return (int)(t < 0 ? 0 : (t >= ps.table_rows ? ps.table_rows - 1 : t));
 }
+// Sum of v over the LANES (4, 8 or 16) consecutive, aligned lanes that hold one row, left in every one of them:
+// data-parallel-primitive moves inside the vector ALU (quad swaps, then the mirrored half rows / rows, whose other
+// half already holds its own partial sum in every lane) instead of permutes through the LDS crossbar.
+template <int LANES>
+__device__ __forceinline__ float lane_group_sum(float v) {
+    static_assert(LANES == 4 || LANES == 8 || LANES == 16, "a row lives in 4, 8 or 16 lanes");
+    auto moved = [](float x, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                     0xf, 0xf, false));
+    };
+    v += moved(v, std::integral_constant<int, 0xB1>{});                             // lanes 1,0,3,2 of each quad
+    v += moved(v, std::integral_constant<int, 0x4E>{});                             // lanes 2,3,0,1
+    if constexpr (LANES >= 8) v += moved(v, std::integral_constant<int, 0x141>{});  // mirrored half row (8 lanes)
+    if constexpr (LANES >= 16) v += moved(v, std::integral_constant<int, 0x140>{}); // mirrored row (16 lanes)
+    return v;
+}
+
 // keep / max(cnt ^ sig, 1) of one position (keep alone when there is no value scaling)
 __device__ __forceinline__ float value_scale(float keep, float cnt, float sig, bool scaled) {
     if (!scaled) return keep;
@@ -578,8 +595,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
         float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
-#pragma unroll
-        for (int off = 1; off < DI / 8; off <<= 1) ss += __shfl_xor(ss, off, 64);
+        ss = lane_group_sum<DI / 8>(ss);
         const float nrm = __builtin_amdgcn_sqrtf(ss);
         const float mul = keep * __builtin_amdgcn_rcpf(nrm > ps.eps ? nrm : ps.eps);
 #pragma unroll
@@ -1338,8 +1354,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
                         if (col >= di) x[e] = 0.f;
                         ss += x[e] * x[e];
                     }
-#pragma unroll
-                    for (int off = 1; off < DI / 8; off <<= 1) ss += __shfl_xor(ss, off, 64);
+                    ss = lane_group_sum<DI / 8>(ss);
                     const float nrm = __builtin_amdgcn_sqrtf(ss);
                     const float mul = keep_b[s][u] * __builtin_amdgcn_rcpf(nrm > prep.eps ? nrm : prep.eps);
 #pragma unroll

@@ -216,9 +216,9 @@ _prep_supported_cache = {}
 
 
 def fused_preparation_supported(dtype, b, h, n, dk, dv, rotary_dim=0):
-    """Whether causal_dot_product_prepared has a kernel for the shape: bf16 / fp16, head dims 32..128 in steps of 16,
-    a rotary width that is a multiple of 8, enough heads that no head is cut into sequence groups, and not the
-    undivided 128 x 128 tiles (cott_causal_fwd_prep_supported)."""
+    """Whether causal_dot_product_prepared has a kernel for the shape: bf16 / fp16, Dk 32..64 and Dv 32..128 in steps
+    of 16, a rotary width that is a multiple of 8, enough heads that no head is cut into sequence groups
+    (cott_causal_fwd_prep_supported)."""
     if dtype not in (torch.bfloat16, torch.float16):
         return False
     key = (dtype, b, h, n, dk, dv, rotary_dim)

@@ -258,9 +258,9 @@ COTT_API int cott_prep_ex_bwd(const void *q, const void *k, const void *v,
  * cott_prep_ex_bwd); any of them may be NULL.  keep, cnt, sig as in cott_prep_fwd.  rot_table: (table_rows,
  * rotary_dim) fp32 as in cott_prep_ex_fwd, rotary_dim a multiple of 8, or NULL; the table row of position s is
  * pos0 + s (clamped to the table): positions that are not consecutive take cott_prep_ex_fwd.  in_bnhd: q, k, v
- * are (B,N,H,D); o_bnhd: o is (B,N,H,Dv).  bf16 / fp16, head dims 32..128 in steps of 16, B*H large enough that a
- * head is not cut into sequence groups, and not the undivided 128 x 128 tiles (no room in LDS for the prepared q
- * tile): cott_causal_fwd_prep_supported() says (1 / 0) whether a shape qualifies; otherwise the call returns
+ * are (B,N,H,D); o_bnhd: o is (B,N,H,Dv).  bf16 / fp16, Dk of 32..64 and Dv of 32..128 in steps of 16, B*H large
+ * enough that a head is not cut into sequence groups (wider q / k rows are faster through the separate pass):
+ * cott_causal_fwd_prep_supported() says (1 / 0) whether a shape qualifies; otherwise the call returns
  * COTT_ERR_UNSUPPORTED and the caller prepares the inputs with cott_prep_ex_fwd.  Needs no workspace. */
 COTT_API int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim);
 COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o,

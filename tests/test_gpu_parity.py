@@ -728,7 +728,7 @@ def test_calls_can_be_captured_in_a_hip_graph_and_replayed(ct, oracle):
 FUSED_PREP_CASES = [
     # b, h, n, dk, dv, dtype, rotary_dim, projections' layout, masked   launch form
     (8, 16, 256, 64, 64, BF, 64, True, True),      # two column halves per head, outputs staged through LDS
-    (8, 16, 130, 128, 128, BF, 64, True, True),    # 128-wide heads in column halves, rotation of half of the columns
+    (8, 16, 130, 64, 128, BF, 32, True, True),     # wide values in column halves, rotation of half of the columns
     (32, 16, 200, 48, 80, HF, 32, False, True),    # padded head dims, two workgroups per CU
     (16, 16, 63, 32, 64, BF, 0, False, False),     # no rotation, no mask, a single partial chunk
     (8, 32, 1000, 64, 64, HF, 16, True, True),     # several chunks, ragged tail
@@ -867,6 +867,7 @@ def test_fused_preparation_is_refused_where_not_built(ct):
     assert not ct.fused_preparation_supported(F32, 8, 16, 256, 64, 64)
     assert not ct.fused_preparation_supported(BF, 1, 2, 4096, 64, 64)        # few heads: sequence groups
     assert not ct.fused_preparation_supported(BF, 8, 16, 256, 64, 64, 12)    # rotary width not a multiple of 8
+    assert not ct.fused_preparation_supported(BF, 8, 16, 256, 128, 128, 64)  # wide q / k rows: the separate pass
     assert not ct.fused_preparation_supported(BF, 16, 16, 130, 128, 128)     # undivided 128 x 128 tiles
     q, k, v, _ = inputs(1, 2, 4096, 64, 64, BF, seed=1)
     with pytest.raises(RuntimeError, match="one group per head"):
