@@ -83,9 +83,23 @@ __device__ __forceinline__ void store4(void *base, int dtype, size_t idx, const 
 }
 
 // Sum over the `lpr` (power of two, <= 64) consecutive lanes that hold one row.
-template <class ACC>
-__device__ __forceinline__ ACC row_sum(ACC v, int lpr) {
+__device__ __forceinline__ double row_sum(double v, int lpr) {
     for (int off = 1; off < lpr; off <<= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+// fp32: the steps inside a row of 16 lanes are data-parallel-primitive moves in the vector ALU (quad swaps, then the
+// mirrored half row and row, whose other half already holds its partial sum in every lane); only rows of 32 or 64
+// lanes go on through LDS permutes.
+template <int CTRL>
+__device__ __forceinline__ float dpp_moved(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row_sum(float v, int lpr) {
+    if (lpr >= 2) v += dpp_moved<0xB1>(v);    // lanes 1,0,3,2 of each quad
+    if (lpr >= 4) v += dpp_moved<0x4E>(v);    // lanes 2,3,0,1
+    if (lpr >= 8) v += dpp_moved<0x141>(v);   // mirrored half row
+    if (lpr >= 16) v += dpp_moved<0x140>(v);  // mirrored row
+    for (int off = 16; off < lpr; off <<= 1) v += __shfl_xor(v, off, 64);
     return v;
 }
 
