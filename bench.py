@@ -469,6 +469,22 @@ def run_extras(torch, ct, dev):
                                                          "frac_hbm": pb / s_f / 1e9 / HBM_PEAK_GBS,
                                                          "torch_elementwise_us": s_e * 1e6}
     del keep, cnt, sig
+    # the BERT block's preparation inside the non-causal kernel (cott_noncausal_fwd_prep) at the BERT-base shape, on
+    # the projections' (B,S,H,D) tensors with a padding mask, next to the separate pass followed by the plain kernel
+    bq, bk, bv = (torch.randn(32, 512, 12, 64, device=dev).bfloat16() for _ in range(3))
+    bkeep = torch.arange(512, device=dev)[None, :] < torch.randint(256, 513, (32, 1), device=dev)
+    bcnt = bkeep.sum(-1, keepdim=True).float().expand(32, 512).contiguous()
+    bsig = torch.sigmoid(torch.randn(12, device=dev))
+
+    def nc_two_kernels():
+        p = ct.prepare_inputs(bq, bk, bv, bkeep, bcnt, bsig, out_dtype=torch.bfloat16, bnhd=True)
+        return ct.noncausal_dot_product(*p, merged_heads=True)
+    s_nf = time_region(torch, lambda: ct.noncausal_dot_product_prepared(bq, bk, bv, bkeep, bcnt, bsig, bnhd=True,
+                                                                        merged_heads=True), 100, 10)
+    s_n2 = time_region(torch, nc_two_kernels, 100, 10)
+    ex["noncausal_fwd_with_preparation_B32_H12_N512_D64"] = {"one_launch_us": s_nf * 1e6,
+                                                             "separate_pass_plus_kernel_us": s_n2 * 1e6}
+    del bq, bk, bv, bkeep, bcnt, bsig
     # whole GPT attention block (projections, rotary, preparation, attention, output projection), fwd+bwd under
     # bf16 autocast at the GPT-300M shape; second figure: same block with rotary / head permute as torch ops
     block_step = gpt_block_step(torch, dev)
