@@ -144,6 +144,23 @@ def test_c_abi_argument_errors_without_a_gpu():
     assert prep(1, 2, 4096, 64, 64, _loader.BF16) == _loader.ERR_UNSUPPORTED
     assert "one group per head" in _loader.last_error()
     assert prep(0, 16, 256, 64, 64, _loader.BF16) == _loader.OK
+    assert prep(8, 16, 256, 128, 128, _loader.BF16) == _loader.ERR_UNSUPPORTED     # q / k rows of more than 64 columns
+    assert L.cott_causal_fwd_prep_supported(8, 16, 256, 64, 128, _loader.BF16, 64) == 1
+    assert L.cott_causal_fwd_prep_supported(8, 16, 256, 128, 128, _loader.BF16, 64) == 0
+    # ... and inside the non-causal kernel: 16-bit, head dims of at most 64, a head must fit one workgroup
+    ncprep = lambda *shape_dtype, cnt=None, sig=None: L.cott_noncausal_fwd_prep(
+        16, 16, 16, 16, None, None, None, None, cnt, sig, 1, 1, *shape_dtype, None)
+    assert ncprep(32, 12, 512, 64, 64, _loader.F32) == _loader.ERR_UNSUPPORTED
+    assert "bf16 / fp16" in _loader.last_error()
+    assert ncprep(32, 12, 512, 64, 64, _loader.BF16, cnt=16) == _loader.ERR_INVALID
+    assert "cnt and sig" in _loader.last_error()
+    assert ncprep(1, 2, 4096, 64, 64, _loader.BF16) == _loader.ERR_UNSUPPORTED
+    assert "one workgroup" in _loader.last_error()
+    assert ncprep(16, 16, 512, 128, 128, _loader.BF16) == _loader.ERR_UNSUPPORTED
+    assert ncprep(0, 12, 512, 64, 64, _loader.BF16) == _loader.OK
+    assert L.cott_noncausal_fwd_prep_supported(32, 12, 512, 64, 64, _loader.BF16) == 1
+    assert L.cott_noncausal_fwd_prep_supported(32, 12, 512, 64, 64, _loader.F32) == 0
+    assert L.cott_noncausal_fwd_prep_supported(1, 2, 4096, 64, 64, _loader.BF16) == 0
 
 
 def test_no_alloc_entry_point_checks_and_its_scratch_symbol(tmp_path):
