@@ -267,3 +267,42 @@ def test_dropin_module_names_resolve():
         kernel.float32(q, q, q, 1, False, False)
     with pytest.raises(ValueError):                                               # Custom_Kernel.py:31-32
         Custom_Kernel.CustomAttention.apply(q.to(torch.int32), q, q)
+
+
+def test_plan_queries_stay_sane_over_random_shapes():
+    """The host-side planner behind the workspace, saved-state and fused-preparation queries, over 400 seeded shapes
+    (no GPU involved): sizes are multiples of 16 bytes and bounded by what a full chip of 64 KiB state slots per
+    problem can need, a saved-state plan's cuts fit the sequence, and the `supported` answers agree with their
+    documented preconditions."""
+    import ctypes
+    import random
+    from cottention_transformer_amd import _loader
+    L = _loader.lib()
+    rnd = random.Random(7)
+    for _ in range(400):
+        b = rnd.choice([1, 2, 3, 8, 32, 100]); h = rnd.choice([1, 2, 8, 12, 16])
+        n = rnd.choice([1, 63, 64, 65, 512, 2048, 4097, 16384, 65536])
+        dk = rnd.choice([32, 48, 64, 96, 128]); dv = rnd.choice([32, 64, 80, 128])
+        dt = rnd.choice([_loader.BF16, _loader.F16, _loader.F32])
+        if n * max(dk, dv) > 1 << 30:
+            continue
+        nchunks = (n + 63) // 64
+        for fn in (L.cott_causal_workspace_bytes, L.cott_causal_bwd_workspace_bytes, L.cott_noncausal_workspace_bytes):
+            ws = fn(b, h, n, dk, dv, dt)
+            # at most a few hundred workgroups hold a slot of 128 x 128 floats each, per problem (six with halves)
+            assert ws % 16 == 0 and 0 <= ws <= 6 * 4096 * 128 * 128 * 4, (fn.__name__, b, h, n, dk, dv, dt, ws)
+        cpc, cuts, slot, wsb = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
+        rc = L.cott_causal_saved_plan(b, h, n, dk, dv, dt, ctypes.byref(cpc), ctypes.byref(cuts), ctypes.byref(slot),
+                                      ctypes.byref(wsb))
+        assert rc == _loader.OK
+        if cuts.value > 0:
+            assert dt != _loader.F32 and nchunks >= 16
+            assert cpc.value >= 1 and (cuts.value - 1) * cpc.value <= nchunks - 1
+            assert slot.value >= dk * dv and wsb.value % 16 == 0
+        sup = L.cott_causal_fwd_prep_supported(b, h, n, dk, dv, dt, 0)
+        if sup:
+            assert dt != _loader.F32 and dk <= 64 and L.cott_causal_workspace_bytes(b, h, n, dk, dv, dt) == 0
+        sup = L.cott_noncausal_fwd_prep_supported(b, h, n, dk, dv, dt)
+        if sup:
+            assert dt != _loader.F32 and dk <= 64 and dv <= 64
+            assert L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, dt) == 0
