@@ -235,7 +235,7 @@ def _weight_gradient(gy, x):
 
 class InputProjections(torch.autograd.Function):
     """(x, w_0, b_0, w_1, b_1, ...) -> (x w_0^T + b_0, x w_1^T + b_1, ...): the q / k / v projections of an attention
-    block (GPT_Trainer/GPTCosAttention.py:447-449, BERT_Trainer/BertCosAttention.py:253-255 with biases) as one
+    block (GPT_Trainer/GPTCosAttention.py:443-445, BERT_Trainer/BertCosAttention.py:121,143-144 with biases) as one
     operator.  Under autocast x is converted once for all of them, the gradient of x is accumulated by the GEMMs
     themselves and converted back once, and the weight gradients take `_weight_gradient`.  b_i may be None."""
 
