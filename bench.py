@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--block-only", action="store_true",
                     help="run only the GPT attention block fwd+bwd (a secondary figure) for --steps steps: for profiling")
+    ap.add_argument("--bert-block-only", action="store_true",
+                    help="run only the BERT self-attention block fwd+bwd (a secondary figure) for --steps steps: for profiling")
     ap.add_argument("--long-only", type=int, default=0, metavar="N",
                     help="run only the long-context configuration B1 H16 D128 bf16 at sequence length N (fwd and bwd "
                          "separately, per-kernel durations) for --steps steps: for profiling")
@@ -115,6 +117,12 @@ def main():
         block_step = gpt_block_step(torch, dev)
         s = time_region(torch, lambda: block_step(False), args.steps, args.warmup)
         print(json.dumps({"gpt_block_fwd_bwd_B8_S2048_E1024_H16_autocast_bf16_us": s * 1e6, "steps": args.steps,
+                          "warmup": args.warmup}))
+        return
+    if args.bert_block_only:
+        step = bert_block_step(torch, dev)
+        s = time_region(torch, step, args.steps, args.warmup)
+        print(json.dumps({"bert_block_fwd_bwd_B32_S512_E768_H12_autocast_bf16_us": s * 1e6, "steps": args.steps,
                           "warmup": args.warmup}))
         return
     if args.calibration_copy:
@@ -329,6 +337,28 @@ def gpt_block_step(torch, dev):
     return step
 
 
+def bert_block_step(torch, dev):
+    """step(): forward + backward of the BERT self-attention block (projections, preparation, non-causal attention)
+    under bf16 autocast at the BERT-base shape B32 S512 E768 H12, with the padding mask of a batch whose sequences
+    end between half and full length."""
+    from types import SimpleNamespace
+    from cottention_transformer_amd import modules
+    bert = modules.BertCosAttention(SimpleNamespace(hidden_size=768, num_attention_heads=12,
+                                                    attention_probs_dropout_prob=0.0)).to(dev)
+    hid = torch.randn(32, 512, 768, device=dev, requires_grad=True)
+    gout = torch.randn(32, 512, 768, device=dev, dtype=torch.bfloat16)
+    keep = torch.arange(512, device=dev)[None, :] < torch.randint(256, 513, (32, 1), device=dev)
+    mask = ((~keep).float() * torch.finfo(torch.float32).min)[:, None, None, :]
+
+    def step():
+        hid.grad = None
+        bert.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = bert(hid, attention_mask=mask)[0]
+        out.backward(gout)
+    return step
+
+
 def module_anchor(torch, dev):
     """Forward latency of the two attention modules at batch 1, hidden 2048, 16 heads (D = 128), the one point the
     reference publishes for this path: its module-level plots (tests/MemoryTest.py:118-143, 233-278: eval mode, fp32,
@@ -494,23 +524,10 @@ def run_extras(torch, ct, dev):
         "us": s_fused * 1e6, "tokens_per_s": 8 * 2048 / s_fused,
         "us_with_rotary_and_permute_as_torch_ops": s_torch * 1e6}
     del block_step
-    # the BERT self-attention block (projections, preparation, non-causal attention), fwd+bwd under bf16 autocast at
-    # the BERT-base shape B32 S512 E768 H12
-    from types import SimpleNamespace as _NS
-    from cottention_transformer_amd import modules as _modules
-    bert = _modules.BertCosAttention(_NS(hidden_size=768, num_attention_heads=12, attention_probs_dropout_prob=0.0)).to(dev)
-    bh_in = torch.randn(32, 512, 768, device=dev, requires_grad=True)
-    bg = torch.randn(32, 512, 768, device=dev, dtype=torch.bfloat16)
-
-    def bert_step():
-        bh_in.grad = None
-        bert.zero_grad(set_to_none=True)
-        with torch.autocast("cuda", dtype=torch.bfloat16):
-            out = bert(bh_in)[0]
-        out.backward(bg)
+    bert_step = bert_block_step(torch, dev)
     s_b = time_region(torch, bert_step, 20, 3)
     ex["bert_block_fwd_bwd_B32_S512_E768_H12_autocast_bf16"] = {"us": s_b * 1e6, "tokens_per_s": 32 * 512 / s_b}
-    del bert, bh_in, bg
+    del bert_step
     ex["module_forward_latency_batch1_hidden2048_heads16"] = module_anchor(torch, dev)
     # prompt pass that also hands the state to decoding (cott_causal_fwd_state), headline shape
     qp, kp, vp, _ = make_inputs(torch, 8, 16, 2048, 64, 64, torch.bfloat16, dev)
