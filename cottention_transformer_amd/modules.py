@@ -282,7 +282,8 @@ class BertCosAttention(nn.Module):
             keep, cnt = cached[1], cached[2]
         else:
             keep = _keep_from_additive_mask(attention_mask, b, s, query_layer.device)
-            cnt = keep.sum(-1, keepdim=True).to(torch.float32).expand(b, s)
+            # (made contiguous here, once, rather than by the forward and again by the backward of the preparation)
+            cnt = keep.sum(-1, keepdim=True).to(torch.float32).expand(b, s).contiguous()
         dt = _autocast_target(query_layer)
         d = self.attention_head_size
         if (query_layer.dtype == dt and ops.noncausal_fused_preparation_supported(dt, b, h, s, d, d)

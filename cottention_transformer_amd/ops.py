@@ -505,7 +505,10 @@ def _prep_side_inputs(b, h, n, keep, cnt, sig, device):
     if keep is not None:
         if keep.shape != (b, n):
             raise RuntimeError(f"keep must have shape {(b, n)}, got {tuple(keep.shape)}")
-        keep = keep.to(device=device, dtype=torch.uint8).contiguous()
+        if keep.dtype == torch.bool and keep.device == device and keep.is_contiguous():
+            keep = keep.view(torch.uint8)  # a bool tensor already holds one 0 / 1 byte per element: no copy
+        else:
+            keep = keep.to(device=device, dtype=torch.uint8).contiguous()
     if (cnt is None) != (sig is None):
         raise RuntimeError("cnt and sig are given together (or neither)")
     if cnt is not None:
