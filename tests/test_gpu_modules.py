@@ -233,3 +233,45 @@ def test_blocks_without_a_mask_reuse_their_constant_side_inputs(mods):
                                       bert.norm_const.detach().double().cpu().reshape(-1), 4, keep)
         (out,) = bert(hidden.to(DEV))
         assert rel_l2(out.float(), ref.numpy()) <= 1e-4
+
+
+@pytest.mark.parametrize("masked", [False, True], ids=["no-mask", "masked"])
+def test_bert_block_with_the_preparation_inside_the_attention_kernel(mods, masked):
+    """Enough heads that a head is handled by one workgroup, bf16 autocast: the forward of the block then runs mask,
+    normalisation, value scaling and Q (K^T V) as one launch (PreparedNonCausalAttention).  Against the fp64 CPU
+    statement of the block, outputs and all gradients."""
+    from unittest import mock
+    from oracle import torch_forms as tf
+    from cottention_transformer_amd import ops
+    say("bert block, fused preparation", masked)
+    torch.manual_seed(0)
+    cfg = SimpleNamespace(hidden_size=768, num_attention_heads=12, attention_probs_dropout_prob=0.0, is_decoder=False)
+    m = mods.BertCosAttention(cfg).to(DEV)
+    with torch.no_grad():
+        m.norm_const.copy_(torch.linspace(-1.0, 1.0, 12).reshape(1, 12, 1, 1))
+    b, s = 24, 136
+    g = torch.Generator().manual_seed(4)
+    hidden = torch.randn(b, s, cfg.hidden_size, generator=g)
+    keep = (torch.arange(s)[None, :] < torch.randint(1, s + 1, (b, 1), generator=g)) if masked \
+        else torch.ones(b, s, dtype=torch.bool)
+    gout = torch.randn(b, s, cfg.hidden_size, generator=g)
+    names = ("query", "key", "value")
+    w = [getattr(m, n).weight.detach().double().cpu().requires_grad_(True) for n in names]
+    bias = [getattr(m, n).bias.detach().double().cpu().requires_grad_(True) for n in names]
+    nc = m.norm_const.detach().double().cpu().reshape(-1).requires_grad_(True)
+    h64 = hidden.double().requires_grad_(True)
+    ref = tf.bert_attention_block(h64, w[0], bias[0], w[1], bias[1], w[2], bias[2], nc, cfg.num_attention_heads, keep)
+    ref_grads = torch.autograd.grad(ref, [h64, *w, *bias, nc], gout.double())
+    hd = hidden.to(DEV).requires_grad_(True)
+    with mock.patch.object(ops, "noncausal_dot_product_prepared", wraps=ops.noncausal_dot_product_prepared) as spy:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            (out,) = m(hd, attention_mask=additive_mask(keep).to(DEV) if masked else None)
+        assert spy.call_count == 1, "the fused forward was not taken"
+    assert rel_l2(out.float(), ref.detach().numpy()) <= 3e-2
+    out.backward(gout.to(DEV).to(out.dtype))
+    got = [hd.grad] + [getattr(m, n).weight.grad for n in names] + [getattr(m, n).bias.grad for n in names] \
+        + [m.norm_const.grad.reshape(-1)]
+    labels = ("hidden", "wq", "wk", "wv", "bq", "bk", "bv", "norm_const")
+    for name, a, r in zip(labels, got, ref_grads):
+        # (the value bias only reaches the output through masked, scaled rows; its gradient is small against the others)
+        assert rel_l2(a.float(), r.numpy()) <= 3e-2, name
