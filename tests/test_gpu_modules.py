@@ -275,3 +275,48 @@ def test_bert_block_with_the_preparation_inside_the_attention_kernel(mods, maske
     for name, a, r in zip(labels, got, ref_grads):
         # (the value bias only reaches the output through masked, scaled rows; its gradient is small against the others)
         assert rel_l2(a.float(), r.numpy()) <= 3e-2, name
+
+
+def test_module_options_of_the_reference_signatures(mods):
+    """The forward options the blocks keep from the reference's signatures: `use_cache` / `output_attentions` of the GPT
+    block (GPT_Trainer/GPTCosAttention.py:481-508: rotated keys and values handed back, the attention output repeated
+    in place of the weights) and `output_attentions` / `is_decoder` of the BERT block
+    (BERT_Trainer/BertCosAttention.py:319-334).  These paths rotate and permute with torch ops; their outputs must
+    equal the default path's."""
+    torch.manual_seed(1)
+    cfg = gpt_cfg()
+    m = mods.GPTCosAttention(cfg).to(DEV)
+    for p_ in m.parameters():
+        p_.requires_grad_(False)
+    g = torch.Generator().manual_seed(5)
+    b, s = 2, 150
+    hidden = torch.randn(b, s, cfg.hidden_size, generator=g).to(DEV)
+    keep = torch.rand(b, s, generator=g) > 0.2
+    mask = additive_mask(keep).to(DEV)
+    base = m(hidden, attention_mask=mask)
+    assert len(base) == 2 and base[1] is None
+    out_c, present = m(hidden, attention_mask=mask, use_cache=True)
+    h, d = cfg.num_attention_heads, cfg.hidden_size // cfg.num_attention_heads
+    assert present[0].shape == (b, h, s, d) and present[1].shape == (b, h, s, d)
+    assert rel_l2(out_c, base[0].double().cpu().numpy()) <= 1e-5
+    # the values come back as projected, the keys rotated (their norms are those of the projections)
+    v_proj = m.v_proj(hidden).view(b, s, h, d).permute(0, 2, 1, 3)
+    k_proj = m.k_proj(hidden).view(b, s, h, d).permute(0, 2, 1, 3)
+    assert rel_l2(present[1], v_proj.double().cpu().numpy()) <= 1e-6
+    assert torch.allclose(present[0].norm(dim=-1), k_proj.norm(dim=-1), rtol=1e-4, atol=1e-5)
+    assert not torch.allclose(present[0], k_proj)
+    out_a = m(hidden, attention_mask=mask, output_attentions=True)
+    assert len(out_a) == 3 and out_a[2].shape == (b, h, s, d)
+    assert rel_l2(out_a[0], base[0].double().cpu().numpy()) <= 1e-5
+
+    bcfg = SimpleNamespace(hidden_size=256, num_attention_heads=4, attention_probs_dropout_prob=0.0, is_decoder=True)
+    bert = mods.BertCosAttention(bcfg).to(DEV)
+    for p_ in bert.parameters():
+        p_.requires_grad_(False)
+    plain = bert(hidden, attention_mask=mask)
+    assert len(plain) == 2 and plain[1][0].shape == (b, 4, s, 64) and plain[1][1].shape == (b, 4, s, 64)
+    with_attn = bert(hidden, attention_mask=mask, output_attentions=True)
+    assert len(with_attn) == 3 and with_attn[1] is None
+    assert torch.equal(with_attn[0], plain[0])
+    with pytest.raises(NotImplementedError):
+        bert(hidden, encoder_hidden_states=hidden)
