@@ -797,7 +797,19 @@ int scratch_of_current_device(const char *fn, void **out) {
 }
 }  // namespace
 
-size_t cott_noalloc_scratch_bytes(void) { return (size_t)COTT_SCRATCH_BYTES; }
+// Also resolves the scratch array's address on the current device (when there is one), so that a caller who asks for
+// the size before recording cott_causal_fwd_noalloc into a HIP graph has the symbol lookup, and whatever code-object
+// loading it triggers, behind it when the capture starts.
+size_t cott_noalloc_scratch_bytes(void) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) == hipSuccess && count > 0) {
+        void *p = nullptr;
+        (void)scratch_of_current_device("cott_noalloc_scratch_bytes", &p);
+    } else {
+        (void)hipGetLastError();  // no device: only the size is wanted (host-side checks)
+    }
+    return (size_t)COTT_SCRATCH_BYTES;
+}
 
 int cott_causal_fwd_noalloc(const void *q, const void *k, const void *v, void *o, int B, int H, int N, int Dk, int Dv,
                             int dtype, int reversed, void *stream) {

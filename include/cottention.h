@@ -69,7 +69,9 @@ COTT_API int cott_causal_fwd_may_alias_v(int B, int H, int N, int Dk, int Dv, in
  * device memory around the call: code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  Same arguments, results (bit for bit) and errors as cott_causal_fwd; a shape whose slots exceed
  * cott_noalloc_scratch_bytes() (32 MiB, enough for every plan this build makes) returns COTT_ERR_WORKSPACE.
- * The first call on a device looks the array's address up (hipGetSymbolAddress); no call allocates or frees.
+ * The array's address is looked up once per device (hipGetSymbolAddress): by cott_noalloc_scratch_bytes() when a
+ * device is current, else by the first call of the entry point on that device.  Call cott_noalloc_scratch_bytes()
+ * before a stream capture starts, so that the lookup does not happen inside it.  No call allocates or frees.
  * All calls on one GPU share that GPU's array: calls that may overlap on one GPU (different streams or threads)
  * race on it and must be ordered by the caller.  Keep cott_profile_enable off (it creates HIP events). */
 COTT_API size_t cott_noalloc_scratch_bytes(void);

@@ -763,7 +763,6 @@ def test_input_preparation_inside_the_forward_kernel(ct, oracle, case):
                                    x[..., rdim:]], -1)
         qh, kh = rot(qh), rot(kh)
     rq, rk, rv, cnt = tf.input_prep_gpt(qh, kh, vh, keep, s64)
-    ro = tf.causal_cumsum(rq, rk, rv) if n <= 300 else None
     ref_o = oracle.causal(rq.detach(), rk.detach(), rv.detach())
     # the kernel
     args = dict(keep=None if keep is None else keep.to(DEV), cnt=cnt.float().to(DEV), sig=sig.to(DEV),
@@ -781,10 +780,16 @@ def test_input_preparation_inside_the_forward_kernel(ct, oracle, case):
     assert rel_l2(o2, o.permute(0, 2, 1, 3).double().cpu().numpy()) <= 1e-2
     o_np, none = ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV), want_prepared=False, **args)
     assert none is None and rel_l2(o_np, ref_o) <= TOL[dt]
-    if ro is None:
-        return
-    # gradients through the autograd function
-    ref_grads = torch.autograd.grad(ro, [q64, k64, v64, s64], go.double())
+    # Gradients through the autograd function, at every length: the oracle's closed forms (Custom_Kernel.py:63,68,72)
+    # give the gradients with respect to the prepared tensors, and autograd carries those through the CPU statement of
+    # the preparation; no O(N D^2) cumsum tensor is needed.  Short sequences also go through the cumsum form, whose
+    # gradients autograd derives on its own.
+    d_prepared = [torch.from_numpy(x) for x in oracle.causal_bwd(rq.detach(), rk.detach(), rv.detach(), go)]
+    ref_grads = torch.autograd.grad([rq, rk, rv], [q64, k64, v64, s64], d_prepared, retain_graph=n <= 300)
+    if n <= 300:
+        by_cumsum = torch.autograd.grad(tf.causal_cumsum(rq, rk, rv), [q64, k64, v64, s64], go.double())
+        for a, r in zip(ref_grads, by_cumsum):
+            assert rel_l2(a, r.numpy()) <= 1e-9
     qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sig))
     out = ct.PreparedCausalAttention.apply(qd, kd, vd, args["keep"], args["cnt"], sd, table.to(DEV) if rdim else None, pos0,
                                            bnhd, False)

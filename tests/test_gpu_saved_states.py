@@ -41,6 +41,7 @@ SAVED_CASES = [
     (1, 16, 7777, 128, 64, BF),     # Dk != Dv: dQ and dK form the set, dV runs apart
     (1, 16, 30000, 64, 128, BF),
     (1, 5, 30000, 128, 128, BF),    # 16 cuts; forward and backward cut the sequence differently
+    (1, 16, 65536, 128, 128, BF),   # the long-context benchmark configuration at its full size, as the benchmark runs it
 ]
 
 

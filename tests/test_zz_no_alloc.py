@@ -58,6 +58,33 @@ def test_no_alloc_entry_point_equals_workspace_entry_point(L, oracle, dt):
     assert torch.equal(got, want)
 
 
+def test_no_alloc_entry_point_in_a_hip_graph(L):
+    """What the entry point is for: recorded into a HIP graph (no allocation may happen under capture).  The size
+    query before the capture resolves the scratch address; every replay, with eager work and a synchronisation
+    between replays, equals cott_causal_fwd bit for bit."""
+    from cottention_transformer_amd import _loader
+    b, h, n, d = 1, 4, 4096, 64
+    assert L.cott_causal_workspace_bytes(b, h, n, d, d, _loader.BF16) > 0, "the shape must use group-state slots"
+    q, k, v, _ = (x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=7))
+    out = torch.full_like(v, float("nan"))
+    assert L.cott_noalloc_scratch_bytes() == 32 << 20            # resolves the symbol, outside the capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        rc = L.cott_causal_fwd_noalloc(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b, h, n, d, d, _loader.BF16,
+                                       0, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, _loader.last_error()
+    for rep in range(3):
+        new = [x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=70 + rep)[:3]]
+        for dst, src in zip((q, k, v), new):
+            dst.copy_(src)
+        graph.replay()
+        want, _, _ = both(L, *new, _loader.BF16)                 # eager calls (they use the scratch too) and a sync
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {rep}"
+
+
 def test_no_alloc_entry_point_rejects_like_the_workspace_entry_point(L):
     from cottention_transformer_amd import _loader
     z = torch.zeros(1, 1, 64, 64, dtype=BF, device=DEV)
