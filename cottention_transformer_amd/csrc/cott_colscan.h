@@ -1,0 +1,458 @@
+// Chunk recurrence for 128-wide heads (bf16 / fp16) with the state kept out of LDS.
+//
+// Same op and chunk recurrence as scan_kernel (cott_mfma.h):
+//     out_c = ((A_c B_c^T) o mask) C_c + A_c S_c ;   S_{c+1} = S_c + B_c^T C_c
+// but with a different split of the work inside a workgroup.  In scan_kernel four state wavefronts carry S and publish
+// a 16-bit copy of it in LDS every chunk (DI x DJ x 2 bytes written, and read once by each output wavefront), and two
+// output wavefronts do all the products that make up out_c: with 128 x 128 states 96 KiB of LDS traffic per chunk for
+// the state alone and 108 matrix instructions per chunk on each of two wavefronts.
+//
+// Here every compute wavefront owns DJ / 4 COLUMNS of the state, all DI rows, in its accumulators, and produces the
+// same columns of out_c for all 64 positions of the chunk:
+//   * A_c S_c for its columns comes straight from its own accumulators: converted to 16 bits in registers they ARE the
+//     A operand of the product (see the row order below), so the state is never written to or read from LDS;
+//   * the ten masked score tiles on the live side of the diagonal are formed once per workgroup, three to a
+//     wavefront, and handed round through 5 KiB of LDS at a second barrier in the middle of the chunk;
+//   * the C fragments of its columns serve both the score-times-C product and the state update.
+// About 86 matrix instructions per wavefront and chunk on each of the four SIMDs, and 30 % less LDS traffic.
+// Four loader wavefronts stage THREE tiles per chunk (the A rows as well: all four compute wavefronts read them) and
+// write the finished output tile, which the compute wavefronts leave in LDS, to memory one chunk later as 16-byte
+// row segments.  All tiles double-buffered.
+//
+// What it buys is modest, and the measurements that say why are worth keeping next to the code.  At B1 H16 N65536
+// D128 (three gradient problems per head in 5 groups, 240 workgroups) this kernel with its compute wavefronts idle,
+// i.e. the loaders alone moving the launch's 1.97 GB, takes 389 us (5.1 TB/s); with all matrix instructions but no
+// LDS reads in the compute wavefronts 390 us; complete 448 us (scan_kernel: 467 us).  Under the profiler's counter
+// collection, which leaves gaps between kernels, the complete kernel takes 404 us at 2.28 GHz against 383 us at
+// 2.44 GHz idle (GRBM_GUI_ACTIVE over the duration): the data path through the chip scales with the core clock, the
+// core clock gives way under the power the products draw, and in a loop of back-to-back launches it gives way
+// further.  Work removed from a chunk (matrix instructions, LDS traffic) therefore shows up as time even though no
+// unit is saturated; prefetch depths of 3 and 4 chunks, the order of the loaders' steps and issuing the LDS reads a
+// pipeline step ahead of their products change nothing.
+//
+// Row order of a state tile.  The matrix instruction fixes where accumulator elements live: lane (g, m) holds rows
+// 4g .. 4g+3 of column m of a 16 x 16 tile.  As the A operand of the next product the same lane must hold EIGHT
+// consecutive steps of the contraction (8g .. 8g+7).  The state update is therefore done with the rows of two
+// neighbouring tiles interleaved: tile 2ks + t (t = 0, 1), row 4g' + q holds state row 32ks + 8g' + 4t + q, which the
+// transposing LDS read delivers for free (each lane of a quarter-wave names the 8-byte piece it contributes, so the
+// four column groups of a tile may lie 16 bytes apart instead of side by side).  The accumulators of tiles 2ks and
+// 2ks + 1 of a lane, packed to 16 bits, are then state rows 32ks + 8g .. 32ks + 8g + 7 of column m: operand order.
+// States in memory (group-state slots, states saved for a backward pass, hand-over states) keep the plain layout of
+// cott_mfma.h; they are gathered into this row order when a workgroup starts and scattered back where it writes them.
+#pragma once
+#include "cott_mfma.h"
+
+namespace cott {
+
+__device__ __forceinline__ u32x4 ld128(const u16 *p) { return *reinterpret_cast<const u32x4 *>(p); }
+
+template <int DI, int DJ>
+struct ColTiling {
+    static_assert(DI % 32 == 0 && DJ % 64 == 0, "padded head dims: rows a multiple of 32, columns a multiple of 64");
+    using TL = Tiling<DI, DJ>;
+    static constexpr int NJW = TL::NJT / 4;  // column tiles owned by one compute wavefront
+    static constexpr int SA = kChunk * TL::BS, SC = kChunk * TL::CS, SO = kChunk * TL::OS;
+    static constexpr int LDS_BYTES = 2 * (2 * SA + SC + SO) * 2;
+};
+
+// Loader role: LT threads move the A, B and C tiles global -> registers -> LDS, PF chunks ahead, and send the output
+// tile that the compute wavefronts finished one chunk earlier from LDS to memory.  Loads and stores are unconditional
+// (rows past N read as zero and are dropped on the way out: buffer range check).
+template <int DI, int DJ, int PF, int LT, bool STREAM>
+__device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_head, const u16 *C_head, u16 *O_head, int di,
+                                                int dj, int lda, int ldb, int ldc, int ldo, const ScanRange &r, int tid,
+                                                u16 *sA, u16 *sB, u16 *sC, const u16 *sO) {
+    using TL = Tiling<DI, DJ>;
+    using CT = ColTiling<DI, DJ>;
+    static_assert((8 * DI) % LT == 0 && (8 * DJ) % LT == 0, "tile vectors divide over the loader threads");
+    const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
+    const rsrc_t rB = make_rsrc(B_head, ((uint32_t)(r.N - 1) * ldb + di) * 2u);
+    const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
+    const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldo + dj) * 2u);
+    auto write_out = [&](int p) {
+        const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
+        const u16 *tile = sO + ((p - r.p0) & 1) * CT::SO;
+#pragma unroll
+        for (int u = 0; u < 8 * DJ / LT; ++u) {
+            const int v = tid + LT * u;
+            const int row = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+            const u32x4 val = *reinterpret_cast<const u32x4 *>(tile + row * TL::OS + col);
+            const uint32_t off = (col < dj) ? (uint32_t)((row0 + row) * ldo + col) * 2u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(val, rO, (int)off, 0, 0);
+        }
+    };
+    u32x4 ra[PF][8 * DI / LT], rb[PF][8 * DI / LT], rc[PF][8 * DJ / LT];
+    auto load_chunk = [&](int s, int p) {
+        const int pc = min(p, r.p1 - 1);
+        const int row0 = (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
+        load_tile<DI, LT, STREAM>(ra[s], rA, row0, lda, tid);
+        load_tile<DI, LT, STREAM>(rb[s], rB, row0, ldb, tid);
+        load_tile<DJ, LT, STREAM>(rc[s], rC, row0, ldc, tid);
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_chunk(s, r.p0 + s);
+    store_tile<DI, TL::BS, LT>(sA, ra[0], di, tid);
+    store_tile<DI, TL::BS, LT>(sB, rb[0], di, tid);
+    store_tile<DJ, TL::CS, LT>(sC, rc[0], dj, tid);
+    load_chunk(0, r.p0 + PF);
+    __syncthreads();
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+        const int s1 = (s + 1) % PF;
+        const int buf = (p - r.p0) & 1;
+        store_tile<DI, TL::BS, LT>(sA + (buf ^ 1) * CT::SA, ra[s1], di, tid);
+        store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * CT::SA, rb[s1], di, tid);
+        store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * CT::SC, rc[s1], dj, tid);
+        load_chunk(s1, p + 1 + PF);
+        chunk_barrier();  // (the compute wavefronts hand their score tiles round here)
+        if (p > r.p0) write_out(p - 1);
+        chunk_barrier();
+    });
+    if (r.p1 > r.p0) write_out(r.p1 - 1);
+}
+
+// Where the compute wavefront `w` of a workgroup finds and leaves its state (all pointers already at this head, and
+// group where that applies; any may be null).
+struct ColStateIO {
+    const float *seed = nullptr;      // group prefix, plain tile layout with DJ / 16 tiles per tile row
+    const float *seed_t = nullptr;    // the TRANSPOSE of this state in the plain tile layout, seed_t_njt tiles per tile row
+    int seed_t_njt = 0;
+    const float *sin = nullptr;       // row-major [di][lds] hand-over state to start from
+    float *sout = nullptr;            // ... and to leave at the end (last group only)
+    int lds = 0;
+    float *save = nullptr;            // states for a backward pass (ProblemT::save): first slot of this head
+    int save_njt = 0, save_jt0 = 0, save_slot = 0, save_cpg = 1, save_n = 0;
+};
+
+// Compute role: wavefront w of 4 owns column tiles NJW * w .. NJW * w + NJW - 1.  FUT: the scores that count are
+// those of keys at or after the query (ops that sum over the future, or over the past in complement form).
+// The ten score tiles on the live side of the diagonal are dealt three to a wavefront (the last wavefront forms its
+// one tile three times), left in LDS (sP: 16 tiles of 512 bytes in accumulator order, which is operand order for the
+// next product), and after a second barrier in the middle of the chunk every wavefront reads the tiles of all blocks.
+// Everything that does not need the scores (A_c S_c for all blocks, the state update) sits between writing the tiles
+// and that barrier, so nobody waits long at it.
+// The chunk is written as a software pipeline: the LDS reads of step k + 1 are issued, as a block, before the matrix
+// instructions of step k, and scheduling fences keep the compiler from sinking them back down to their first use
+// (left to itself it places every read a few instructions before the product that needs it, and the wavefront then
+// pays the full LDS latency some forty times per chunk).
+__device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+
+template <class TR, int DI, int DJ, bool FUT>
+__device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, int dj, const ScanRange &r, int w, int l,
+                                                   const u16 *sA, const u16 *sB, const u16 *sC, u16 *sO, u32x2 *sP) {
+    using TL = Tiling<DI, DJ>;
+    using CT = ColTiling<DI, DJ>;
+    constexpr int KS = TL::KS, NIT = TL::NIT, NJW = CT::NJW;
+    static_assert(NIT == 2 * KS && NIT % 4 == 0, "two row tiles per contraction step, row tiles in batches of four");
+    const int g = l >> 4, m = l & 15;
+    const bool mask_rev = r.mask_rev != 0, comp = r.comp != 0;
+    auto live = [&](int pb, int jt) { return FUT ? jt >= pb : jt <= pb; };
+    // score tiles of this wavefront: (position block, key tile), four bits each, three per wavefront
+    //   FUT:  w0 (0,0) (0,1) (0,2)   w1 (0,3) (1,1) (1,2)   w2 (1,3) (2,2) (2,3)   w3 (3,3) x 3
+    //   else: w0 (0,0) (1,0) (1,1)   w1 (2,0) (2,1) (2,2)   w2 (3,0) (3,1) (3,2)   w3 (3,3) x 3
+    int spb[3], sjt[3];
+    {
+        const int fut_pb[12] = {0, 0, 0, 0, 1, 1, 1, 2, 2, 3, 3, 3}, fut_jt[12] = {0, 1, 2, 3, 1, 2, 3, 2, 3, 3, 3, 3};
+        const int pst_pb[12] = {0, 1, 1, 2, 2, 2, 3, 3, 3, 3, 3, 3}, pst_jt[12] = {0, 0, 1, 0, 1, 2, 0, 1, 2, 3, 3, 3};
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            int pbv = 0, jtv = 0;
+#pragma unroll
+            for (int e = 0; e < 12; ++e)
+                if (e == 3 * w + t) {
+                    pbv = FUT ? fut_pb[e] : pst_pb[e];
+                    jtv = FUT ? fut_jt[e] : pst_jt[e];
+                }
+            spb[t] = __builtin_amdgcn_readfirstlane(pbv);
+            sjt[t] = __builtin_amdgcn_readfirstlane(jtv);
+        }
+    }
+    f32x4 S[NIT][NJW];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int jw = 0; jw < NJW; ++jw) S[it][jw] = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto plain_index = [&](int it, int jt, int njt) {
+        const int ks = it >> 1, t = it & 1;
+        return (size_t)((2 * ks + (g >> 1)) * njt + jt) * 64 + 16 * (2 * (g & 1) + t) + m;
+    };
+    if (io.seed != nullptr) {
+        const f32x4 *gs = reinterpret_cast<const f32x4 *>(io.seed);
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw) S[it][jw] = gs[plain_index(it, NJW * w + jw, TL::NJT)];
+    }
+    if (io.seed_t != nullptr) {
+        float *scr = reinterpret_cast<float *>(sO) + w * 512;
+        const f32x4 *src = reinterpret_cast<const f32x4 *>(io.seed_t);
+#pragma unroll
+        for (int jw = 0; jw < NJW; ++jw) {
+            const int jt = NJW * w + jw;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const f32x4 t0 = src[(size_t)(jt * io.seed_t_njt + 2 * ks) * 64 + l];
+                const f32x4 t1 = src[(size_t)(jt * io.seed_t_njt + 2 * ks + 1) * 64 + l];
+                *reinterpret_cast<f32x4 *>(scr + 4 * l) = t0;
+                *reinterpret_cast<f32x4 *>(scr + 256 + 4 * l) = t1;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int i = 32 * ks + 8 * g + 4 * t + q;
+                        const float x = scr[(g >> 1) * 256 + (16 * (m >> 2) + ((8 * g + 4 * t) & 15) + q) * 4 + (m & 3)];
+                        if (i < di && 16 * jt + m < dj) S[2 * ks + t][jw][q] += x;
+                    }
+            }
+        }
+    }
+    if (io.sin != nullptr) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int i = 32 * (it >> 1) + 8 * g + 4 * (it & 1) + q, j = 16 * (NJW * w + jw) + m;
+                    if (i < di && j < dj) S[it][jw][q] += io.sin[(size_t)i * io.lds + j];
+                }
+    }
+    u32x4 sop[KS][NJW];
+    auto pack_state = [&]() {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw)
+                sop[ks][jw] = u32x4{TR::pack2(S[2 * ks][jw][0], S[2 * ks][jw][1]), TR::pack2(S[2 * ks][jw][2], S[2 * ks][jw][3]),
+                                    TR::pack2(S[2 * ks + 1][jw][0], S[2 * ks + 1][jw][1]),
+                                    TR::pack2(S[2 * ks + 1][jw][2], S[2 * ks + 1][jw][3])};
+    };
+    pack_state();
+    const uint32_t flip = comp ? 0x80008000u : 0u;
+    __syncthreads();
+    for (int p = r.p0; p < r.p1; ++p) {
+        const int buf = (p - r.p0) & 1;
+        const u16 *cA = sA + buf * CT::SA, *cB = sB + buf * CT::SA, *cC = sC + buf * CT::SC;
+        u16 *cO = sO + buf * CT::SO;
+        // fragment readers (each a block of LDS reads, nothing else)
+        u32x4 sq[2][KS], sk[2][KS];  // query rows and key rows of a score tile, two tiles in flight
+        auto read_score = [&](int slot, int t) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                sq[slot][ks] = ld128(cA + (16 * spb[t] + m) * TL::BS + 32 * ks + 8 * g);
+                sk[slot][ks] = ld128(cB + (16 * sjt[t] + m) * TL::BS + 32 * ks + 8 * g);
+            }
+        };
+        auto score_tile = [&](int slot, int t) {
+            f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks & 1) a1 = TR::mfma(sk[slot][ks], sq[slot][ks], a1);
+                else a0 = TR::mfma(sk[slot][ks], sq[slot][ks], a0);
+            }
+            f32x4 acc = a0 + a1;
+            const int d0 = 16 * (sjt[t] - spb[t]) + 4 * g - m;  // key position - query position at element 0
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bool keep = mask_rev ? (d0 + q >= 0) : (d0 + q <= 0);
+                acc[q] = (keep != comp) ? (comp ? -acc[q] : acc[q]) : 0.f;
+            }
+            sP[(spb[t] * 4 + sjt[t]) * 64 + l] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
+        };
+        u32x4 qf[2][KS];
+        auto read_q = [&](int slot, int pb) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) qf[slot][ks] = ld128(cA + (16 * pb + m) * TL::BS + 32 * ks + 8 * g);
+        };
+        f32x4 o[4][NJW];
+        auto state_product = [&](int slot, int pb) {  // out^T tiles (columns 16jt + 4g .. + 3, position 16pb + m)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw) {
+                f32x4 o1 = {0.f, 0.f, 0.f, 0.f}, o2 = o1;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    if (ks & 1) o2 = TR::mfma(sop[ks][jw], qf[slot][ks], o2);
+                    else o1 = TR::mfma(sop[ks][jw], qf[slot][ks], o1);
+                }
+                o[pb][jw] = o1 + o2;
+            }
+        };
+        u32x4 cf[NJW][2], bf[2][4];
+        auto read_c = [&]() {
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+                    cf[jw][kb] = cat(lds_read_tr16(cC + (32 * kb + 4 * g + (m >> 2)) * TL::CS + 16 * (NJW * w + jw) + 4 * (m & 3)),
+                                     lds_read_tr16(cC + (32 * kb + 16 + 4 * g + (m >> 2)) * TL::CS + 16 * (NJW * w + jw) + 4 * (m & 3)));
+        };
+        auto read_b = [&](int slot, int kb, int it0) {  // B^T fragments of row tiles it0 .. it0 + 3, rows interleaved
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int it = it0 + e;
+                const int c = 32 * (it >> 1) + 8 * (m & 3) + 4 * (it & 1);
+                bf[slot][e] = cat(lds_read_tr16(cB + (32 * kb + 4 * g + (m >> 2)) * TL::BS + c),
+                                  lds_read_tr16(cB + (32 * kb + 16 + 4 * g + (m >> 2)) * TL::BS + c));
+            }
+        };
+        auto update = [&](int slot, int kb, int it0) {  // S += B_c^T C_c (complement form: -=)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const u32x4 b = bf[slot][e] ^ u32x4{flip, flip, flip, flip};
+#pragma unroll
+                for (int jw = 0; jw < NJW; ++jw) S[it0 + e][jw] = TR::mfma(b, cf[jw][kb], S[it0 + e][jw]);
+            }
+        };
+
+        read_score(0, 0);
+        sched_fence();
+        read_score(1, 1);
+        sched_fence();
+        score_tile(0, 0);
+        sched_fence();
+        read_score(0, 2);
+        sched_fence();
+        score_tile(1, 1);
+        sched_fence();
+        read_q(0, 0);
+        sched_fence();
+        score_tile(0, 2);
+        sched_fence();
+#pragma unroll
+        for (int pb = 0; pb < 4; ++pb) {
+            if (pb < 3) read_q((pb + 1) & 1, pb + 1);
+            else {
+                read_c();
+                read_b(0, 0, 0);
+            }
+            sched_fence();
+            state_product(pb & 1, pb);
+            sched_fence();
+        }
+        constexpr int NB = 2 * (NIT / 4);  // batches of four row tiles over the two key halves
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (b + 1 < NB) read_b((b + 1) & 1, (b + 1) / (NIT / 4), 4 * ((b + 1) % (NIT / 4)));
+            sched_fence();
+            update(b & 1, b / (NIT / 4), 4 * (b % (NIT / 4)));
+            sched_fence();
+        }
+        chunk_barrier();  // every block's score tiles are in sP
+        // ---- (scores) x C for every block, then the finished tiles go to the staging tile
+        u32x4 pf[4][2];
+#pragma unroll
+        for (int pb = 0; pb < 4; ++pb)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const u32x2 z = {0u, 0u};
+                if (live(pb, 2 * kb) || live(pb, 2 * kb + 1))
+                    pf[pb][kb] = cat(live(pb, 2 * kb) ? sP[(pb * 4 + 2 * kb) * 64 + l] : z,
+                                     live(pb, 2 * kb + 1) ? sP[(pb * 4 + 2 * kb + 1) * 64 + l] : z);
+            }
+        sched_fence();
+#pragma unroll
+        for (int pb = 0; pb < 4; ++pb) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if (!(live(pb, 2 * kb) || live(pb, 2 * kb + 1))) continue;
+#pragma unroll
+                for (int jw = 0; jw < NJW; ++jw) o[pb][jw] = TR::mfma(cf[jw][kb], pf[pb][kb], o[pb][jw]);
+            }
+        }
+#pragma unroll
+        for (int pb = 0; pb < 4; ++pb)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw)
+                *reinterpret_cast<u32x2 *>(cO + (16 * pb + m) * TL::OS + 16 * (NJW * w + jw) + 4 * g) =
+                    u32x2{TR::pack2(o[pb][jw][0], o[pb][jw][1]), TR::pack2(o[pb][jw][2], o[pb][jw][3])};
+        pack_state();
+        if (io.save != nullptr) {  // (an op that walks forwards: p is the chunk's place in the sequence)
+            const int back = r.nchunks - 1 - p;
+            if (back % io.save_cpg == 0 && back / io.save_cpg < io.save_n) {
+                f32x4 *dst = reinterpret_cast<f32x4 *>(io.save + (size_t)(back / io.save_cpg) * io.save_slot);
+#pragma unroll
+                for (int it = 0; it < NIT; ++it)
+#pragma unroll
+                    for (int jw = 0; jw < NJW; ++jw)
+                        if (16 * (NJW * w + jw) < dj) dst[plain_index(it, io.save_jt0 + NJW * w + jw, io.save_njt)] = S[it][jw];
+            }
+        }
+        chunk_barrier();
+    }
+    if (io.sout != nullptr) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int i = 32 * (it >> 1) + 8 * g + 4 * (it & 1) + q, j = 16 * (NJW * w + jw) + m;
+                    if (i < di && j < dj) io.sout[(size_t)i * io.lds + j] = S[it][jw][q];
+                }
+    }
+}
+
+// One problem per workgroup: 4 compute wavefronts, 4 loader wavefronts.  Same grid, problem set and state slots as
+// scan_kernel.
+template <class TR, int DI, int DJ, int PF, bool STREAM>
+__global__ __launch_bounds__(512) void colscan_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G) {
+    using TL = Tiling<DI, DJ>;
+    using CT = ColTiling<DI, DJ>;
+    __shared__ __attribute__((aligned(16))) u16 sA[2 * CT::SA];
+    __shared__ __attribute__((aligned(16))) u16 sB[2 * CT::SA];
+    __shared__ __attribute__((aligned(16))) u16 sC[2 * CT::SC];
+    __shared__ __attribute__((aligned(16))) u16 sO[2 * CT::SO];
+    __shared__ __attribute__((aligned(16))) u32x2 sP[16 * 64];  // masked score tiles, handed round in the middle of a chunk
+    static_assert(2 * CT::SO * 2 >= 4 * 2048, "room to turn the transposed seeds");
+    const int l = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
+    if (wi.grp >= G) return;
+    const Problem &pr = set.p[wi.prob];
+    const int di = pr.di, dj = pr.dj;
+    ScanRange r;
+    r.N = N;
+    r.nchunks = nchunks;
+    r.p0 = wi.grp * cpg;
+    r.p1 = min(r.p0 + cpg, nchunks);
+    r.reversed = pr.reversed;
+    r.mask_rev = pr.mask_rev;
+    r.comp = pr.comp;
+    if (wv >= 4) {
+        col_loader_role<DI, DJ, PF, 256, STREAM>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
+                                                 pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh),
+                                                 pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
+                                                 pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldb, pr.ldc,
+                                                 pr.ldo, r, (int)threadIdx.x - 256, sA, sB, sC, sO);
+        return;
+    }
+    ColStateIO io;
+    const size_t slot = ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS;
+    if (pr.ext != nullptr) {  // the state the forward pass saved at this group's cut is this one's transpose
+        io.seed_t = pr.ext + ((size_t)wi.bh * G + wi.grp) * pr.save_slot;
+        io.seed_t_njt = pr.save_njt;
+    } else if (pr.seed_from >= 0) {  // the twin problem's group prefix, transposed (square padded dims)
+        if (set.p[pr.seed_from].gstate != nullptr) {
+            io.seed_t = set.p[pr.seed_from].gstate + slot;
+            io.seed_t_njt = TL::NIT;
+        }
+    } else if (pr.gstate != nullptr) {
+        io.seed = pr.gstate + slot;
+    }
+    if (pr.sin != nullptr) io.sin = pr.sin + (size_t)wi.bh * di * pr.lds;
+    if (pr.sout != nullptr && wi.grp == G - 1) io.sout = pr.sout + (size_t)wi.bh * di * pr.lds;
+    io.lds = pr.lds;
+    if (pr.save != nullptr) {
+        io.save = pr.save + (size_t)wi.bh * pr.save_n * pr.save_slot;
+        io.save_njt = pr.save_njt;
+        io.save_jt0 = pr.c0 / 16;
+        io.save_slot = pr.save_slot;
+        io.save_cpg = pr.save_cpg;
+        io.save_n = pr.save_n;
+    }
+    if ((pr.mask_rev != 0) != (pr.comp != 0))
+        col_compute_role<TR, DI, DJ, true>(io, di, dj, r, wv, l, sA, sB, sC, sO, sP);
+    else
+        col_compute_role<TR, DI, DJ, false>(io, di, dj, r, wv, l, sA, sB, sC, sO, sP);
+}
+
+}  // namespace cott
