@@ -325,6 +325,8 @@ def gpt_block_step(torch, dev):
     blk = modules.GPTCosAttention(cfg).to(dev)
     hid = torch.randn(8, 2048, 1024, device=dev, requires_grad=True)
     gout = torch.randn(8, 2048, 1024, device=dev, dtype=torch.bfloat16)
+    # the ids as GPT-J's model hands them to every block: one arange row for the whole batch (GPTCosAttention.py:458)
+    position_ids = torch.arange(0, 2048, dtype=torch.long, device=dev).unsqueeze(0)
 
     def step(use_cache):
         # gradients start from None, as after a training loop's zero_grad(set_to_none=True): the hidden states of a
@@ -332,7 +334,7 @@ def gpt_block_step(torch, dev):
         hid.grad = None
         blk.zero_grad(set_to_none=True)
         with torch.autocast("cuda", dtype=torch.bfloat16):
-            out = blk(hid, use_cache=use_cache)[0]
+            out = blk(hid, position_ids=position_ids, use_cache=use_cache)[0]
         out.backward(gout)
     return step
 

@@ -159,29 +159,35 @@ class PreparedCausalAttention(torch.autograd.Function):
     """(q, k, v, keep, cnt, sig, rot_table, first_position, bnhd, merged_heads) -> O: the preparation steps of
     PrepareInputs and the causal attention op as ONE forward launch on the raw projections
     (ops.causal_dot_product_prepared).  The kernel also leaves the prepared q, k, v for the backward pass, which is
-    the attention gradient on them followed by the fused backward of the preparation.  Positions are consecutive:
-    the table row of position s is first_position + s.  Only where ops.fused_preparation_supported() holds."""
+    the attention gradient on them followed by the fused backward of the preparation.  first_position: an int (the
+    table row of position s is first_position + s) or the block's (B,N) position_ids tensor, any values, which is never
+    read back to the host.  Only where ops.fused_preparation_supported() holds."""
 
     @staticmethod
     def forward(ctx, q, k, v, keep, cnt, sig, rot_table=None, first_position=0, bnhd=False, merged_heads=False):
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        rotary = (rot_table, int(first_position)) if rot_table is not None else None
+        ids = first_position if torch.is_tensor(first_position) else None
+        rotary = (rot_table, ids if ids is not None else int(first_position)) if rot_table is not None else None
         out, prepared, states = ops.causal_dot_product_prepared(q, k, v, keep, cnt, sig, rotary=rotary, bnhd=bnhd,
                                                                 merged_heads=merged_heads, want_prepared=True,
                                                                 save_states=True)
-        ctx.save_for_backward(q, k, v, keep, cnt, sig, rot_table, *prepared, *(() if states is None else (states,)))
-        ctx.first_position, ctx.bnhd, ctx.merged = int(first_position), bool(bnhd), bool(merged_heads)
+        ctx.save_for_backward(q, k, v, keep, cnt, sig, rot_table, ids, *prepared, *(() if states is None else (states,)))
+        ctx.first_position = 0 if ids is not None else int(first_position)
+        ctx.bnhd, ctx.merged = bool(bnhd), bool(merged_heads)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        q, k, v, keep, cnt, sig, rot_table, qh, kh, vh, *states = ctx.saved_tensors
+        q, k, v, keep, cnt, sig, rot_table, ids, qh, kh, vh, *states = ctx.saved_tensors
         gq, gk, gv = ops.causal_backward(qh, kh, vh, grad_output.contiguous().to(qh.dtype), merged_heads=ctx.merged,
                                          saved=states[0] if states else None)
         rotary = None
         if rot_table is not None:
             b, n = (q.shape[0], q.shape[1]) if ctx.bnhd else (q.shape[0], q.shape[2])
-            pos = torch.arange(ctx.first_position, ctx.first_position + n, device=q.device).expand(b, n)
+            if ids is not None:
+                pos = (ids if ids.dim() == 2 else ids[None, :]).expand(b, n)
+            else:
+                pos = torch.arange(ctx.first_position, ctx.first_position + n, device=q.device).expand(b, n)
             rotary = (rot_table, pos)
         want = sig is not None and ctx.needs_input_grad[5]
         dq, dk, dv, dsig = ops.prepare_inputs_backward(q, k, v, gq, gk, gv, keep, cnt, sig, want_dsig=want, rotary=rotary,

@@ -643,7 +643,7 @@ int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtyp
 namespace {
 int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out,
                   void *v_out, const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
-                  long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved, int chunks_per_cut,
+                  const long long *pos_ids, long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved, int chunks_per_cut,
                   int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *stream) {
     if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
     if (dtype != COTT_BF16 && dtype != COTT_F16)
@@ -669,6 +669,8 @@ int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, v
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(q_out) || !aligned16(k_out) ||
         !aligned16(v_out) || !aligned16(rot_table))
         return fail(COTT_ERR_INVALID, "%s: tensor pointers must be 16-byte aligned", fn);
+    if (reinterpret_cast<uintptr_t>(pos_ids) & 7u) return fail(COTT_ERR_INVALID, "%s: position ids must be 8-byte aligned", fn);
+    if ((long)N > (1L << 28)) return fail(COTT_ERR_UNSUPPORTED, "%s: N = %d exceeds 2^28", fn, N);
     Op op{q, k, v, o, Dk, Dv, 0};
     op.H = H;
     if (in_bnhd) op.lay[0] = op.lay[1] = op.lay[2] = 1;
@@ -688,6 +690,7 @@ int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, v
     prep.cnt = cnt;
     prep.sig = sig;
     prep.rot = rot_table;
+    prep.pos = rot_table ? pos_ids : nullptr;
     prep.pos0 = pos0;
     prep.R = rot_table ? rotary_dim : 0;
     prep.table_rows = table_rows;
@@ -702,19 +705,19 @@ int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, v
 
 int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
                          const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
-                         long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, int B, int H, int N, int Dk,
-                         int Dv, int dtype, void *stream) {
-    return fwd_prep_impl("cott_causal_fwd_prep", q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos0, rotary_dim,
+                         const long long *pos_ids, long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, int B,
+                         int H, int N, int Dk, int Dv, int dtype, void *stream) {
+    return fwd_prep_impl("cott_causal_fwd_prep", q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos_ids, pos0, rotary_dim,
                          table_rows, in_bnhd, o_bnhd, nullptr, 0, 0, B, H, N, Dk, Dv, dtype, stream);
 }
 
 int cott_causal_fwd_prep_save(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
                               const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
-                              long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved,
+                              const long long *pos_ids, long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved,
                               int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *stream) {
     const char *fn = "cott_causal_fwd_prep_save";
     if ((long)B * H * N != 0 && saved == nullptr) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
-    return fwd_prep_impl(fn, q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos0, rotary_dim, table_rows,
+    return fwd_prep_impl(fn, q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos_ids, pos0, rotary_dim, table_rows,
                          in_bnhd, o_bnhd, saved, chunks_per_cut, ncuts, B, H, N, Dk, Dv, dtype, stream);
 }
 

@@ -56,6 +56,7 @@ struct SetArgs {
         bool on = false;
         const unsigned char *keep = nullptr;
         const float *cnt = nullptr, *sig = nullptr, *rot = nullptr;
+        const long long *pos = nullptr;  // (B,N) position ids, or null: consecutive positions from pos0
         long long pos0 = 0;
         int R = 0, table_rows = 0, H = 1, dv = 0;
         float eps = 1e-12f;

@@ -118,13 +118,15 @@ struct Tiling {
 // q, k, v are the RAW projections; every tile is prepared on its way from registers to LDS (k, v: loader
 // wavefronts) or to the MFMA operands (q: output wavefronts):
 //     q_hat = keep * rot(q) / max(|q|, eps),  k_hat likewise,  v_hat = keep * v / max(cnt ^ sig[h], 1)
-// with rot the GPT-J rotation of the first R columns by the table row of the position (row = pos0 + s, clamped to
-// the table).  The prepared rows also go to qo / ko / vo, (BH,N,D) tensors, for the backward pass.
+// with rot the GPT-J rotation of the first R columns by the table row of the position (row = pos[b][s], or pos0 + s
+// when no position ids are given, clamped to the table).  The prepared rows also go to qo / ko / vo, (BH,N,D)
+// tensors, for the backward pass.
 struct PrepSide {
     const unsigned char *keep;  // (B,N) 0 / 1, or null
     const float *cnt;           // (B,N) and
     const float *sig;           // (H): value scaling, or both null
     const float *rot;           // (table_rows, R) [sin | cos], or null
+    const long long *pos;       // (B,N) position ids (table row of every position), or null: row = pos0 + s
     long long pos0;
     int R, table_rows, H;
     int dv;                     // full width of the value rows (a problem may own a column slice of them)
@@ -153,8 +155,7 @@ __device__ __forceinline__ void rotate8(float *x, f32x4 sn, f32x4 cs) {
         x[2 * e + 1] = od * cs[e] + ev * sn[e];
     }
 }
-__device__ __forceinline__ int table_row(const PrepSide &ps, int s) {
-    long long t = ps.pos0 + s;
+__device__ __forceinline__ int clamp_row(const PrepSide &ps, long long t) {
     return (int)(t < 0 ? 0 : (t >= ps.table_rows ? ps.table_rows - 1 : t));
 }
 // Sum of v over the LANES (4, 8 or 16) consecutive, aligned lanes that hold one row, left in every one of them:
@@ -557,8 +558,32 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
         const int pc = min(p, r.p1 - 1);
         return (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
     };
+    // Position ids, when given, are fetched one call of load_chunk ahead of the table entries they select (a load whose
+    // address depends on a load issued in the same call would make that call wait for everything in flight).  The
+    // chunks are loaded in walking order, so the next call is the next chunk.  A descriptor of zero bytes stands in
+    // when there are none: the loads return zero and the row is pos0 + s.
+    const bool has_pos = ps.pos != nullptr && ps.rot != nullptr;
+    const rsrc_t rPos = make_rsrc(has_pos ? ps.pos + tok0 : nullptr, has_pos ? (uint32_t)r.N * 8u : 0u);
+    u32x2 pnext[NB];
+    auto fetch_positions = [&](int p) {
+        const int row0 = row0_of(p);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int srow = min(row0 + (tid + LT * u) / (DI / 8), r.N - 1);
+            pnext[u] = __builtin_amdgcn_raw_buffer_load_b64(rPos, (int)((uint32_t)srow * 8u), 0, 0);
+        }
+    };
+    fetch_positions(r.p0);
     auto load_chunk = [&](int s, int p) {
         const int row0 = row0_of(p);
+        int trow[NB];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int srow = min(row0 + (tid + LT * u) / (DI / 8), r.N - 1);
+            const long long given = (long long)(((unsigned long long)pnext[u].y << 32) | pnext[u].x);
+            trow[u] = clamp_row(ps, has_pos ? given : ps.pos0 + srow);
+        }
+        fetch_positions(p + 1);
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
             const int v = tid + LT * u;
@@ -568,7 +593,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
             const int srow = min(row, r.N - 1);
             keep_ab[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
             if (ps.rot != nullptr && col < ps.R) {
-                const float *t = ps.rot + (size_t)table_row(ps, srow) * ps.R + col / 2;
+                const float *t = ps.rot + (size_t)trow[u] * ps.R + col / 2;
                 sn[s][u] = *reinterpret_cast<const f32x4 *>(t);
                 cs[s][u] = *reinterpret_cast<const f32x4 *>(t + ps.R / 2);
             }

@@ -144,8 +144,9 @@ class GPTCosAttention(nn.Module):
         rotation, the head permute and the preparation steps are one fused pass.
         merge_heads: the caller wants the output as (B,S,H,D) (:500); returned that way, with None in place of
         the second value, when the training path can write it directly, else (B,H,S,D) as usual.
-        first_position: the positions are first_position, first_position + 1, ... (the caller made them itself); the
-        preparation then runs inside the attention kernel where that is built."""
+        first_position: an int when the positions are first_position, first_position + 1, ... (the block made them
+        itself), else None; the preparation runs inside the attention kernel where that is built, with the consecutive
+        positions or with the caller's position_ids as they are."""
         if bnhd:
             b, s, h, _ = query.shape
         else:
@@ -175,13 +176,14 @@ class GPTCosAttention(nn.Module):
         # kept keys at positions <= s (:241)
         cnt = cnt_all if cnt_all is not None else keep.to(torch.float32).cumsum(-1)
         dt = _autocast_target(query)
-        if (bnhd and first_position is not None and merge_heads and query.dtype == dt
+        if (bnhd and merge_heads and query.dtype == dt and (table is None or first_position is not None or pos is not None)
                 and ops.fused_preparation_supported(dt, b, h, s, query.shape[-1], value.shape[-1],
                                                     0 if table is None else table.shape[-1])
                 and ops.merged_heads_supported(dt, s, h, query.shape[-1], value.shape[-1])):
             # one forward launch: rotation, normalisation, value scaling, mask and the attention op
             return PreparedCausalAttention.apply(query, key, value, None if attention_mask is None else keep, cnt, sig,
-                                                 table, first_position, True, True), None
+                                                 table, first_position if first_position is not None else pos, True,
+                                                 True), None
         q, k, v = PrepareInputs.apply(query, key, value, keep, cnt, sig, dt, table, pos, bnhd)
         if merge_heads and ops.merged_heads_supported(q.dtype, s, h, q.shape[-1], v.shape[-1]):
             return CustomAttentionMergedHeads.apply(q, k, v), None

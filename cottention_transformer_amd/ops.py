@@ -233,8 +233,10 @@ def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=N
                                 want_prepared=True, save_states=False):
     """Causal forward on the RAW projections q, k, v: rotation, normalisation, value scaling and masking
     (prepare_inputs) happen inside the attention kernel (GPT_Trainer/GPTCosAttention.py:229-248, 462-476 in front
-    of :282 as one launch).  rotary = (table (P,R) fp32, first position): the table row of position s is
-    first position + s.  bnhd: q, k, v are (B,N,H,D); merged_heads: o is returned as (B,N,H,Dv).
+    of :282 as one launch).  rotary = (table (P,R) fp32, positions): positions is either an int, the table row of
+    position s then being that int + s, or the (B,N) integer position_ids tensor of the block (:458), any values
+    (rows outside the table are clamped to it on the device; nothing is read back).  bnhd: q, k, v are (B,N,H,D);
+    merged_heads: o is returned as (B,N,H,Dv).
     Returns (o, (q_hat, k_hat, v_hat)) with the prepared tensors (B,H,N,D) that the backward pass needs, or
     (o, None) when want_prepared is false.  Raises where fused_preparation_supported() is false.
     save_states: returns (o, prepared, saved) with the states causal_backward(q_hat, k_hat, v_hat, ..., saved=saved)
@@ -245,13 +247,20 @@ def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=N
         raise RuntimeError("Q, K and V must have the same dtype")
     code = _dtype_code(q)
     keep, cnt, sig = _prep_side_inputs(b, h, n, keep, cnt, sig, q.device)
-    table, pos0, rdim, rows = None, 0, 0, 0
+    table, pos0, rdim, rows, pos_ids = None, 0, 0, 0, None
     if rotary is not None:
         table, pos0 = rotary
         if table.dim() != 2 or table.size(1) % 8 != 0 or table.size(1) > dk:
             raise RuntimeError("rotary table must be (positions, rotary_dim), rotary_dim a multiple of 8 and <= Dk")
         table = table.to(device=q.device, dtype=torch.float32).contiguous()
         rows, rdim = table.shape
+        if torch.is_tensor(pos0):
+            if pos0.dim() == 1:
+                pos0 = pos0[None, :]
+            if pos0.shape[-1] != n or pos0.shape[0] not in (1, b) or pos0.dim() != 2:
+                raise RuntimeError(f"position ids must be (B,N) = {(b, n)}, got {tuple(pos0.shape)}")
+            pos_ids = pos0.to(device=q.device, dtype=torch.int64).expand(b, n).contiguous()
+            pos0 = 0
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     o = torch.empty((b, n, h, dv) if merged_heads else (b, h, n, dv), dtype=q.dtype, device=q.device)
     prepared = None
@@ -265,7 +274,8 @@ def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=N
     with _on(q.device):
         head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                 *((t.data_ptr() for t in prepared) if prepared else (None, None, None)),
-                _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), int(pos0), rdim, rows, int(bool(bnhd)), int(bool(merged_heads)))
+                _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), _ptr(pos_ids), int(pos0), rdim, rows, int(bool(bnhd)),
+                int(bool(merged_heads)))
         if plan is not None:
             cpc, cuts, slot, _ = plan
             saved = torch.empty((b, h, cuts, slot), dtype=torch.float32, device=q.device)
@@ -539,6 +549,8 @@ def _rotary_args(rotary, b, n, dk, device, check=True):
     table, pos = rotary
     if table.dim() != 2 or table.size(1) % 4 != 0 or table.size(1) > dk:
         raise RuntimeError("rotary table must be (positions, rotary_dim), rotary_dim a multiple of 4 and <= Dk")
+    if pos.dim() == 2 and pos.shape == (1, n):  # one row for the whole batch, as GPT-J's model makes them
+        pos = pos.expand(b, n)
     if pos.shape != (b, n):
         raise RuntimeError(f"position ids must have shape {(b, n)}")
     # (this check reads the positions back and so waits for the device; callers in a hot loop pass check=False,

@@ -258,8 +258,9 @@ COTT_API int cott_prep_ex_bwd(const void *q, const void *k, const void *v,
  * (GPT_Trainer/GPTCosAttention.py:229-248 normalise / scale / mask and :462-476 rotary, in front of :282).
  * q_out, k_out, v_out: (B,H,N,D) receive q_hat, k_hat, v_hat for the backward pass (cott_causal_bwd on them, then
  * cott_prep_ex_bwd); any of them may be NULL.  keep, cnt, sig as in cott_prep_fwd.  rot_table: (table_rows,
- * rotary_dim) fp32 as in cott_prep_ex_fwd, rotary_dim a multiple of 8, or NULL; the table row of position s is
- * pos0 + s (clamped to the table): positions that are not consecutive take cott_prep_ex_fwd.  in_bnhd: q, k, v
+ * rotary_dim) fp32 as in cott_prep_ex_fwd, rotary_dim a multiple of 8, or NULL; the table row of position s of batch
+ * element b is pos_ids[b * N + s] (position_ids of GPT_Trainer/GPTCosAttention.py:458: int64, (B,N), any values) or,
+ * with pos_ids NULL, pos0 + s; rows outside the table are clamped to it.  in_bnhd: q, k, v
  * are (B,N,H,D); o_bnhd: o is (B,N,H,Dv).  bf16 / fp16, Dk of 32..64 and Dv of 32..128 in steps of 16, B*H large
  * enough that a head is not cut into sequence groups (wider q / k rows are faster through the separate pass):
  * cott_causal_fwd_prep_supported() says (1 / 0) whether a shape qualifies; otherwise the call returns
@@ -268,7 +269,7 @@ COTT_API int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv,
 COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o,
                          void *q_out, void *k_out, void *v_out,
                          const unsigned char *keep, const float *cnt, const float *sig,
-                         const float *rot_table, long long pos0, int rotary_dim, int table_rows,
+                         const float *rot_table, const long long *pos_ids, long long pos0, int rotary_dim, int table_rows,
                          int in_bnhd, int o_bnhd,
                          int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
 /* The non-causal counterpart: o = q_hat (k_hat^T v_hat) on the raw projections in one launch, q_hat, k_hat, v_hat as
@@ -290,8 +291,8 @@ COTT_API int cott_noncausal_fwd_prep(const void *q, const void *k, const void *v
 COTT_API int cott_causal_fwd_prep_save(const void *q, const void *k, const void *v, void *o,
                               void *q_out, void *k_out, void *v_out,
                               const unsigned char *keep, const float *cnt, const float *sig,
-                              const float *rot_table, long long pos0, int rotary_dim, int table_rows,
-                              int in_bnhd, int o_bnhd,
+                              const float *rot_table, const long long *pos_ids, long long pos0, int rotary_dim,
+                              int table_rows, int in_bnhd, int o_bnhd,
                               float *saved, int chunks_per_cut, int ncuts,
                               int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
 

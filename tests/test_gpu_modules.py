@@ -76,11 +76,14 @@ def test_gpt_block_forward_backward(mods, autocast):
         assert rel_l2(a.float(), r.numpy()) <= tol, name
 
 
+@pytest.mark.parametrize("positions", ["none", "model", "custom"])
 @pytest.mark.parametrize("masked", [False, True], ids=["no-mask", "masked"])
-def test_gpt_block_with_the_preparation_inside_the_attention_kernel(mods, masked):
-    """Enough heads that no head is cut into sequence groups, bf16 autocast, positions made by the block itself: the
-    forward of the block then runs rotation, normalisation, value scaling, mask and attention as one launch
-    (PreparedCausalAttention).  Same check as above, against the fp64 CPU statement of the block."""
+def test_gpt_block_with_the_preparation_inside_the_attention_kernel(mods, masked, positions):
+    """Enough heads that no head is cut into sequence groups, bf16 autocast: the forward of the block then runs rotation,
+    normalisation, value scaling, mask and attention as one launch (PreparedCausalAttention), whether the block makes
+    the positions itself (position_ids=None), receives them the way GPT-J's model passes them (one arange row for the
+    whole batch, GPT_Trainer/GPTCosAttention.py:458) or receives other ids per batch element.  Same check as above,
+    against the fp64 CPU statement of the block."""
     from unittest import mock
     from oracle import torch_forms as tf
     from cottention_transformer_amd import ops
@@ -98,12 +101,16 @@ def test_gpt_block_with_the_preparation_inside_the_attention_kernel(mods, masked
     w = [getattr(m, n).weight.detach().double().cpu().requires_grad_(True) for n in ("q_proj", "k_proj", "v_proj", "out_proj")]
     nc = m.norm_const.detach().double().cpu().reshape(-1).requires_grad_(True)
     h64 = hidden.double().requires_grad_(True)
-    ref = tf.gpt_attention_block(h64, *w, nc, cfg.num_attention_heads, cfg.rotary_dim, cfg.max_position_embeddings, keep)
+    ids = {"none": None, "model": torch.arange(0, s)[None, :],
+           "custom": torch.randint(0, cfg.max_position_embeddings, (b, s), generator=g)}[positions]
+    ref = tf.gpt_attention_block(h64, *w, nc, cfg.num_attention_heads, cfg.rotary_dim, cfg.max_position_embeddings, keep,
+                                 position_ids=None if ids is None else ids.expand(b, s))
     ref_grads = torch.autograd.grad(ref, [h64, *w, nc], gout.double())
     hd = hidden.to(DEV).requires_grad_(True)
     with mock.patch.object(ops, "causal_dot_product_prepared", wraps=ops.causal_dot_product_prepared) as spy:
         with torch.autocast("cuda", dtype=torch.bfloat16):
-            out, present = m(hd, attention_mask=additive_mask(keep).to(DEV) if masked else None)
+            out, present = m(hd, attention_mask=additive_mask(keep).to(DEV) if masked else None,
+                             position_ids=None if ids is None else ids.to(DEV))
         assert spy.call_count == 1, "the fused forward was not taken"
     assert rel_l2(out.float(), ref.detach().numpy()) <= 3e-2
     out.backward(gout.to(DEV).to(out.dtype))

@@ -799,6 +799,56 @@ def test_input_preparation_inside_the_forward_kernel(ct, oracle, case):
         assert got.shape == ref.shape and rel_l2(got, ref.numpy()) <= 2e-2, name
 
 
+@pytest.mark.parametrize("case", [(8, 16, 256, 64, 64, BF, 64, True), (4, 32, 1000, 64, 128, HF, 16, False)],
+                         ids=["8x16x256-bf16-bnhd", "4x32x1000-fp16"])
+def test_fused_preparation_with_position_ids(ct, oracle, case):
+    """cott_causal_fwd_prep with the block's own position_ids tensor (GPT_Trainer/GPTCosAttention.py:458): ids that are
+    neither consecutive nor equal across the batch, one row repeated for the whole batch as GPT-J's model passes them,
+    and ids outside the table (clamped on the device), forward and gradients, against the CPU statements."""
+    from oracle import torch_forms as tf
+    b, h, n, dk, dv, dt, rdim, bnhd = case
+    say("fused preparation, position ids", case)
+    g = torch.Generator().manual_seed(n + rdim)
+    shape = (lambda d: (b, n, h, d)) if bnhd else (lambda d: (b, h, n, d))
+    q, k, v = (torch.randn(shape(d), generator=g).to(dt) for d in (dk, dk, dv))
+    keep = torch.rand(b, n, generator=g) > 0.2
+    sig = torch.sigmoid(torch.randn(h, generator=g))
+    go = torch.randn(b, h, n, dv, generator=g).to(dt)
+    rows = n + 40
+    table = tf.gptj_sinusoid_table(rows, rdim).float()
+    for kind in ("scattered", "one row", "outside the table"):
+        if kind == "scattered":
+            ids = torch.randint(0, rows, (b, n), generator=g)
+        elif kind == "one row":
+            ids = torch.arange(7, 7 + n)[None, :]
+        else:
+            ids = torch.randint(-5, rows + 9, (b, n), generator=g)
+        ref_ids = ids.clamp(0, rows - 1).expand(b, n)
+        q64, k64, v64, s64 = (t.double().requires_grad_(True) for t in (q, k, v, sig))
+        qh, kh, vh = ((t.permute(0, 2, 1, 3) if bnhd else t) for t in (q64, k64, v64))
+        sin, cos = torch.split(table.double()[ref_ids], rdim // 2, dim=-1)
+        rot = lambda x: torch.cat([tf.gptj_rotate(x.permute(0, 2, 1, 3)[..., :rdim], sin, cos).permute(0, 2, 1, 3),
+                                   x[..., rdim:]], -1)
+        rq, rk, rv, cnt = tf.input_prep_gpt(rot(qh), rot(kh), vh, keep, s64)
+        ref_o = oracle.causal(rq.detach(), rk.detach(), rv.detach())
+        d_prepared = [torch.from_numpy(x) for x in oracle.causal_bwd(rq.detach(), rk.detach(), rv.detach(), go)]
+        ref_grads = torch.autograd.grad([rq, rk, rv], [q64, k64, v64, s64], d_prepared)
+        o, prepared = ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV), keep=keep.to(DEV), cnt=cnt.float().to(DEV),
+                                                     sig=sig.to(DEV), rotary=(table.to(DEV), ids.to(DEV)), bnhd=bnhd)
+        assert rel_l2(o, ref_o) <= TOL[dt], kind
+        for name, got, ref in zip("qkv", prepared, (rq, rk, rv)):
+            assert rel_l2(got, ref.detach().numpy()) <= TOL[dt], (kind, name)
+        if kind == "outside the table":
+            continue  # (the separate backward of the preparation clamps the same way; covered by its own test)
+        qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sig))
+        out = ct.PreparedCausalAttention.apply(qd, kd, vd, keep.to(DEV), cnt.float().to(DEV), sd, table.to(DEV), ids.to(DEV),
+                                               bnhd, False)
+        assert rel_l2(out, ref_o) <= TOL[dt], kind
+        out.backward(go.to(DEV))
+        for name, got, ref in zip(("dq", "dk", "dv", "dsig"), (qd.grad, kd.grad, vd.grad, sd.grad), ref_grads):
+            assert got.shape == ref.shape and rel_l2(got, ref.numpy()) <= 2e-2, (kind, name)
+
+
 NC_FUSED_PREP_CASES = [
     # b, h, n, dk, dv, dtype, projections' layout, masked      launch form
     (32, 12, 512, 64, 64, BF, True, True),     # the BERT-base shape: two column halves per head, eight chunks

@@ -135,7 +135,7 @@ def test_c_abi_argument_errors_without_a_gpu():
     assert L.cott_causal_fwd_bnhd(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, None, 0, None) == _loader.OK
     # preparation inside the forward kernel: 16-bit MFMA shapes, rotary width a multiple of 8, one group per head
     prep = lambda *shape_dtype, rot=None, rdim=0, rows=0: L.cott_causal_fwd_prep(
-        16, 16, 16, 16, None, None, None, None, None, None, rot, 0, rdim, rows, 0, 0, *shape_dtype, None)
+        16, 16, 16, 16, None, None, None, None, None, None, rot, None, 0, rdim, rows, 0, 0, *shape_dtype, None)
     assert prep(8, 16, 256, 64, 64, _loader.F32) == _loader.ERR_UNSUPPORTED
     assert "bf16 / fp16" in _loader.last_error()
     assert prep(8, 16, 256, 256, 64, _loader.BF16) == _loader.ERR_UNSUPPORTED
