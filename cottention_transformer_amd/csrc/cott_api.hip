@@ -168,8 +168,12 @@ bool pair_eligible(const Op *ops, int n, int dtype, bool causal) {
 SetPlan plan_set(long BH, int N, int nops, int di, int dj, bool causal, int dtype, bool no_split = false,
                  bool has_ext = false) {
     SetPlan p;
-    // the fp32 kernels are MFMA-bound with four wavefronts per workgroup: two workgroups per CU overlap well
-    const long tgt = target_workgroups() * (dtype == COTT_F32 ? 2 : 1);
+    // the kernels on the fp32 matrix pipe are bound by it, with four wavefronts per workgroup: two workgroups per CU
+    // overlap well.  Causal fp32 ops of padded head dims 64 x 64 run from split operands on the bf16 matrix cores,
+    // one workgroup of eight wavefronts per CU like the 16-bit kernels.
+    const bool f32_split = dtype == COTT_F32 && causal && cott::mfma_pad(di) == 64 && cott::mfma_pad(dj) == 64 &&
+                           exp_int("COTT_F32_SPLIT", 1) != 0;
+    const long tgt = target_workgroups() * ((dtype == COTT_F32 && !f32_split) ? 2 : 1);
     const bool can_split = !no_split && dtype != COTT_F32 && dj >= 64 && dj % 32 == 0 && 2 * nops <= 6;
     const int pol = split_policy();
     const long xcds = device_xcds();

@@ -1,12 +1,40 @@
 // fp32 storage on the fp32 MFMA: launchers for one padded (DI, DJ) pair.
 #include "cott_mfma_launch.inc"
 #include "cott_mfma_f32.h"
+#include "cott_split.h"
 
 namespace cott {
 namespace {
 
+// Padded head dims 64 x 64: the products run on the bf16 matrix cores from split operands (cott_split.h).
+template <int DI, int DJ>
+hipError_t run_causal_split(const SetArgs &a) {
+    using TL = Tiling<DI, DJ>;
+    constexpr int PF = 2;
+    const ProblemSetF ps = make_set<float, DI, DJ>(a);
+    if (a.G > 1) {
+        if (ps.nact > 0) {
+            ProfScope prof(K_GROUP_STATE, a.stream);
+            group_state_split_kernel<DI, DJ, PF><<<dim3(grid_for(a.BH, ps.nact, a.G - 1, a.xcds)), dim3(kThreads), 0, a.stream>>>(
+                ps, a.BH, a.N, a.nchunks, a.cpg, a.G, a.G - 1);
+        }
+        const int bps = (TL::STATE_FLOATS / 4 + kThreads - 1) / kThreads;
+        ProfScope prof(K_STATE_PREFIX, a.stream);
+        state_prefix_kernel<float><<<dim3((unsigned)(a.BH * ps.count * bps)), dim3(kThreads), 0, a.stream>>>(
+            ps, a.BH, a.G, 1, a.G - 1, TL::STATE_FLOATS, 0);
+    }
+    ProfScope prof(a.scan_prof_id, a.stream);
+    split_scan_kernel<DI, DJ, PF><<<dim3(grid_for(a.BH, a.count, a.G, a.xcds)), dim3(512), 0, a.stream>>>(
+        ps, a.BH, a.N, a.nchunks, a.cpg, a.G);
+    return hipGetLastError();
+}
+
 template <int DI, int DJ>
 hipError_t run_causal_f32(const SetArgs &a) {
+    if constexpr (DI == 64 && DJ == 64) {
+        static const int split = exp_env("COTT_F32_SPLIT", 1);
+        if (split) return run_causal_split<DI, DJ>(a);
+    }
     using TL = TilingF32<DI, DJ>;
     const ProblemSetF32 ps = make_set<float, DI, DJ>(a);
     if (a.G > 1) {

@@ -304,10 +304,14 @@ def test_prefill_hands_state_to_next_piece_and_to_decode(ct, oracle, case):
     assert s2.dtype == (F64 if dt == F64 else F32) and s2.shape == (b, h, dk, dv)
     assert rel_l2(torch.cat([o1, o2], 2), ref[:, :, :n]) <= TOL[dt]
     kv = np.einsum("bhni,bhnj->bhij", k[:, :, :n].double().numpy(), v[:, :, :n].double().numpy())
-    assert rel_l2(s2, kv) <= (1e-12 if dt == F64 else 2e-6)
+    # fp32 state from 16-bit inputs: the products are exact, only the fp32 sums round (2e-6).  fp32 inputs of 33..64
+    # columns are multiplied as split bf16 operands, 16 of their 24 significant bits (about 6e-6 per product, the
+    # arithmetic of every fp32 result of those shapes, bounded well inside the 1e-4 of fp32 inputs)
+    state_tol = 1e-12 if dt == F64 else (2e-5 if dt == F32 else 2e-6)
+    assert rel_l2(s2, kv) <= state_tol
     # one call over the whole prompt gives the same state
     o, s = ct.causal_prefill(qd[:, :, :n], kd[:, :, :n], vd[:, :, :n])
-    assert rel_l2(o, ref[:, :, :n]) <= TOL[dt] and rel_l2(s, kv) <= (1e-12 if dt == F64 else 2e-6)
+    assert rel_l2(o, ref[:, :, :n]) <= TOL[dt] and rel_l2(s, kv) <= state_tol
     if dv % 4 == 0:
         rows = [ct.decode_step(s2, qd[:, :, t], kd[:, :, t], vd[:, :, t]) for t in range(n, n + extra)]
         assert rel_l2(torch.stack(rows, 2), ref[:, :, n:]) <= TOL[dt]
