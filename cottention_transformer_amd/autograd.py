@@ -1,6 +1,7 @@
 """torch.autograd boundary: `CustomAttention` with the reference's signature, plus the
 non-causal counterpart.  Reference: Cuda_Kernel/Custom_Kernel.py:7-141."""
 import torch
+import torch.nn.utils.parametrize
 
 from . import ops
 
@@ -282,8 +283,25 @@ class InputProjections(torch.autograd.Function):
         return tuple(grads)
 
 
+def _is_plain_linear(lin):
+    """Whether calling the layer is nothing but x w^T + b with the parameters it holds: exactly torch.nn.Linear, no
+    forward (pre-)hooks and no parametrization.  Adapters, quantised linears and hooked layers must be CALLED."""
+    if type(lin) is not torch.nn.Linear:
+        return False
+    if lin._forward_hooks or lin._forward_pre_hooks or getattr(lin, "_forward_hooks_with_kwargs", None):
+        return False
+    if getattr(torch.nn.modules.module, "_global_forward_hooks", None) or getattr(
+            torch.nn.modules.module, "_global_forward_pre_hooks", None):
+        return False
+    return not torch.nn.utils.parametrize.is_parametrized(lin)
+
+
 def project(x, *linears):
-    """The outputs of the given nn.Linear layers on x, through `InputProjections`."""
+    """The outputs of the given nn.Linear layers on x: through `InputProjections` when every layer is a plain
+    nn.Linear, else by calling the layers as the reference does (GPT_Trainer/GPTCosAttention.py:443-445), so that hooks,
+    parametrizations and subclasses (LoRA adapters, quantised linears) keep their effect."""
+    if not all(_is_plain_linear(lin) for lin in linears):
+        return tuple(lin(x) for lin in linears)
     args = []
     for lin in linears:
         args += [lin.weight, lin.bias]

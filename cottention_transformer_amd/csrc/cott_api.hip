@@ -329,7 +329,10 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
     // does not fill the chip, every group is cut into up to four pieces (one workgroup and one slot each).  With k
     // workgroups on the fullest CU the pass takes about k * (1.15 if k == 2) / pieces of its one-piece time
     // (measured at B1 H16 N65536 D128: 144 workgroups 194 us, 288: 193, 432: 158, 576: 187; 240 -> 480: 84 -> 90).
-    if (p.G > 1 && half) {
+    // (fp32 ops on split operands have a group-state pass of the same kind, one 80 KiB workgroup per CU)
+    const bool split32 = dtype == COTT_F32 && causal && cott::mfma_pad(first.di) == 64 && cott::mfma_pad(first.dj) == 64 &&
+                         exp_int("COTT_F32_SPLIT", 1) != 0;
+    if (p.G > 1 && (half || split32)) {
         long wgs = 0;
         if (L.pair)
             wgs = (ops[members[0]].ext != nullptr ? 1L : 2L) * (p.G - 1);
@@ -347,7 +350,7 @@ SetLayout layout_set(const Op *ops, int n, const int *members, int cnt, long BH,
         for (int s = 1; s <= 4; ++s) {
             if (s > 1 && (p.cpg + s - 1) / s < 4) break;
             const long k = (wgs * s + cus - 1) / cus;
-            if (k > 2) break;
+            if (k > (split32 ? 1 : 2)) break;
             const double cost = (double)k * (k == 2 ? 1.15 : 1.0) / s;
             if (cost < best - 1e-9) {
                 best = cost;

@@ -12,7 +12,8 @@
 //   * A_c S_c for its columns comes straight from its own accumulators: converted to 16 bits in registers they ARE the
 //     A operand of the product (see the row order below), so the state is never written to or read from LDS;
 //   * the ten masked score tiles on the live side of the diagonal are formed once per workgroup, three to a
-//     wavefront, and handed round through 5 KiB of LDS at a second barrier in the middle of the chunk;
+//     wavefront, and handed round through 5 KiB of LDS; the product that needs them is finished at the start of the
+//     next chunk, so the one barrier per chunk covers the hand-over;
 //   * the C fragments of its columns serve both the score-times-C product and the state update.
 // About 86 matrix instructions per wavefront and chunk on each of the four SIMDs, and 30 % less LDS traffic.
 // Four loader wavefronts stage THREE tiles per chunk (the A rows as well: all four compute wavefronts read them) and
@@ -22,7 +23,8 @@
 // What it buys is modest, and the measurements that say why are worth keeping next to the code.  At B1 H16 N65536
 // D128 (three gradient problems per head in 5 groups, 240 workgroups) this kernel with its compute wavefronts idle,
 // i.e. the loaders alone moving the launch's 1.97 GB, takes 389 us (5.1 TB/s); with all matrix instructions but no
-// LDS reads in the compute wavefronts 390 us; complete 448 us (scan_kernel: 467 us).  Under the profiler's counter
+// LDS reads in the compute wavefronts 390 us; complete 434 us (scan_kernel: 467 us; 448 us with a second barrier per chunk for
+// the score tiles instead of finishing each chunk after the barrier that ends it).  Under the profiler's counter
 // collection, which leaves gaps between kernels, the complete kernel takes 404 us at 2.28 GHz against 383 us at
 // 2.44 GHz idle (GRBM_GUI_ACTIVE over the duration): the data path through the chip scales with the core clock, the
 // core clock gives way under the power the products draw, and in a loop of back-to-back launches it gives way
@@ -56,7 +58,7 @@ struct ColTiling {
 };
 
 // Loader role: LT threads move the A, B and C tiles global -> registers -> LDS, PF chunks ahead, and send the output
-// tile that the compute wavefronts finished one chunk earlier from LDS to memory.  Loads and stores are unconditional
+// tile that the compute wavefronts finished one chunk earlier (i.e. the tile of the chunk two before) from LDS to memory.  Loads and stores are unconditional
 // (rows past N read as zero and are dropped on the way out: buffer range check).
 template <int DI, int DJ, int PF, int LT, bool STREAM>
 __device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_head, const u16 *C_head, u16 *O_head, int di,
@@ -103,10 +105,11 @@ __device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_
         store_tile<DI, TL::BS, LT>(sB + (buf ^ 1) * CT::SA, rb[s1], di, tid);
         store_tile<DJ, TL::CS, LT>(sC + (buf ^ 1) * CT::SC, rc[s1], dj, tid);
         load_chunk(s1, p + 1 + PF);
-        chunk_barrier();  // (the compute wavefronts hand their score tiles round here)
-        if (p > r.p0) write_out(p - 1);
+        if (p > r.p0 + 1) write_out(p - 2);  // (the compute wavefronts finish a chunk's tile at the start of the next chunk)
         chunk_barrier();
     });
+    if (r.p1 > r.p0 + 1) write_out(r.p1 - 2);
+    __syncthreads();  // the last chunk's tile is finished after the loop
     if (r.p1 > r.p0) write_out(r.p1 - 1);
 }
 
@@ -126,10 +129,9 @@ struct ColStateIO {
 // Compute role: wavefront w of 4 owns column tiles NJW * w .. NJW * w + NJW - 1.  FUT: the scores that count are
 // those of keys at or after the query (ops that sum over the future, or over the past in complement form).
 // The ten score tiles on the live side of the diagonal are dealt three to a wavefront (the last wavefront forms its
-// one tile three times), left in LDS (sP: 16 tiles of 512 bytes in accumulator order, which is operand order for the
-// next product), and after a second barrier in the middle of the chunk every wavefront reads the tiles of all blocks.
-// Everything that does not need the scores (A_c S_c for all blocks, the state update) sits between writing the tiles
-// and that barrier, so nobody waits long at it.
+// one tile three times) and left in LDS (sP: 16 tiles of 512 bytes in accumulator order, which is operand order for the
+// next product, double-buffered); every wavefront reads the tiles of all blocks after the barrier that ends the chunk
+// and finishes the chunk's outputs then, before it starts on the next chunk.
 // The chunk is written as a software pipeline: the LDS reads of step k + 1 are issued, as a block, before the matrix
 // instructions of step k, and scheduling fences keep the compiler from sinking them back down to their first use
 // (left to itself it places every read a few instructions before the product that needs it, and the wavefront then
@@ -228,11 +230,49 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
     };
     pack_state();
     const uint32_t flip = comp ? 0x80008000u : 0u;
+    // The (scores) x C product of a chunk is finished at the start of the NEXT chunk, after the barrier that ends this
+    // one: by then every wavefront's score tiles are in LDS, and no second barrier in the middle of a chunk is needed
+    // (which would hold the loader wavefronts as well).  Carried across the barrier: the partial outputs o (A_c S_c),
+    // the C fragments, and the score tiles in the LDS buffer of the chunk's parity.
+    f32x4 o[4][NJW];
+    u32x4 cf[NJW][2];
+    auto finish = [&](int pbuf) {  // adds (scores) x C to o and leaves the tile in the staging buffer of that chunk
+        const u32x2 *tiles = sP + pbuf * 16 * 64;
+        u16 *cO = sO + pbuf * CT::SO;
+        u32x4 pf[2][2];  // the score tiles of a block are read one block ahead of their products
+        auto read_block = [&](int slot, int pb) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const u32x2 z = {0u, 0u};
+                if (live(pb, 2 * kb) || live(pb, 2 * kb + 1))
+                    pf[slot][kb] = cat(live(pb, 2 * kb) ? tiles[(pb * 4 + 2 * kb) * 64 + l] : z,
+                                       live(pb, 2 * kb + 1) ? tiles[(pb * 4 + 2 * kb + 1) * 64 + l] : z);
+            }
+        };
+        read_block(0, 0);
+        sched_fence();
+#pragma unroll
+        for (int pb = 0; pb < 4; ++pb) {
+            if (pb < 3) read_block((pb + 1) & 1, pb + 1);
+            sched_fence();
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if (!(live(pb, 2 * kb) || live(pb, 2 * kb + 1))) continue;
+#pragma unroll
+                for (int jw = 0; jw < NJW; ++jw) o[pb][jw] = TR::mfma(cf[jw][kb], pf[pb & 1][kb], o[pb][jw]);
+            }
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw)
+                *reinterpret_cast<u32x2 *>(cO + (16 * pb + m) * TL::OS + 16 * (NJW * w + jw) + 4 * g) =
+                    u32x2{TR::pack2(o[pb][jw][0], o[pb][jw][1]), TR::pack2(o[pb][jw][2], o[pb][jw][3])};
+            sched_fence();
+        }
+    };
     __syncthreads();
     for (int p = r.p0; p < r.p1; ++p) {
         const int buf = (p - r.p0) & 1;
         const u16 *cA = sA + buf * CT::SA, *cB = sB + buf * CT::SA, *cC = sC + buf * CT::SC;
-        u16 *cO = sO + buf * CT::SO;
+        u32x2 *cP = sP + buf * 16 * 64;
         // fragment readers (each a block of LDS reads, nothing else)
         u32x4 sq[2][KS], sk[2][KS];  // query rows and key rows of a score tile, two tiles in flight
         auto read_score = [&](int slot, int t) {
@@ -256,14 +296,13 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
                 const bool keep = mask_rev ? (d0 + q >= 0) : (d0 + q <= 0);
                 acc[q] = (keep != comp) ? (comp ? -acc[q] : acc[q]) : 0.f;
             }
-            sP[(spb[t] * 4 + sjt[t]) * 64 + l] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
+            cP[(spb[t] * 4 + sjt[t]) * 64 + l] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
         };
         u32x4 qf[2][KS];
         auto read_q = [&](int slot, int pb) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) qf[slot][ks] = ld128(cA + (16 * pb + m) * TL::BS + 32 * ks + 8 * g);
         };
-        f32x4 o[4][NJW];
         auto state_product = [&](int slot, int pb) {  // out^T tiles (columns 16jt + 4g .. + 3, position 16pb + m)
 #pragma unroll
             for (int jw = 0; jw < NJW; ++jw) {
@@ -276,7 +315,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
                 o[pb][jw] = o1 + o2;
             }
         };
-        u32x4 cf[NJW][2], bf[2][4];
+        u32x4 bf[2][4];
         auto read_c = [&]() {
 #pragma unroll
             for (int jw = 0; jw < NJW; ++jw)
@@ -303,6 +342,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
             }
         };
 
+        if (p > r.p0) finish(buf ^ 1);
         read_score(0, 0);
         sched_fence();
         read_score(1, 1);
@@ -336,34 +376,6 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
             update(b & 1, b / (NIT / 4), 4 * (b % (NIT / 4)));
             sched_fence();
         }
-        chunk_barrier();  // every block's score tiles are in sP
-        // ---- (scores) x C for every block, then the finished tiles go to the staging tile
-        u32x4 pf[4][2];
-#pragma unroll
-        for (int pb = 0; pb < 4; ++pb)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const u32x2 z = {0u, 0u};
-                if (live(pb, 2 * kb) || live(pb, 2 * kb + 1))
-                    pf[pb][kb] = cat(live(pb, 2 * kb) ? sP[(pb * 4 + 2 * kb) * 64 + l] : z,
-                                     live(pb, 2 * kb + 1) ? sP[(pb * 4 + 2 * kb + 1) * 64 + l] : z);
-            }
-        sched_fence();
-#pragma unroll
-        for (int pb = 0; pb < 4; ++pb) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                if (!(live(pb, 2 * kb) || live(pb, 2 * kb + 1))) continue;
-#pragma unroll
-                for (int jw = 0; jw < NJW; ++jw) o[pb][jw] = TR::mfma(cf[jw][kb], pf[pb][kb], o[pb][jw]);
-            }
-        }
-#pragma unroll
-        for (int pb = 0; pb < 4; ++pb)
-#pragma unroll
-            for (int jw = 0; jw < NJW; ++jw)
-                *reinterpret_cast<u32x2 *>(cO + (16 * pb + m) * TL::OS + 16 * (NJW * w + jw) + 4 * g) =
-                    u32x2{TR::pack2(o[pb][jw][0], o[pb][jw][1]), TR::pack2(o[pb][jw][2], o[pb][jw][3])};
         pack_state();
         if (io.save != nullptr) {  // (an op that walks forwards: p is the chunk's place in the sequence)
             const int back = r.nchunks - 1 - p;
@@ -378,6 +390,10 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
         }
         chunk_barrier();
     }
+    if (r.p1 > r.p0) {
+        finish((r.p1 - 1 - r.p0) & 1);
+    }
+    __syncthreads();  // (the loader wavefronts send the last tile out after this)
     if (io.sout != nullptr) {
 #pragma unroll
         for (int it = 0; it < NIT; ++it)
@@ -401,7 +417,7 @@ __global__ __launch_bounds__(512) void colscan_kernel(ProblemSet set, int BH, in
     __shared__ __attribute__((aligned(16))) u16 sB[2 * CT::SA];
     __shared__ __attribute__((aligned(16))) u16 sC[2 * CT::SC];
     __shared__ __attribute__((aligned(16))) u16 sO[2 * CT::SO];
-    __shared__ __attribute__((aligned(16))) u32x2 sP[16 * 64];  // masked score tiles, handed round in the middle of a chunk
+    __shared__ __attribute__((aligned(16))) u32x2 sP[2 * 16 * 64];  // masked score tiles of the current and the previous chunk
     static_assert(2 * CT::SO * 2 >= 4 * 2048, "room to turn the transposed seeds");
     const int l = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));

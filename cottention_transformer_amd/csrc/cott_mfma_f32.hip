@@ -15,13 +15,13 @@ hipError_t run_causal_split(const SetArgs &a) {
     if (a.G > 1) {
         if (ps.nact > 0) {
             ProfScope prof(K_GROUP_STATE, a.stream);
-            group_state_split_kernel<DI, DJ, PF><<<dim3(grid_for(a.BH, ps.nact, a.G - 1, a.xcds)), dim3(kThreads), 0, a.stream>>>(
+            group_state_split_kernel<DI, DJ, PF><<<dim3(grid_for(a.BH, ps.nact * a.sub, a.G - 1, a.xcds)), dim3(kThreads), 0, a.stream>>>(
                 ps, a.BH, a.N, a.nchunks, a.cpg, a.G, a.G - 1);
         }
         const int bps = (TL::STATE_FLOATS / 4 + kThreads - 1) / kThreads;
         ProfScope prof(K_STATE_PREFIX, a.stream);
         state_prefix_kernel<float><<<dim3((unsigned)(a.BH * ps.count * bps)), dim3(kThreads), 0, a.stream>>>(
-            ps, a.BH, a.G, 1, a.G - 1, TL::STATE_FLOATS, 0);
+            ps, a.BH, a.G, a.sub, a.G - 1, TL::STATE_FLOATS, 0);
     }
     ProfScope prof(a.scan_prof_id, a.stream);
     split_scan_kernel<DI, DJ, PF><<<dim3(grid_for(a.BH, a.count, a.G, a.xcds)), dim3(512), 0, a.stream>>>(

@@ -51,6 +51,11 @@ __device__ __forceinline__ void split4(f32x4 v, u32x2 &hi, u32x2 &lo) {
         lo[e] = Bf16::pack2(v[2 * e] - bitcast<float>(h << 16), v[2 * e + 1] - bitcast<float>(h & 0xffff0000u));
     }
 }
+// Term t = 0, 1, 2 of a product: a_lo b_hi, a_hi b_lo, a_hi b_hi.  Callers with several independent accumulators run term
+// 0 for all of them, then term 1, then term 2, so that a matrix instruction never follows the one it depends on.
+__device__ __forceinline__ f32x4 mfma_term(int t, u32x4 ah, u32x4 al, u32x4 bh, u32x4 bl, f32x4 c) {
+    return Bf16::mfma(t == 0 ? al : ah, t == 1 ? bl : bh, c);
+}
 // c + a b from the three leading terms of (a_hi + a_lo)(b_hi + b_lo)
 __device__ __forceinline__ f32x4 mfma3(u32x4 ah, u32x4 al, u32x4 bh, u32x4 bl, f32x4 c) {
     c = Bf16::mfma(al, bh, c);
@@ -84,7 +89,7 @@ __device__ __forceinline__ void store_tile_split(u16 *th, u16 *tl, const u32x4 (
 }
 
 // Sum of B^T C over each group of chunks of each head, in the slot layout of group_state_kernel (cott_mfma.h):
-// float4 index (w * TPW + u) * 64 + lane of slot (bh * G + grp).
+// float4 index (w * TPW + u) * 64 + lane of slot (bh * G + grp) * sub + piece.
 template <int DI, int DJ, int PF>
 __global__ __launch_bounds__(kThreads) void group_state_split_kernel(ProblemSetF set, int BH, int N, int nchunks, int cpg,
                                                                      int G, int ngroups) {
@@ -96,17 +101,27 @@ __global__ __launch_bounds__(kThreads) void group_state_split_kernel(ProblemSetF
     __shared__ __attribute__((aligned(16))) u16 sCl[2 * SC];
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = decode_workgroup(set.nact, BH, set.xcds);
+    // every group is cut into `sub` pieces, one workgroup and one slot each (slot (bh * G + grp) * sub + piece)
+    const int sub = set.sub;
+    const WorkItem wi = decode_workgroup(set.nact * sub, BH, set.xcds);
     if (wi.grp >= ngroups) return;
-    const ProblemF &pr = set.p[set.act[wi.prob]];
+    const ProblemF &pr = set.p[set.act[wi.prob / sub]];
+    const int piece = wi.prob % sub;
     const int di = pr.di, dj = pr.dj, ldb = pr.ldb, ldc = pr.ldc, reversed = pr.reversed;
     const rsrc_t rB = make_rsrc(pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh), ((uint32_t)(N - 1) * ldb + di) * 4u);
     const rsrc_t rC = make_rsrc(pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), ((uint32_t)(N - 1) * ldc + dj) * 4u);
-    const int p0 = wi.grp * cpg;
-    const int p1 = min(p0 + cpg, nchunks);
+    const int cps = (cpg + sub - 1) / sub;  // chunks per piece
+    const int p0 = wi.grp * cpg + piece * cps;
+    const int p1 = min(p0 + cps, min((wi.grp + 1) * cpg, nchunks));
     f32x4 S[TL::TPW];
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 *slot = reinterpret_cast<f32x4 *>(pr.gstate + (((size_t)wi.bh * G + wi.grp) * sub + piece) * TL::STATE_FLOATS);
+    if (p1 <= p0) {  // a piece past the end of its group: its slot is zero
+#pragma unroll
+        for (int u = 0; u < TL::TPW; ++u) slot[(w * TL::TPW + u) * 64 + l] = S[u];
+        return;
+    }
     u32x4 rb[PF][DI / 32][2], rc[PF][DJ / 32][2];
     auto load_chunk = [&](int s, int p) {
         const int pc = min(p, p1 - 1);
@@ -157,7 +172,6 @@ __global__ __launch_bounds__(kThreads) void group_state_split_kernel(ProblemSetF
         update(buf);
         chunk_barrier();
     });
-    f32x4 *slot = reinterpret_cast<f32x4 *>(pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS);
 #pragma unroll
     for (int u = 0; u < TL::TPW; ++u) slot[(w * TL::TPW + u) * 64 + l] = S[u];
 }
@@ -297,19 +311,31 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
     };
     auto finish_previous = [&](int pprev) {
         const int row0 = (r.reversed ? r.nchunks - 1 - pprev : pprev) * kChunk;
+        f32x4 acc2[4][NJW];
 #pragma unroll
-        for (int pb = 0; pb < 4; ++pb) {
+        for (int pb = 0; pb < 4; ++pb)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw) acc2[pb][jw] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 3; ++t)
+#pragma unroll
+            for (int pb = 0; pb < 4; ++pb)
+#pragma unroll
+                for (int jw = 0; jw < NJW; ++jw) {
+                    if (live(pb, 0) || live(pb, 1))
+                        o[pb][jw] = mfma_term(t, cfh[jw][0], cfl[jw][0], pfh[pb][0], pfl[pb][0], o[pb][jw]);
+                    if (live(pb, 2) || live(pb, 3))
+                        acc2[pb][jw] = mfma_term(t, cfh[jw][1], cfl[jw][1], pfh[pb][1], pfl[pb][1], acc2[pb][jw]);
+                }
+#pragma unroll
+        for (int pb = 0; pb < 4; ++pb)
 #pragma unroll
             for (int jw = 0; jw < NJW; ++jw) {
-                f32x4 acc = o[pb][jw], acc2 = {0.f, 0.f, 0.f, 0.f};
-                if (live(pb, 0) || live(pb, 1)) acc = mfma3(cfh[jw][0], cfl[jw][0], pfh[pb][0], pfl[pb][0], acc);
-                if (live(pb, 2) || live(pb, 3)) acc2 = mfma3(cfh[jw][1], cfl[jw][1], pfh[pb][1], pfl[pb][1], acc2);
-                acc += acc2;
+                const f32x4 acc = o[pb][jw] + acc2[pb][jw];
                 const int col = 16 * (NJW * w + jw) + 4 * g;
                 const uint32_t off = (col < dj) ? (uint32_t)((row0 + 16 * pb + m) * ldo + col) * 4u : kOobOffset;
                 __builtin_amdgcn_raw_buffer_store_b128(bitcast<u32x4>(acc), rO, (int)off, 0, 0);
             }
-        }
     };
     __syncthreads();
     for (int p = r.p0; p < r.p1; ++p) {
@@ -332,8 +358,12 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
         auto score_tile = [&](int slot, int t) {
             f32x4 acc[KS];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-                acc[ks] = mfma3(skh[slot][ks], skl[slot][ks], sqh[slot][ks], sql[slot][ks], f32x4{0.f, 0.f, 0.f, 0.f});
+            for (int ks = 0; ks < KS; ++ks) acc[ks] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < 3; ++t)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    acc[ks] = mfma_term(t, skh[slot][ks], skl[slot][ks], sqh[slot][ks], sql[slot][ks], acc[ks]);
 #pragma unroll
             for (int ks = 1; ks < KS; ++ks) acc[0] += acc[ks];
             const int d0 = 16 * (sjt[t] - spb[t]) + 4 * g - m;  // key position - query position at element 0
@@ -360,8 +390,12 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
             for (int jw = 0; jw < NJW; ++jw) {
                 f32x4 acc[KS];
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    acc[ks] = mfma3(soph[ks][jw], sopl[ks][jw], qfh[slot][ks], qfl[slot][ks], f32x4{0.f, 0.f, 0.f, 0.f});
+                for (int ks = 0; ks < KS; ++ks) acc[ks] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 3; ++t)
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        acc[ks] = mfma_term(t, soph[ks][jw], sopl[ks][jw], qfh[slot][ks], qfl[slot][ks], acc[ks]);
 #pragma unroll
                 for (int ks = 1; ks < KS; ++ks) acc[0] += acc[ks];
                 o[pb][jw] = acc[0];
@@ -389,10 +423,12 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
         };
         auto update = [&](int slot, int kb, int it0) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
+            for (int t = 0; t < 3; ++t)
 #pragma unroll
-                for (int jw = 0; jw < NJW; ++jw)
-                    S[it0 + e][jw] = mfma3(bfh[slot][e], bfl[slot][e], cfh[jw][kb], cfl[jw][kb], S[it0 + e][jw]);
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int jw = 0; jw < NJW; ++jw)
+                        S[it0 + e][jw] = mfma_term(t, bfh[slot][e], bfl[slot][e], cfh[jw][kb], cfl[jw][kb], S[it0 + e][jw]);
         };
 
         read_score(0, 0);
@@ -482,7 +518,7 @@ __global__ __launch_bounds__(512) void split_scan_kernel(ProblemSetF set, int BH
         return;
     }
     ColStateIO io;
-    if (pr.gstate != nullptr) io.seed = pr.gstate + ((size_t)wi.bh * G + wi.grp) * TL::STATE_FLOATS;
+    if (pr.gstate != nullptr) io.seed = pr.gstate + ((size_t)wi.bh * G + wi.grp) * set.sub * TL::STATE_FLOATS;
     if (pr.sin != nullptr) io.sin = pr.sin + (size_t)wi.bh * di * pr.lds;
     if (pr.sout != nullptr && wi.grp == G - 1) io.sout = pr.sout + (size_t)wi.bh * di * pr.lds;
     io.lds = pr.lds;

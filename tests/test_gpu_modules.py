@@ -322,6 +322,13 @@ def test_module_options_of_the_reference_signatures(mods):
         p_.requires_grad_(False)
     plain = bert(hidden, attention_mask=mask)
     assert len(plain) == 2 and plain[1][0].shape == (b, 4, s, 64) and plain[1][1].shape == (b, 4, s, 64)
+    # is_decoder: the tuple handed back is (key_layer, value_layer) as projected and split into heads, BEFORE the mask
+    # and the normalisation touch them -- a literal restatement of BERT_Trainer/BertCosAttention.py:143-144,158,332-333
+    lit_k = bert.key(hidden).view(b, s, 4, 64).permute(0, 2, 1, 3)
+    lit_v = bert.value(hidden).view(b, s, 4, 64).permute(0, 2, 1, 3)
+    assert rel_l2(plain[1][0], lit_k.double().cpu().numpy()) <= 1e-6 and rel_l2(plain[1][1], lit_v.double().cpu().numpy()) <= 1e-6
+    # output_attentions: the reference's active path never assigns attention_probs (every assignment is commented out,
+    # :198-268), so its `(context_layer, attention_probs)` at :330 would raise; here None stands in for the weights
     with_attn = bert(hidden, attention_mask=mask, output_attentions=True)
     assert len(with_attn) == 3 and with_attn[1] is None
     assert torch.equal(with_attn[0], plain[0])

@@ -124,3 +124,35 @@ def test_input_projections_equal_separate_linear_layers(bias):
     assert len(got) == len(ref)
     for a, b in zip(got, ref):
         assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
+
+
+def test_projections_call_layers_that_are_not_plain_linears():
+    """`project` reads weight and bias of plain nn.Linear layers; a layer with a forward hook, a parametrization or a
+    subclass (adapters, quantised linears) is CALLED, as the reference calls its projections
+    (GPT_Trainer/GPTCosAttention.py:443-445), so what those add is not skipped."""
+    from cottention_transformer_amd.autograd import project, _is_plain_linear
+    torch.manual_seed(0)
+    x = torch.randn(2, 3, 8, dtype=torch.float64)
+    plain = torch.nn.Linear(8, 4).double()
+    assert _is_plain_linear(plain)
+    hooked = torch.nn.Linear(8, 4).double()
+    hooked.register_forward_hook(lambda mod, inp, out: out + 1.0)
+
+    class Scaled(torch.nn.Linear):
+        def forward(self, inp):
+            return 2.0 * super().forward(inp)
+
+    sub = Scaled(8, 4).double()
+    par = torch.nn.Linear(8, 4).double()
+
+    class Double(torch.nn.Module):
+        def forward(self, w):
+            return 2.0 * w
+
+    torch.nn.utils.parametrize.register_parametrization(par, "weight", Double())
+    for lin in (hooked, sub, par):
+        assert not _is_plain_linear(lin)
+        (got,) = project(x, lin)
+        assert torch.allclose(got, lin(x), rtol=1e-12, atol=1e-12)
+    a, b2 = project(x, plain, hooked)          # one odd layer sends the whole group through the modules
+    assert torch.allclose(a, plain(x)) and torch.allclose(b2, hooked(x))
