@@ -82,8 +82,9 @@ def test_workspace_queries_are_pure_host_functions():
     # fp32 has MFMA kernels too and is cut the same way; fp64 takes the plain-FMA path -> none
     assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F32) > 0
     # (no column halves in fp32.  33..64 columns run from split bf16 operands, one workgroup per CU: 128 heads in two
-    # groups; other widths stay on the fp32 matrix pipe, two workgroups per CU: 128 heads of 32 columns in four groups)
-    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 2 * 128 * 64 * 64 * 4
+    # groups, the one group that is summed cut into two pieces with a slot each; other widths stay on the fp32 matrix
+    # pipe, two workgroups per CU: 128 heads of 32 columns in four groups)
+    assert L.cott_causal_workspace_bytes(8, 16, 2048, 64, 64, _loader.F32) == 2 * 2 * 128 * 64 * 64 * 4
     assert L.cott_causal_workspace_bytes(8, 16, 2048, 32, 32, _loader.F32) == 4 * 128 * 32 * 32 * 4
     assert L.cott_causal_workspace_bytes(32, 16, 2048, 64, 64, _loader.F32) == 0
     assert L.cott_causal_workspace_bytes(1, 2, 8192, 64, 64, _loader.F64) == 0
