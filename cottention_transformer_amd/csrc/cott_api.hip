@@ -451,9 +451,6 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         return COTT_OK;
     }
     const size_t need = ops_workspace(ops, n, BH, N, dtype, causal);
-    if (prep != nullptr && need > 0)
-        return fail(COTT_ERR_UNSUPPORTED, "%s: B*H = %ld heads are cut into sequence groups at N = %d; the fused preparation "
-                    "needs one group per head (prepare the inputs with cott_prep_ex_fwd instead)", fn, BH, N);
     if (need > 0 && (ws == nullptr || ws_bytes < need || !aligned16(ws)))
         return fail(COTT_ERR_WORKSPACE, "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", fn, need,
                     ws ? ws_bytes : (size_t)0);
@@ -467,12 +464,7 @@ int run_ops(const char *fn, bool causal, const Op *ops, int n, long BH, int N, i
         const int i = members[0];
         const SetLayout L = layout_set(ops, n, members, cnt, BH, N, dtype, causal);
         const SetPlan &p = L.p;
-        if (prep != nullptr) {
-            if (p.G != 1)
-                return fail(COTT_ERR_UNSUPPORTED, "%s: B*H = %ld heads are cut into %d sequence groups at N = %d; the fused "
-                            "preparation needs one group per head (prepare the inputs with cott_prep_ex_fwd instead)", fn, BH, p.G, N);
-            a.prep = *prep;
-        }
+        if (prep != nullptr) a.prep = *prep;
         const bool pair = L.pair, complement = L.complement;
         const int *twin_of = L.twin_of;
         a.pair = pair ? 1 : 0;
@@ -641,17 +633,19 @@ int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtyp
     if ((long)N * H * dmax > (1L << 30) || (long)B * H > (1L << 22)) return 0;
     if ((long)B * H * N == 0) return 1;
     const SetPlan p = plan_set((long)B * H, N, 1, Dk, Dv, true, dtype);
-    // one group per head, and q / k rows of at most 64 columns: with 128 the loader wavefronts hold four pieces of q and
-    // of k per chunk with their table entries, and the launch takes 400 us where the preparation pass and the plain
-    // forward take 165 (B8 H16 N2048)
-    return p.G == 1 && cott::mfma_pad(Dk) <= 64 && cott::mfma_pad(Dk) * cott::mfma_pad(Dv / p.halves) <= 128 * 64;
+    // q / k rows of up to 64 columns are prepared by scan_kernel's loader wavefronts, 128-wide rows by colscan_kernel's
+    // (value tiles of 64 or 128 columns there); sequences cut into groups take a group-state pass that prepares k and v
+    // the same way
+    const int pk = cott::mfma_pad(Dk), pv = cott::mfma_pad(Dv / p.halves);
+    return (pk <= 64 && pk * pv <= 128 * 64) || (pk == 128 && pv >= 64);
 }
 
 namespace {
 int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out,
                   void *v_out, const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
                   const long long *pos_ids, long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved, int chunks_per_cut,
-                  int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *stream) {
+                  int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace, size_t workspace_bytes,
+                  void *stream) {
     if (int rc = check_common(fn, B, H, N, Dk, Dv, dtype)) return rc;
     if (dtype != COTT_BF16 && dtype != COTT_F16)
         return fail(COTT_ERR_UNSUPPORTED, "%s: needs bf16 / fp16 tensors", fn);
@@ -665,8 +659,8 @@ int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, v
     }
     if ((long)B * H * N == 0) return COTT_OK;
     if (!cott_causal_fwd_prep_supported(B, H, N, Dk, Dv, dtype, rot_table ? rotary_dim : 0))
-        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation needs one group per head and q / k rows of at most 64 "
-                    "columns (cott_causal_fwd_prep_supported); prepare the inputs with cott_prep_ex_fwd instead", fn);
+        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation is not built for these head dims "
+                    "(cott_causal_fwd_prep_supported); prepare the inputs with cott_prep_ex_fwd instead", fn);
     if (in_bnhd || o_bnhd) {
         const long dmax = Dk > Dv ? Dk : Dv;
         if ((long)N * H * dmax > (1L << 30))
@@ -706,26 +700,27 @@ int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, v
     prep.qo = q_out;
     prep.ko = k_out;
     prep.vo = v_out;
-    return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, nullptr, 0, static_cast<hipStream_t>(stream), &prep);
+    return run_ops(fn, true, &op, 1, (long)B * H, N, dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream), &prep);
 }
 }  // namespace
 
 int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
                          const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
                          const long long *pos_ids, long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, int B,
-                         int H, int N, int Dk, int Dv, int dtype, void *stream) {
+                         int H, int N, int Dk, int Dv, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
     return fwd_prep_impl("cott_causal_fwd_prep", q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos_ids, pos0, rotary_dim,
-                         table_rows, in_bnhd, o_bnhd, nullptr, 0, 0, B, H, N, Dk, Dv, dtype, stream);
+                         table_rows, in_bnhd, o_bnhd, nullptr, 0, 0, B, H, N, Dk, Dv, dtype, workspace, workspace_bytes, stream);
 }
 
 int cott_causal_fwd_prep_save(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
                               const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,
                               const long long *pos_ids, long long pos0, int rotary_dim, int table_rows, int in_bnhd, int o_bnhd, float *saved,
-                              int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *stream) {
+                              int chunks_per_cut, int ncuts, int B, int H, int N, int Dk, int Dv, int dtype, void *workspace,
+                              size_t workspace_bytes, void *stream) {
     const char *fn = "cott_causal_fwd_prep_save";
     if ((long)B * H * N != 0 && saved == nullptr) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
     return fwd_prep_impl(fn, q, k, v, o, q_out, k_out, v_out, keep, cnt, sig, rot_table, pos_ids, pos0, rotary_dim, table_rows,
-                         in_bnhd, o_bnhd, saved, chunks_per_cut, ncuts, B, H, N, Dk, Dv, dtype, stream);
+                         in_bnhd, o_bnhd, saved, chunks_per_cut, ncuts, B, H, N, Dk, Dv, dtype, workspace, workspace_bytes, stream);
 }
 
 int cott_noncausal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype) {

@@ -113,6 +113,143 @@ __device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_
     if (r.p1 > r.p0) write_out(r.p1 - 1);
 }
 
+// Loader role with the input preparation folded in (PrepSide, cott_mfma.h): A, B, C are the RAW q, k, v projections; every
+// 16-byte piece is rotated / normalised (q, k) or scaled / masked (v) between the registers and the LDS tiles, and the
+// prepared rows also go to qo / ko / vo for the backward pass.  A row of DI columns lives in DI / 8 consecutive loader
+// lanes, which reduce its squared norm among themselves; the A and B pieces of a thread have the same row and columns
+// and share their rotary table entries.  Side inputs (keep, count, table entries) travel with the pieces, PF chunks
+// ahead; position ids one call earlier than the table entries they select.  first_half: this workgroup writes qo and
+// ko (the two column halves of a head prepare the same q and k rows).
+template <class TR, int DI, int DJ, int PF, int LT>
+__device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u16 *B_head, const u16 *C_head, u16 *O_head,
+                                                     int di, int dj, int lda, int ldb, int ldc, int ldo, const ScanRange &r,
+                                                     int tid, u16 *sA, u16 *sB, u16 *sC, const u16 *sO, const PrepSide &ps,
+                                                     int bh, int c0, bool first_half) {
+    using TL = Tiling<DI, DJ>;
+    using CT = ColTiling<DI, DJ>;
+    constexpr int NB = 8 * DI / LT, NC = 8 * DJ / LT;
+    static_assert((8 * DI) % LT == 0 && (8 * DJ) % LT == 0, "tile vectors divide over the loader threads");
+    const rsrc_t rA = make_rsrc(A_head, ((uint32_t)(r.N - 1) * lda + di) * 2u);
+    const rsrc_t rB = make_rsrc(B_head, ((uint32_t)(r.N - 1) * ldb + di) * 2u);
+    const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
+    const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldo + dj) * 2u);
+    const uint32_t qk_bytes = first_half ? (uint32_t)r.N * di * 2u : 0u;
+    const rsrc_t rQo = make_rsrc(ps.qo ? ps.qo + (size_t)bh * r.N * di : nullptr, ps.qo ? qk_bytes : 0u);
+    const rsrc_t rKo = make_rsrc(ps.ko ? ps.ko + (size_t)bh * r.N * di : nullptr, ps.ko ? qk_bytes : 0u);
+    const rsrc_t rVo = make_rsrc(ps.vo ? ps.vo + (size_t)bh * r.N * ps.dv + c0 : nullptr,
+                                 ps.vo ? ((uint32_t)(r.N - 1) * ps.dv + dj) * 2u : 0u);
+    const size_t tok0 = (size_t)(bh / ps.H) * r.N;
+    const bool scaled = ps.cnt != nullptr && ps.sig != nullptr;
+    const float sig = scaled ? ps.sig[bh % ps.H] : 0.f;
+    auto write_out = [&](int p) {
+        const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
+        const u16 *tile = sO + ((p - r.p0) & 1) * CT::SO;
+#pragma unroll
+        for (int u = 0; u < NC; ++u) {
+            const int v = tid + LT * u;
+            const int row = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+            const u32x4 val = *reinterpret_cast<const u32x4 *>(tile + row * TL::OS + col);
+            const uint32_t off = (col < dj) ? (uint32_t)((row0 + row) * ldo + col) * 2u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(val, rO, (int)off, 0, 0);
+        }
+    };
+    u32x4 ra[PF][NB], rb[PF][NB], rc[PF][NC];
+    f32x4 sn[PF][NB], cs[PF][NB];
+    float keep_ab[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
+    auto row0_of = [&](int p) {
+        const int pc = min(p, r.p1 - 1);
+        return (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
+    };
+    const bool has_pos = ps.pos != nullptr && ps.rot != nullptr;
+    const rsrc_t rPos = make_rsrc(has_pos ? ps.pos + tok0 : nullptr, has_pos ? (uint32_t)r.N * 8u : 0u);
+    u32x2 pnext[NB];
+    auto fetch_positions = [&](int p) {
+        const int row0 = row0_of(p);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int srow = min(row0 + (tid + LT * u) / (DI / 8), r.N - 1);
+            pnext[u] = __builtin_amdgcn_raw_buffer_load_b64(rPos, (int)((uint32_t)srow * 8u), 0, 0);
+        }
+    };
+    fetch_positions(r.p0);
+    auto load_chunk = [&](int s, int p) {
+        const int row0 = row0_of(p);
+        int trow[NB];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int srow = min(row0 + (tid + LT * u) / (DI / 8), r.N - 1);
+            const long long given = (long long)(((unsigned long long)pnext[u].y << 32) | pnext[u].x);
+            trow[u] = clamp_row(ps, has_pos ? given : ps.pos0 + srow);
+        }
+        fetch_positions(p + 1);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int v = tid + LT * u;
+            const int row = row0 + v / (DI / 8), col = (v % (DI / 8)) * 8;
+            ra[s][u] = buf_load16(rA, (uint32_t)(row * lda + col) * 2u);
+            rb[s][u] = buf_load16(rB, (uint32_t)(row * ldb + col) * 2u);
+            const int srow = min(row, r.N - 1);
+            keep_ab[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            if (ps.rot != nullptr && col < ps.R) {
+                const float *t = ps.rot + (size_t)trow[u] * ps.R + col / 2;
+                sn[s][u] = *reinterpret_cast<const f32x4 *>(t);
+                cs[s][u] = *reinterpret_cast<const f32x4 *>(t + ps.R / 2);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NC; ++u) {
+            const int v = tid + LT * u;
+            const int row = row0 + v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+            rc[s][u] = buf_load16(rC, (uint32_t)(row * ldc + col) * 2u);
+            const int srow = min(row, r.N - 1);
+            keep_c[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            cnt_c[s][u] = scaled ? ps.cnt[tok0 + srow] : 0.f;
+        }
+    };
+    // registers of stage s (chunk p) -> prepared tiles in the LDS buffers ta, tb, tc and in qo / ko / vo
+    auto stage = [&](int s, int p, u16 *ta, u16 *tb, u16 *tc) {
+        const int row0 = row0_of(p);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int v = tid + LT * u;
+            const int lrow = v / (DI / 8), col = (v % (DI / 8)) * 8;
+            const bool rotate = ps.rot != nullptr && col < ps.R;
+            const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
+            const u32x4 yb = prep_qk_piece<TR, DI / 8>(rb[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
+            *reinterpret_cast<u32x4 *>(ta + lrow * TL::BS + col) = ya;
+            *reinterpret_cast<u32x4 *>(tb + lrow * TL::BS + col) = yb;
+            const uint32_t off = (col < di && p < r.p1) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(ya, rQo, (int)off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(yb, rKo, (int)off, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < NC; ++u) {
+            const int v = tid + LT * u;
+            const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
+            const u32x4 y = prep_v_piece<TR>(rc[s][u], col < dj, keep_c[s][u], cnt_c[s][u], sig, scaled);
+            *reinterpret_cast<u32x4 *>(tc + lrow * TL::CS + col) = y;
+            const uint32_t off = (col < dj && p < r.p1) ? (uint32_t)((row0 + lrow) * ps.dv + col) * 2u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);
+        }
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s) load_chunk(s, r.p0 + s);
+    stage(0, r.p0, sA, sB, sC);
+    load_chunk(0, r.p0 + PF);
+    __syncthreads();
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+        const int s1 = (s + 1) % PF;
+        const int buf = (p - r.p0) & 1;
+        stage(s1, p + 1, sA + (buf ^ 1) * CT::SA, sB + (buf ^ 1) * CT::SA, sC + (buf ^ 1) * CT::SC);
+        load_chunk(s1, p + 1 + PF);
+        if (p > r.p0 + 1) write_out(p - 2);
+        chunk_barrier();
+    });
+    if (r.p1 > r.p0 + 1) write_out(r.p1 - 2);
+    __syncthreads();
+    if (r.p1 > r.p0) write_out(r.p1 - 1);
+}
+
 // Where the compute wavefront `w` of a workgroup finds and leaves its state (all pointers already at this head, and
 // group where that applies; any may be null).
 struct ColStateIO {
@@ -409,8 +546,10 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
 
 // One problem per workgroup: 4 compute wavefronts, 4 loader wavefronts.  Same grid, problem set and state slots as
 // scan_kernel.
-template <class TR, int DI, int DJ, int PF, bool STREAM>
-__global__ __launch_bounds__(512) void colscan_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G) {
+// PREP: q, k, v are the raw projections and are prepared inside the kernel (PrepSide; forward direction).
+template <class TR, int DI, int DJ, int PF, bool STREAM, bool PREP = false>
+__global__ __launch_bounds__(512) void colscan_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G,
+                                                      PrepSide prep) {
     using TL = Tiling<DI, DJ>;
     using CT = ColTiling<DI, DJ>;
     __shared__ __attribute__((aligned(16))) u16 sA[2 * CT::SA];
@@ -434,6 +573,15 @@ __global__ __launch_bounds__(512) void colscan_kernel(ProblemSet set, int BH, in
     r.mask_rev = pr.mask_rev;
     r.comp = pr.comp;
     if (wv >= 4) {
+        if constexpr (PREP) {
+            col_loader_role_prep<TR, DI, DJ, PF, 256>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
+                                                      pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh),
+                                                      pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),
+                                                      pr.O + head_base(pr.bsO, pr.hsO, pr.H, wi.bh), di, dj, pr.lda, pr.ldb,
+                                                      pr.ldc, pr.ldo, r, (int)threadIdx.x - 256, sA, sB, sC, sO, prep, wi.bh,
+                                                      pr.c0, pr.c0 == 0);
+            return;
+        }
         col_loader_role<DI, DJ, PF, 256, STREAM>(pr.A + head_base(pr.bsA, pr.hsA, pr.H, wi.bh),
                                                  pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh),
                                                  pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh),

@@ -175,11 +175,45 @@ __device__ __forceinline__ float lane_group_sum(float v) {
     return v;
 }
 
+// One raw 16-byte piece (eight columns from `col`) of a q or k row -> rotated, normalised, masked.  The row lives in
+// LANES consecutive lanes, which hold its other pieces; di: real width of the row; sn, cs: table entries of the piece's
+// four pairs (used when rotate).
+template <class TR, int LANES>
+__device__ __forceinline__ u32x4 prep_qk_piece(u32x4 raw, int col, int di, bool rotate, f32x4 sn, f32x4 cs, float keep,
+                                                float eps) {
+    float x[8];
+    unpack8<TR>(raw, x);
+    if (col >= di) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = 0.f;
+    }
+    if (rotate) rotate8(x, sn, cs);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+    ss = lane_group_sum<LANES>(ss);
+    const float nrm = __builtin_amdgcn_sqrtf(ss);
+    const float mul = keep * __builtin_amdgcn_rcpf(nrm > eps ? nrm : eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] *= mul;
+    return pack8<TR>(x);
+}
+
 // keep / max(cnt ^ sig, 1) of one position (keep alone when there is no value scaling)
 __device__ __forceinline__ float value_scale(float keep, float cnt, float sig, bool scaled) {
     if (!scaled) return keep;
     const float p = cnt > 0.f ? __expf(sig * __logf(cnt)) : 0.f;
     return p > 1.f ? keep * __builtin_amdgcn_rcpf(p) : keep;
+}
+// one raw 16-byte piece of a v row -> scaled and masked (zero past the real width)
+template <class TR>
+__device__ __forceinline__ u32x4 prep_v_piece(u32x4 raw, bool inside, float keep, float cnt, float sig, bool scaled) {
+    float x[8];
+    unpack8<TR>(raw, x);
+    const float mul = inside ? value_scale(keep, cnt, sig, scaled) : 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] *= mul;
+    return inside ? pack8<TR>(x) : u32x4{0u, 0u, 0u, 0u};
 }
 
 // Workgroup -> (head, problem, group).  Linear id i runs on XCD i % xcds.  The (head, group) units, numbered
@@ -313,9 +347,12 @@ __device__ __forceinline__ void chunk_barrier() {
 // float4 index (w*TPW + u)*64 + lane of slot (bh*G + grp)*sub + piece.  `ngroups` of the G groups are launched
 // (the causal scan never needs the last group's sum, except for ops in complement form; all_groups: the non-causal
 // form, which needs every group of every op).
-template <class TR, int DI, int DJ, int PF, bool STREAM>
-__global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg,
-                                                               int G, int ngroups, int all_groups) {
+// PREP: B and C are the raw k and v projections of a forward pass whose scan prepares its inputs itself (PrepSide): the
+// rows are rotated / normalised (B) and scaled / masked (C) on their way into the tiles, exactly as that scan does, so
+// that the sums are those of the prepared tensors.  Nothing is written back here (the scan leaves the prepared rows).
+template <class TR, int DI, int DJ, int PF, bool STREAM, bool PREP = false>
+__global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg,
+                                                               int G, int ngroups, int all_groups, PrepSide prep) {
     using TL = Tiling<DI, DJ>;
     constexpr int SB = kChunk * TL::BS, SC = kChunk * TL::CS;
     __shared__ __attribute__((aligned(16))) u16 sB[2 * SB];
@@ -350,28 +387,111 @@ __global__ __launch_bounds__(kThreads) void group_state_kernel(ProblemSet set, i
         return;
     }
 
-    u32x4 rb[PF][DI / 32], rc[PF][DJ / 32];
-    auto load_chunk = [&](int s, int p) {
+    constexpr int NB = DI / 32, NC = DJ / 32;
+    u32x4 rb[PF][NB], rc[PF][NC];
+    // PREP: the side inputs of a chunk (keep, count, rotary table entries of the rows of this thread's pieces) are
+    // fetched ONE chunk before the chunk is staged, into a single set of registers and through buffer descriptors
+    // (the tiles themselves run PF chunks ahead; with 128-wide tiles there are no registers for PF sets of side inputs),
+    // and issued before that iteration's tile loads, so that waiting for them does not wait for those.  Position ids
+    // are fetched one step earlier still, since the table entries' addresses depend on them.
+    f32x4 sn[NB], cs[NB];
+    float keep_b[NB], keep_c[NC], cnt_c[NC];
+    const size_t tok0 = PREP ? (size_t)(wi.bh / prep.H) * N : 0;
+    const bool scaled = PREP && prep.cnt != nullptr && prep.sig != nullptr;
+    const float sig = scaled ? prep.sig[wi.bh % prep.H] : 0.f;
+    const bool has_pos = PREP && prep.pos != nullptr && prep.rot != nullptr;
+    const rsrc_t rPos = make_rsrc(has_pos ? prep.pos + tok0 : nullptr, has_pos ? (uint32_t)N * 8u : 0u);
+    const rsrc_t rKeep = make_rsrc(PREP && prep.keep ? prep.keep + tok0 : nullptr, PREP && prep.keep ? (uint32_t)N : 0u);
+    const rsrc_t rCnt = make_rsrc(scaled ? prep.cnt + tok0 : nullptr, scaled ? (uint32_t)N * 4u : 0u);
+    const bool rotary = PREP && prep.rot != nullptr;
+    const rsrc_t rRot = make_rsrc(rotary ? prep.rot : nullptr, rotary ? (uint32_t)prep.table_rows * prep.R * 4u : 0u);
+    u32x2 pnext[NB];
+    auto row0_of = [&](int p) {
         const int pc = min(p, p1 - 1);
-        const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
+        return (reversed ? nchunks - 1 - pc : pc) * kChunk;
+    };
+    auto fetch_positions = [&](int p) {
+        const int row0 = row0_of(p);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int srow = min(row0 + (tid + kThreads * u) / (DI / 8), N - 1);
+            pnext[u] = __builtin_amdgcn_raw_buffer_load_b64(rPos, (int)((uint32_t)srow * 8u), 0, 0);
+        }
+    };
+    auto load_side = [&](int p) {  // side inputs of chunk p (uses the positions fetched one call earlier)
+        const int row0 = row0_of(p);
+        int trow[NB];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int srow = min(row0 + (tid + kThreads * u) / (DI / 8), N - 1);
+            const long long given = (long long)(((unsigned long long)pnext[u].y << 32) | pnext[u].x);
+            trow[u] = clamp_row(prep, has_pos ? given : prep.pos0 + srow);
+        }
+        fetch_positions(p + 1);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int v = tid + kThreads * u;
+            const int srow = min(row0 + v / (DI / 8), N - 1), col = (v % (DI / 8)) * 8;
+            keep_b[u] = prep.keep != nullptr ? (float)__builtin_amdgcn_raw_buffer_load_b8(rKeep, srow, 0, 0) : 1.f;
+            const uint32_t toff = (rotary && col < prep.R) ? (uint32_t)(trow[u] * prep.R + col / 2) * 4u : kOobOffset;
+            sn[u] = bitcast<f32x4>(__builtin_amdgcn_raw_buffer_load_b128(rRot, (int)toff, 0, 0));
+            cs[u] = bitcast<f32x4>(__builtin_amdgcn_raw_buffer_load_b128(rRot, (int)toff, prep.R * 2, 0));
+        }
+#pragma unroll
+        for (int u = 0; u < NC; ++u) {
+            const int srow = min(row0 + (tid + kThreads * u) / (DJ / 8), N - 1);
+            keep_c[u] = prep.keep != nullptr ? (float)__builtin_amdgcn_raw_buffer_load_b8(rKeep, srow, 0, 0) : 1.f;
+            cnt_c[u] = bitcast<float>(__builtin_amdgcn_raw_buffer_load_b32(rCnt, srow * 4, 0, 0));
+        }
+    };
+    auto load_chunk = [&](int s, int p) {
+        const int row0 = row0_of(p);
         load_tile<DI, kThreads, STREAM>(rb[s], rB, row0, ldb, tid);
         load_tile<DJ, kThreads, STREAM>(rc[s], rC, row0, ldc, tid);
+    };
+    // registers of stage s -> LDS tiles tb, tc
+    auto stage = [&](int s, u16 *tb, u16 *tc) {
+        if constexpr (!PREP) {
+            store_tile<DI, TL::BS>(tb, rb[s], di, tid);
+            store_tile<DJ, TL::CS>(tc, rc[s], dj, tid);
+        } else {
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const int v = tid + kThreads * u;
+                const int col = (v % (DI / 8)) * 8;
+                *reinterpret_cast<u32x4 *>(tb + (v / (DI / 8)) * TL::BS + col) = prep_qk_piece<TR, DI / 8>(
+                    rb[s][u], col, di, rotary && col < prep.R, sn[u], cs[u], keep_b[u], prep.eps);
+                __builtin_amdgcn_sched_barrier(0);  // one piece at a time: eight unpacked columns each are enough registers
+            }
+#pragma unroll
+            for (int u = 0; u < NC; ++u) {
+                const int v = tid + kThreads * u;
+                const int col = (v % (DJ / 8)) * 8;
+                *reinterpret_cast<u32x4 *>(tc + (v / (DJ / 8)) * TL::CS + col) =
+                    prep_v_piece<TR>(rc[s][u], col < dj, keep_c[u], cnt_c[u], sig, scaled);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
     };
     auto finish = [&]() {
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) slot[(w * TL::TPW + u) * 64 + l] = S[u];
     };
+    if constexpr (PREP) {
+        fetch_positions(p0);
+        load_side(p0);
+    }
 #pragma unroll
     for (int s = 0; s < PF; ++s) load_chunk(s, p0 + s);
-    store_tile<DI, TL::BS>(sB, rb[0], di, tid);
-    store_tile<DJ, TL::CS>(sC, rc[0], dj, tid);
+    stage(0, sB, sC);
+    if constexpr (PREP) load_side(p0 + 1);
     load_chunk(0, p0 + PF);
     __syncthreads();
     run_rounds<PF>(p0, p1, [&](int s, int p) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - p0) & 1;
-        store_tile<DI, TL::BS>(sB + (buf ^ 1) * SB, rb[s1], di, tid);
-        store_tile<DJ, TL::CS>(sC + (buf ^ 1) * SC, rc[s1], dj, tid);
+        stage(s1, sB + (buf ^ 1) * SB, sC + (buf ^ 1) * SC);
+        if constexpr (PREP) load_side(p + 2);
         load_chunk(s1, p + 1 + PF);
         state_update<TR, DI, DJ>(S, sB + buf * SB, sC + buf * SC, w, g, m);
         chunk_barrier();
@@ -608,25 +728,6 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
             cnt_c[s][u] = scaled ? ps.cnt[tok0 + srow] : 0.f;
         }
     };
-    // one raw 16-byte piece of a q or k row -> rotated, normalised, masked
-    auto prep_row_piece = [&](u32x4 raw, int col, f32x4 sn_, f32x4 cs_, float keep) {
-        float x[8];
-        unpack8<TR>(raw, x);
-        if (col >= di) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = 0.f;
-        }
-        if (ps.rot != nullptr && col < ps.R) rotate8(x, sn_, cs_);
-        float ss = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
-        ss = lane_group_sum<DI / 8>(ss);
-        const float nrm = __builtin_amdgcn_sqrtf(ss);
-        const float mul = keep * __builtin_amdgcn_rcpf(nrm > ps.eps ? nrm : ps.eps);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] *= mul;
-        return pack8<TR>(x);
-    };
     // registers of stage s (chunk p) -> prepared tiles in the LDS buffers ta, tb, tc and in qo / ko / vo
     auto stage = [&](int s, int p, u16 *ta, u16 *tb, u16 *tc) {
         const int row0 = row0_of(p);
@@ -634,8 +735,9 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
         for (int u = 0; u < NB; ++u) {
             const int v = tid + LT * u;
             const int lrow = v / (DI / 8), col = (v % (DI / 8)) * 8;
-            const u32x4 ya = prep_row_piece(ra[s][u], col, sn[s][u], cs[s][u], keep_ab[s][u]);
-            const u32x4 yb = prep_row_piece(rb[s][u], col, sn[s][u], cs[s][u], keep_ab[s][u]);
+            const bool rotate = ps.rot != nullptr && col < ps.R;
+            const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
+            const u32x4 yb = prep_qk_piece<TR, DI / 8>(rb[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
             *reinterpret_cast<u32x4 *>(ta + lrow * TL::BS + col) = ya;
             *reinterpret_cast<u32x4 *>(tb + lrow * TL::BS + col) = yb;
             const uint32_t off = (col < di) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
@@ -646,12 +748,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
         for (int u = 0; u < NC; ++u) {
             const int v = tid + LT * u;
             const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
-            float x[8];
-            unpack8<TR>(rc[s][u], x);
-            const float mul = (col < dj) ? value_scale(keep_c[s][u], cnt_c[s][u], sig, scaled) : 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] *= mul;
-            const u32x4 y = (col < dj) ? pack8<TR>(x) : u32x4{0u, 0u, 0u, 0u};
+            const u32x4 y = prep_v_piece<TR>(rc[s][u], col < dj, keep_c[s][u], cnt_c[s][u], sig, scaled);
             *reinterpret_cast<u32x4 *>(tc + lrow * TL::CS + col) = y;
             const uint32_t off = (col < dj) ? (uint32_t)((row0 + lrow) * ps.dv + col) * 2u : kOobOffset;
             __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);

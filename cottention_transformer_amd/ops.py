@@ -216,8 +216,8 @@ _prep_supported_cache = {}
 
 
 def fused_preparation_supported(dtype, b, h, n, dk, dv, rotary_dim=0):
-    """Whether causal_dot_product_prepared has a kernel for the shape: bf16 / fp16, Dk 32..64 and Dv 32..128 in steps
-    of 16, a rotary width that is a multiple of 8, enough heads that no head is cut into sequence groups
+    """Whether causal_dot_product_prepared has a kernel for the shape: bf16 / fp16, head dims 32..128 in steps of 16
+    (128-wide q / k rows with value tiles of at least 64 columns), a rotary width that is a multiple of 8
     (cott_causal_fwd_prep_supported)."""
     if dtype not in (torch.bfloat16, torch.float16):
         return False
@@ -276,12 +276,14 @@ def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=N
                 *((t.data_ptr() for t in prepared) if prepared else (None, None, None)),
                 _ptr(keep), _ptr(cnt), _ptr(sig), _ptr(table), _ptr(pos_ids), int(pos0), rdim, rows, int(bool(bnhd)),
                 int(bool(merged_heads)))
+        ws, ws_ptr = _workspace(_ws_bytes("cott_causal_workspace_bytes", b, h, n, dk, dv, code), q.device)
+        tail = (b, h, n, dk, dv, code, ws_ptr, ws.numel() if ws is not None else 0, _stream(q.device))
         if plan is not None:
             cpc, cuts, slot, _ = plan
             saved = torch.empty((b, h, cuts, slot), dtype=torch.float32, device=q.device)
-            rc = L.cott_causal_fwd_prep_save(*head, saved.data_ptr(), cpc, cuts, b, h, n, dk, dv, code, _stream(q.device))
+            rc = L.cott_causal_fwd_prep_save(*head, saved.data_ptr(), cpc, cuts, *tail)
         else:
-            rc = L.cott_causal_fwd_prep(*head, b, h, n, dk, dv, code, _stream(q.device))
+            rc = L.cott_causal_fwd_prep(*head, *tail)
     _check(rc, "cott_causal_fwd_prep")
     return (o, prepared, saved) if save_states else (o, prepared)
 

@@ -261,17 +261,20 @@ COTT_API int cott_prep_ex_bwd(const void *q, const void *k, const void *v,
  * rotary_dim) fp32 as in cott_prep_ex_fwd, rotary_dim a multiple of 8, or NULL; the table row of position s of batch
  * element b is pos_ids[b * N + s] (position_ids of GPT_Trainer/GPTCosAttention.py:458: int64, (B,N), any values) or,
  * with pos_ids NULL, pos0 + s; rows outside the table are clamped to it.  in_bnhd: q, k, v
- * are (B,N,H,D); o_bnhd: o is (B,N,H,Dv).  bf16 / fp16, Dk of 32..64 and Dv of 32..128 in steps of 16, B*H large
- * enough that a head is not cut into sequence groups (wider q / k rows are faster through the separate pass):
+ * are (B,N,H,D); o_bnhd: o is (B,N,H,Dv).  bf16 / fp16; head dims 32..128 in steps of 16 (with Dk above 64 the value
+ * tiles must be 64 or 128 columns wide after any split into column halves, i.e. Dv above 32 resp. 64):
  * cott_causal_fwd_prep_supported() says (1 / 0) whether a shape qualifies; otherwise the call returns
- * COTT_ERR_UNSUPPORTED and the caller prepares the inputs with cott_prep_ex_fwd.  Needs no workspace. */
+ * COTT_ERR_UNSUPPORTED and the caller prepares the inputs with cott_prep_ex_fwd.  workspace: as cott_causal_fwd for the
+ * same shape (cott_causal_workspace_bytes; sequences cut into groups, whose group sums are then formed from rows
+ * prepared the same way; NULL / 0 when that is 0). */
 COTT_API int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim);
 COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o,
                          void *q_out, void *k_out, void *v_out,
                          const unsigned char *keep, const float *cnt, const float *sig,
                          const float *rot_table, const long long *pos_ids, long long pos0, int rotary_dim, int table_rows,
                          int in_bnhd, int o_bnhd,
-                         int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
+                         int B, int H, int N, int Dk, int Dv, int dtype,
+                         void *workspace, size_t workspace_bytes, void *stream);
 /* The non-causal counterpart: o = q_hat (k_hat^T v_hat) on the raw projections in one launch, q_hat, k_hat, v_hat as
  * above without a rotation (BERT_Trainer/BertCosAttention.py:162-178 mask / normalise / scale in front of :249; there
  * cnt is the number of real tokens of the batch element at every position).  q_out, k_out, v_out receive the
@@ -294,7 +297,8 @@ COTT_API int cott_causal_fwd_prep_save(const void *q, const void *k, const void 
                               const float *rot_table, const long long *pos_ids, long long pos0, int rotary_dim,
                               int table_rows, int in_bnhd, int o_bnhd,
                               float *saved, int chunks_per_cut, int ncuts,
-                              int B, int H, int N, int Dk, int Dv, int dtype, void *stream);
+                              int B, int H, int N, int Dk, int Dv, int dtype,
+                              void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- per-kernel timing -----------------------------------------------------------------------
  * While enabled, every kernel launch made by the entry points above is bracketed by a pair of HIP

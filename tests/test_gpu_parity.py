@@ -736,6 +736,15 @@ FUSED_PREP_CASES = [
     (32, 16, 200, 48, 80, HF, 32, False, True),    # padded head dims, two workgroups per CU
     (16, 16, 63, 32, 64, BF, 0, False, False),     # no rotation, no mask, a single partial chunk
     (8, 32, 1000, 64, 64, HF, 16, True, True),     # several chunks, ragged tail
+    # 128-wide q / k rows: the kernel whose loader wavefronts stage all three tiles
+    (8, 16, 300, 128, 128, BF, 64, True, True),    # two column halves per head (value tiles of 64 columns)
+    (40, 8, 200, 128, 128, HF, 128, False, True),  # whole 128 x 128 tiles, every column rotated
+    (8, 16, 130, 96, 80, BF, 32, True, False),     # padded head dims, no mask
+    # sequences cut into groups: the group sums are formed from rows prepared the same way
+    (1, 4, 3000, 64, 64, BF, 64, True, True),      # 64-wide heads in groups
+    (2, 2, 2500, 48, 80, HF, 16, False, True),     # padded, per-head layout
+    (1, 16, 4100, 128, 128, BF, 64, True, True),   # 128-wide: column halves in groups, ragged tail
+    (1, 3, 6000, 128, 128, BF, 32, False, True),   # 128-wide: whole tiles in many groups
 ]
 
 
@@ -924,12 +933,12 @@ def test_non_causal_fused_preparation_is_refused_where_not_built(ct):
 
 def test_fused_preparation_is_refused_where_not_built(ct):
     assert not ct.fused_preparation_supported(F32, 8, 16, 256, 64, 64)
-    assert not ct.fused_preparation_supported(BF, 1, 2, 4096, 64, 64)        # few heads: sequence groups
     assert not ct.fused_preparation_supported(BF, 8, 16, 256, 64, 64, 12)    # rotary width not a multiple of 8
-    assert not ct.fused_preparation_supported(BF, 8, 16, 256, 128, 128, 64)  # wide q / k rows: the separate pass
-    assert not ct.fused_preparation_supported(BF, 16, 16, 130, 128, 128)     # undivided 128 x 128 tiles
-    q, k, v, _ = inputs(1, 2, 4096, 64, 64, BF, seed=1)
-    with pytest.raises(RuntimeError, match="one group per head"):
+    assert not ct.fused_preparation_supported(BF, 8, 16, 256, 128, 32, 64)   # 128-wide q / k rows with narrow value tiles
+    assert ct.fused_preparation_supported(BF, 1, 2, 4096, 64, 64)            # few heads: sequence groups
+    assert ct.fused_preparation_supported(BF, 8, 16, 256, 128, 128, 64)      # wide q / k rows
+    q, k, v, _ = inputs(8, 16, 64, 128, 32, BF, seed=1)
+    with pytest.raises(RuntimeError, match="not built for these head dims"):
         ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV))
     q, k, v, _ = inputs(8, 16, 64, 64, 64, F32, seed=1)
     with pytest.raises(RuntimeError, match="bf16 / fp16"):

@@ -138,18 +138,21 @@ def test_c_abi_argument_errors_without_a_gpu():
     assert L.cott_causal_fwd_bnhd(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, None, 0, None) == _loader.OK
     # preparation inside the forward kernel: 16-bit MFMA shapes, rotary width a multiple of 8, one group per head
     prep = lambda *shape_dtype, rot=None, rdim=0, rows=0: L.cott_causal_fwd_prep(
-        16, 16, 16, 16, None, None, None, None, None, None, rot, None, 0, rdim, rows, 0, 0, *shape_dtype, None)
+        16, 16, 16, 16, None, None, None, None, None, None, rot, None, 0, rdim, rows, 0, 0, *shape_dtype, None, 0, None)
     assert prep(8, 16, 256, 64, 64, _loader.F32) == _loader.ERR_UNSUPPORTED
     assert "bf16 / fp16" in _loader.last_error()
     assert prep(8, 16, 256, 256, 64, _loader.BF16) == _loader.ERR_UNSUPPORTED
     assert prep(8, 16, 256, 64, 64, _loader.BF16, rot=16, rdim=12, rows=8) == _loader.ERR_INVALID
     assert "rotary_dim" in _loader.last_error()
-    assert prep(1, 2, 4096, 64, 64, _loader.BF16) == _loader.ERR_UNSUPPORTED
-    assert "one group per head" in _loader.last_error()
+    assert prep(1, 2, 4096, 64, 64, _loader.BF16) == _loader.ERR_WORKSPACE         # sequence groups: needs the workspace
+    assert "workspace" in _loader.last_error()
     assert prep(0, 16, 256, 64, 64, _loader.BF16) == _loader.OK
-    assert prep(8, 16, 256, 128, 128, _loader.BF16) == _loader.ERR_UNSUPPORTED     # q / k rows of more than 64 columns
+    assert prep(8, 16, 256, 128, 32, _loader.BF16) == _loader.ERR_UNSUPPORTED      # 128-wide q / k rows need value tiles of 64+
     assert L.cott_causal_fwd_prep_supported(8, 16, 256, 64, 128, _loader.BF16, 64) == 1
-    assert L.cott_causal_fwd_prep_supported(8, 16, 256, 128, 128, _loader.BF16, 64) == 0
+    assert L.cott_causal_fwd_prep_supported(8, 16, 256, 128, 128, _loader.BF16, 64) == 1
+    assert L.cott_causal_fwd_prep_supported(1, 16, 65536, 128, 128, _loader.BF16, 64) == 1   # cut into sequence groups
+    assert L.cott_causal_fwd_prep_supported(1, 2, 4096, 64, 64, _loader.BF16, 0) == 1
+    assert L.cott_causal_fwd_prep_supported(8, 16, 256, 128, 32, _loader.BF16, 0) == 0
     # ... and inside the non-causal kernel: 16-bit, head dims of at most 64, a head must fit one workgroup
     ncprep = lambda *shape_dtype, cnt=None, sig=None: L.cott_noncausal_fwd_prep(
         16, 16, 16, 16, None, None, None, None, cnt, sig, 1, 1, *shape_dtype, None)
@@ -303,8 +306,8 @@ def test_plan_queries_stay_sane_over_random_shapes():
             assert cpc.value >= 1 and (cuts.value - 1) * cpc.value <= nchunks - 1
             assert slot.value >= dk * dv and wsb.value % 16 == 0
         sup = L.cott_causal_fwd_prep_supported(b, h, n, dk, dv, dt, 0)
-        if sup:
-            assert dt != _loader.F32 and dk <= 64 and L.cott_causal_workspace_bytes(b, h, n, dk, dv, dt) == 0
+        if sup:  # (any plan, also with sequence groups: the entry point takes the forward pass's workspace)
+            assert dt != _loader.F32 and dk <= 128
         sup = L.cott_noncausal_fwd_prep_supported(b, h, n, dk, dv, dt)
         if sup:
             assert dt != _loader.F32 and dk <= 64 and dv <= 64
