@@ -6,11 +6,11 @@ named like the reference's extension (`FastAttention2.kernel`, `FastAttention.fo
 `Custom_Kernel.CustomAttention`) so its callers import them unchanged.
 """
 from .ops import (causal_backward, causal_dot_product, causal_dot_product_prepared, causal_dot_product_saving, causal_prefill, decode_step, decode_step_prepared,  # noqa: F401
-                  fused_preparation_supported, merged_heads_supported,
+                  fused_preparation_supported, fused_preparation_preferred, merged_heads_supported,
                   noncausal_backward, noncausal_dot_product, noncausal_dot_product_prepared,
                   noncausal_fused_preparation_supported, prepare_inputs, prepare_inputs_backward, saved_states_plan)
 
-__all__ = ["causal_dot_product", "causal_dot_product_prepared", "causal_dot_product_saving", "saved_states_plan", "fused_preparation_supported", "PreparedCausalAttention",
+__all__ = ["causal_dot_product", "causal_dot_product_prepared", "causal_dot_product_saving", "saved_states_plan", "fused_preparation_supported", "fused_preparation_preferred", "PreparedCausalAttention",
            "causal_prefill", "causal_backward", "merged_heads_supported", "noncausal_dot_product",
            "noncausal_backward", "noncausal_dot_product_prepared", "noncausal_fused_preparation_supported",
            "PreparedNonCausalAttention", "decode_step", "decode_step_prepared",

@@ -21,6 +21,7 @@ SIGNATURES = {
     "cott_noalloc_scratch_bytes": (_sz, []),
     "cott_causal_fwd_noalloc": (_i, [_vp] * 4 + [_i] * 7 + [_vp]),
     "cott_causal_fwd_prep_supported": (_i, [_i] * 7),
+    "cott_causal_fwd_prep_preferred": (_i, [_i] * 7),
     "cott_causal_fwd_prep": (_i, [_vp] * 12 + [ctypes.c_longlong] + [_i] * 10 + [_vp, _sz, _vp]),
     "cott_causal_fwd_prep_save": (_i, [_vp] * 12 + [ctypes.c_longlong] + [_i] * 4 + [_vp] + [_i] * 8 + [_vp, _sz, _vp]),
     "cott_noncausal_fwd_prep_supported": (_i, [_i] * 6),

@@ -640,6 +640,19 @@ int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtyp
     return (pk <= 64 && pk * pv <= 128 * 64) || (pk == 128 && pv >= 64);
 }
 
+int cott_causal_fwd_prep_preferred(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim) {
+    if (!cott_causal_fwd_prep_supported(B, H, N, Dk, Dv, dtype, rotary_dim)) return 0;
+    if ((long)B * H * N == 0) return 1;
+    // The preparation is vector-ALU work of the loader wavefronts, which hides behind the other roles only for rows of
+    // up to 64 columns of heads that are one group.  Measured in a loop over one shape, rotary 32 with position ids,
+    // mask and value scaling (one launch against cott_prep_ex_fwd + cott_causal_fwd): B8 H16 N2048 D64 87 against 63 us
+    // (inside the GPT block, where the tensors come from memory, 74 against 71 us and one launch less: the block's step
+    // 741 against 770 us); D128 249 against 160 us; B4 H16 N8192 D128 757 against 348 us; B1 H16 N65536 D128 1553
+    // against 720 us (group-state pass 894 us, scan 659 us); B2 H12 N16384 D64 276 against 143 us.
+    const SetPlan p = plan_set((long)B * H, N, 1, Dk, Dv, true, dtype);
+    return cott::mfma_pad(Dk) <= 64 && p.G == 1;
+}
+
 namespace {
 int fwd_prep_impl(const char *fn, const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out,
                   void *v_out, const unsigned char *keep, const float *cnt, const float *sig, const float *rot_table,

@@ -177,7 +177,7 @@ class GPTCosAttention(nn.Module):
         cnt = cnt_all if cnt_all is not None else keep.to(torch.float32).cumsum(-1)
         dt = _autocast_target(query)
         if (bnhd and merge_heads and query.dtype == dt and (table is None or first_position is not None or pos is not None)
-                and ops.fused_preparation_supported(dt, b, h, s, query.shape[-1], value.shape[-1],
+                and ops.fused_preparation_preferred(dt, b, h, s, query.shape[-1], value.shape[-1],
                                                     0 if table is None else table.shape[-1])
                 and ops.merged_heads_supported(dt, s, h, query.shape[-1], value.shape[-1])):
             # one forward launch: rotation, normalisation, value scaling, mask and the attention op

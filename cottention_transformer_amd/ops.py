@@ -229,6 +229,20 @@ def fused_preparation_supported(dtype, b, h, n, dk, dv, rotary_dim=0):
     return ok
 
 
+def fused_preparation_preferred(dtype, b, h, n, dk, dv, rotary_dim=0):
+    """Whether the one launch of causal_dot_product_prepared is also the faster form for the shape (q / k rows of at
+    most 64 columns, heads that are not cut into sequence groups: cott_causal_fwd_prep_preferred); the modules take
+    prepare_inputs + causal_dot_product elsewhere."""
+    if dtype not in (torch.bfloat16, torch.float16):
+        return False
+    key = ("preferred", dtype, b, h, n, dk, dv, rotary_dim)
+    ok = _prep_supported_cache.get(key)
+    if ok is None:
+        ok = _remember(_prep_supported_cache, key, bool(
+            _loader.lib().cott_causal_fwd_prep_preferred(b, h, n, dk, dv, _DTYPES[dtype], rotary_dim)))
+    return ok
+
+
 def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=None, bnhd=False, merged_heads=False,
                                 want_prepared=True, save_states=False):
     """Causal forward on the RAW projections q, k, v: rotation, normalisation, value scaling and masking
