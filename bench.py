@@ -198,7 +198,7 @@ def main():
     alg_bytes = passes.get(dominant, 4) * tensor_bytes
     achieved = alg_bytes / (kern[dominant]["avg_us"] * 1e-6) / 1e9
     # the same kernels with cold caches: what a training step sees (other kernels run between forward and backward)
-    cold = cold_cache_kernel_times(torch, fwd, bwd, dev)
+    cold = cold_cache_kernel_times(torch, fwd, bwd, dev, tensor_bytes, 256)
     cold_dom = cold["bwd_kernel_us"] if dominant == "scan_grad" else cold["fwd_kernel_us"]
     cold_step_us = cold["fwd_kernel_us"] + cold["bwd_kernel_us"]
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -258,11 +258,32 @@ def cold_kernel_us(torch, fn, kernel, big):
     return 1e3 * ms / n
 
 
-def cold_cache_kernel_times(torch, fwd, bwd, dev):
+def cold_cache_kernel_times(torch, fwd, bwd, dev, tensor_bytes, workgroups):
+    """Forward and gradient launches with cold caches, and beside them a kernel of the same launch shape that only
+    streams the same tensors (cott_stream_probe: `workgroups` workgroups, each walking its contiguous share of three /
+    four tensors in 8 KiB blocks, two in flight, and writing one / three), measured the same way: the memory system's
+    part of the cold durations."""
+    from cottention_transformer_amd import _loader
     big = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
     out = {"fwd_kernel_us": cold_kernel_us(torch, fwd, "scan", big),
            "bwd_kernel_us": cold_kernel_us(torch, bwd, "scan_grad", big)}
-    del big
+    src = torch.ones(4 * tensor_bytes // 4, dtype=torch.int32, device=dev)
+    dst = torch.zeros(3 * tensor_bytes // 4, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def probe(nr, nw):
+        def fn():
+            rc = _loader.lib().cott_stream_probe(src.data_ptr(), dst.data_ptr(), tensor_bytes, nr, nw, workgroups, 8192, stream)
+            if rc != _loader.OK:
+                raise RuntimeError("cott_stream_probe refused the launch")
+        return fn
+    out["streaming_only"] = {
+        "workgroups": workgroups, "block_bytes": 8192,
+        "fwd_shape_3_reads_1_write_us": cold_kernel_us(torch, probe(3, 1), "stream_probe", big),
+        "grad_shape_4_reads_3_writes_us": cold_kernel_us(torch, probe(4, 3), "stream_probe", big)}
+    out["fwd_over_streaming_only"] = out["fwd_kernel_us"] / out["streaming_only"]["fwd_shape_3_reads_1_write_us"]
+    out["bwd_over_streaming_only"] = out["bwd_kernel_us"] / out["streaming_only"]["grad_shape_4_reads_3_writes_us"]
+    del big, src, dst
     return out
 
 

@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build", "obj")
 LIB_PATH = os.path.join(HERE, "lib", "libcottention_hip.so")
 
-SOURCES = ["cott_api.hip", "cott_mfma_bf16.hip", "cott_mfma_fp16.hip", "cott_mfma_f32.hip", "cott_generic.hip", "cott_prep.hip"]
+SOURCES = ["cott_api.hip", "cott_mfma_bf16.hip", "cott_mfma_fp16.hip", "cott_mfma_f32.hip", "cott_generic.hip", "cott_prep.hip", "cott_calib.hip"]
 
 # -packed-fp32-ops off: scalar/float2 fp32 code must not be fused into v_pk_*_f32 instructions.
 HIPCC_FLAGS = [

@@ -594,7 +594,7 @@ int cott_profile_read(int kernel_id, double *total_ms, long *launches) {
 const char *cott_kernel_name(int kernel_id) {
     static const char *names[cott::K_COUNT] = {"group_state_kernel", "state_prefix_kernel", "scan_kernel<causal>",
                                                "scan_kernel<apply>", "scan_kernel<causal> (dQ,dK,dV set)", "generic_scan_kernel",
-                                               "decode_kernel", "prep_kernel"};
+                                               "decode_kernel", "prep_kernel", "stream_probe_kernel"};
     return (kernel_id >= 0 && kernel_id < cott::K_COUNT) ? names[kernel_id] : "";
 }
 

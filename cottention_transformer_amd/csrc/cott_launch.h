@@ -66,7 +66,7 @@ struct SetArgs {
 };
 
 // Kernel families, as reported by cott_profile_read().
-enum KernelId { K_GROUP_STATE = 0, K_STATE_PREFIX, K_SCAN, K_APPLY, K_SCAN_GRAD, K_GENERIC, K_DECODE, K_PREP, K_COUNT };
+enum KernelId { K_GROUP_STATE = 0, K_STATE_PREFIX, K_SCAN, K_APPLY, K_SCAN_GRAD, K_GENERIC, K_DECODE, K_PREP, K_STREAM_PROBE, K_COUNT };
 
 // While profiling is enabled (cott_profile_enable), brackets the launches made in its lifetime
 // with a pair of HIP events on the launch stream; otherwise does nothing.

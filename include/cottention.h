@@ -310,11 +310,21 @@ COTT_API int cott_causal_fwd_prep_save(const void *q, const void *k, const void 
  * cott_profile_read() waits for the recorded launches of one kernel family, returns their summed
  * duration and count, and forgets them.  Kernel ids: 0 group_state, 1 state_prefix, 2 causal scan
  * (forward launch), 3 non-causal apply, 4 causal scan (the launch that computes dQ, dK and dV together),
- * 5 generic scan, 6 decode, 7 input preparation.  Stands where the reference wraps
+ * 5 generic scan, 6 decode, 7 input preparation, 8 the streaming probe below.  Stands where the reference wraps
  * its kernel call in torch.autograd.profiler (Cuda_Kernel/Custom_Kernel.py:165-179). */
 COTT_API int cott_profile_enable(int on);
 COTT_API int cott_profile_read(int kernel_id, double *total_ms, long *launches);
 COTT_API const char *cott_kernel_name(int kernel_id);
+
+/* ---- streaming probe (measurement aid) ---------------------------------------------------------
+ * No counterpart in the reference.  Launches a kernel with the launch shape of the scan kernels and none of their
+ * arithmetic: `workgroups` workgroups of 256 threads, each walking its own contiguous share of n_read tensors
+ * (in + t * tensor_bytes) in blocks of block_bytes (4096, 8192 or 16384) with two blocks of every tensor in flight,
+ * and writing its share of n_write tensors (out + t * tensor_bytes).  (n_read, n_write) is (3, 1), a forward pass, or
+ * (4, 3), the gradients; tensor_bytes a multiple of workgroups * block_bytes.  The benchmark times it through
+ * cott_profile_read beside the kernels to show what the memory system alone needs for a launch of that shape. */
+COTT_API int cott_stream_probe(const void *in, void *out, size_t tensor_bytes, int n_read, int n_write, int workgroups,
+                               int block_bytes, void *stream);
 
 #ifdef __cplusplus
 }
