@@ -647,8 +647,8 @@ int cott_causal_fwd_prep_preferred(int B, int H, int N, int Dk, int Dv, int dtyp
     // up to 64 columns of heads that are one group.  Measured in a loop over one shape, rotary 32 with position ids,
     // mask and value scaling (one launch against cott_prep_ex_fwd + cott_causal_fwd): B8 H16 N2048 D64 87 against 63 us
     // (inside the GPT block, where the tensors come from memory, 74 against 71 us and one launch less: the block's step
-    // 741 against 770 us); D128 249 against 160 us; B4 H16 N8192 D128 757 against 348 us; B1 H16 N65536 D128 1553
-    // against 720 us (group-state pass 894 us, scan 659 us); B2 H12 N16384 D64 276 against 143 us.
+    // 741 against 770 us); D128 248 against 160 us; B4 H16 N8192 D128 508 against 351 us; B1 H16 N65536 D128 1002
+    // against 720 us (group-state pass 352 us, scan 643 us); B2 H12 N16384 D64 274 against 140 us.
     const SetPlan p = plan_set((long)B * H, N, 1, Dk, Dv, true, dtype);
     return cott::mfma_pad(Dk) <= 64 && p.G == 1;
 }
@@ -742,9 +742,9 @@ int cott_noncausal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int d
     const long dmax = Dk > Dv ? Dk : Dv;
     if ((long)N * H * dmax > (1L << 30) || (long)B * H > (1L << 22)) return 0;
     if ((long)B * H * N == 0) return 1;
-    // one workgroup (or two column halves) per head; heads of up to 64 columns (with wider tiles the state fragments
-    // leave no registers for the preparation: B16 H16 N512 D128 176 us against 64 us for the two kernels)
-    return Dk <= 64 && Dv <= 64 && plan_set((long)B * H, N, 1, Dk, Dv, false, dtype).G == 1;
+    // one workgroup (or two column halves) per head (B16 H16 N512 D128: 56 us against 60 us for the two kernels;
+    // B32 H12 N512 D64: 40 against 47 us)
+    return plan_set((long)B * H, N, 1, Dk, Dv, false, dtype).G == 1;
 }
 
 int cott_noncausal_fwd_prep(const void *q, const void *k, const void *v, void *o, void *q_out, void *k_out, void *v_out,
@@ -757,7 +757,7 @@ int cott_noncausal_fwd_prep(const void *q, const void *k, const void *v, void *o
     if ((cnt == nullptr) != (sig == nullptr)) return fail(COTT_ERR_INVALID, "%s: cnt and sig go together", fn);
     if ((long)B * H * N == 0) return COTT_OK;
     if (!cott_noncausal_fwd_prep_supported(B, H, N, Dk, Dv, dtype))
-        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation needs head dims of at most 64 and a head that fits one "
+        return fail(COTT_ERR_UNSUPPORTED, "%s: the fused preparation needs bf16 / fp16 heads that fit one "
                     "workgroup (cott_noncausal_fwd_prep_supported); prepare the inputs with cott_prep_ex_fwd instead", fn);
     if (!q || !k || !v || !o) return fail(COTT_ERR_INVALID, "%s: null tensor pointer", fn);
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(q_out) || !aligned16(k_out) ||

@@ -71,7 +71,7 @@ __device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_
     const rsrc_t rB = make_rsrc(B_head, ((uint32_t)(r.N - 1) * ldb + di) * 2u);
     const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldo + dj) * 2u);
-    auto write_out = [&](int p) {
+    auto write_out = [&](int p) __attribute__((always_inline)) {
         const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
         const u16 *tile = sO + ((p - r.p0) & 1) * CT::SO;
 #pragma unroll
@@ -84,7 +84,7 @@ __device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_
         }
     };
     u32x4 ra[PF][8 * DI / LT], rb[PF][8 * DI / LT], rc[PF][8 * DJ / LT];
-    auto load_chunk = [&](int s, int p) {
+    auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
         const int pc = min(p, r.p1 - 1);
         const int row0 = (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
         load_tile<DI, LT, STREAM>(ra[s], rA, row0, lda, tid);
@@ -98,7 +98,7 @@ __device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_
     store_tile<DJ, TL::CS, LT>(sC, rc[0], dj, tid);
     load_chunk(0, r.p0 + PF);
     __syncthreads();
-    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) __attribute__((always_inline)) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - r.p0) & 1;
         store_tile<DI, TL::BS, LT>(sA + (buf ^ 1) * CT::SA, ra[s1], di, tid);
@@ -141,7 +141,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
     const size_t tok0 = (size_t)(bh / ps.H) * r.N;
     const bool scaled = ps.cnt != nullptr && ps.sig != nullptr;
     const float sig = scaled ? ps.sig[bh % ps.H] : 0.f;
-    auto write_out = [&](int p) {
+    auto write_out = [&](int p) __attribute__((always_inline)) {
         const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
         const u16 *tile = sO + ((p - r.p0) & 1) * CT::SO;
 #pragma unroll
@@ -156,14 +156,14 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
     u32x4 ra[PF][NB], rb[PF][NB], rc[PF][NC];
     f32x4 sn[PF][NB], cs[PF][NB];
     float keep_ab[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
-    auto row0_of = [&](int p) {
+    auto row0_of = [&](int p) __attribute__((always_inline)) {
         const int pc = min(p, r.p1 - 1);
         return (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
     };
     const bool has_pos = ps.pos != nullptr && ps.rot != nullptr;
-    const rsrc_t rPos = make_rsrc(has_pos ? ps.pos + tok0 : nullptr, has_pos ? (uint32_t)r.N * 8u : 0u);
+    const rsrc_t rPos = make_rsrc_uniform(has_pos ? ps.pos + tok0 : nullptr, has_pos ? (uint32_t)r.N * 8u : 0u);
     u32x2 pnext[NB];
-    auto fetch_positions = [&](int p) {
+    auto fetch_positions = [&](int p) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
@@ -172,7 +172,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
         }
     };
     fetch_positions(r.p0);
-    auto load_chunk = [&](int s, int p) {
+    auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
         int trow[NB];
 #pragma unroll
@@ -207,7 +207,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
         }
     };
     // registers of stage s (chunk p) -> prepared tiles in the LDS buffers ta, tb, tc and in qo / ko / vo
-    auto stage = [&](int s, int p, u16 *ta, u16 *tb, u16 *tc) {
+    auto stage = [&](int s, int p, u16 *ta, u16 *tb, u16 *tc) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
@@ -237,7 +237,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
     stage(0, r.p0, sA, sB, sC);
     load_chunk(0, r.p0 + PF);
     __syncthreads();
-    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) __attribute__((always_inline)) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - r.p0) & 1;
         stage(s1, p + 1, sA + (buf ^ 1) * CT::SA, sB + (buf ^ 1) * CT::SA, sC + (buf ^ 1) * CT::SC);
@@ -284,7 +284,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
     static_assert(NIT == 2 * KS && NIT % 4 == 0, "two row tiles per contraction step, row tiles in batches of four");
     const int g = l >> 4, m = l & 15;
     const bool mask_rev = r.mask_rev != 0, comp = r.comp != 0;
-    auto live = [&](int pb, int jt) { return FUT ? jt >= pb : jt <= pb; };
+    auto live = [&](int pb, int jt) __attribute__((always_inline)) { return FUT ? jt >= pb : jt <= pb; };
     // score tiles of this wavefront: (position block, key tile), four bits each, three per wavefront
     //   FUT:  w0 (0,0) (0,1) (0,2)   w1 (0,3) (1,1) (1,2)   w2 (1,3) (2,2) (2,3)   w3 (3,3) x 3
     //   else: w0 (0,0) (1,0) (1,1)   w1 (2,0) (2,1) (2,2)   w2 (3,0) (3,1) (3,2)   w3 (3,3) x 3
@@ -310,7 +310,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
     for (int it = 0; it < NIT; ++it)
 #pragma unroll
         for (int jw = 0; jw < NJW; ++jw) S[it][jw] = f32x4{0.f, 0.f, 0.f, 0.f};
-    auto plain_index = [&](int it, int jt, int njt) {
+    auto plain_index = [&](int it, int jt, int njt) __attribute__((always_inline)) {
         const int ks = it >> 1, t = it & 1;
         return (size_t)((2 * ks + (g >> 1)) * njt + jt) * 64 + 16 * (2 * (g & 1) + t) + m;
     };
@@ -356,7 +356,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
                 }
     }
     u32x4 sop[KS][NJW];
-    auto pack_state = [&]() {
+    auto pack_state = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -373,11 +373,11 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
     // the C fragments, and the score tiles in the LDS buffer of the chunk's parity.
     f32x4 o[4][NJW];
     u32x4 cf[NJW][2];
-    auto finish = [&](int pbuf) {  // adds (scores) x C to o and leaves the tile in the staging buffer of that chunk
+    auto finish = [&](int pbuf) __attribute__((always_inline)) {  // adds (scores) x C to o and leaves the tile in the staging buffer of that chunk
         const u32x2 *tiles = sP + pbuf * 16 * 64;
         u16 *cO = sO + pbuf * CT::SO;
         u32x4 pf[2][2];  // the score tiles of a block are read one block ahead of their products
-        auto read_block = [&](int slot, int pb) {
+        auto read_block = [&](int slot, int pb) __attribute__((always_inline)) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 const u32x2 z = {0u, 0u};
@@ -412,14 +412,14 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
         u32x2 *cP = sP + buf * 16 * 64;
         // fragment readers (each a block of LDS reads, nothing else)
         u32x4 sq[2][KS], sk[2][KS];  // query rows and key rows of a score tile, two tiles in flight
-        auto read_score = [&](int slot, int t) {
+        auto read_score = [&](int slot, int t) __attribute__((always_inline)) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 sq[slot][ks] = ld128(cA + (16 * spb[t] + m) * TL::BS + 32 * ks + 8 * g);
                 sk[slot][ks] = ld128(cB + (16 * sjt[t] + m) * TL::BS + 32 * ks + 8 * g);
             }
         };
-        auto score_tile = [&](int slot, int t) {
+        auto score_tile = [&](int slot, int t) __attribute__((always_inline)) {
             f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -436,11 +436,11 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
             cP[(spb[t] * 4 + sjt[t]) * 64 + l] = u32x2{TR::pack2(acc[0], acc[1]), TR::pack2(acc[2], acc[3])};
         };
         u32x4 qf[2][KS];
-        auto read_q = [&](int slot, int pb) {
+        auto read_q = [&](int slot, int pb) __attribute__((always_inline)) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) qf[slot][ks] = ld128(cA + (16 * pb + m) * TL::BS + 32 * ks + 8 * g);
         };
-        auto state_product = [&](int slot, int pb) {  // out^T tiles (columns 16jt + 4g .. + 3, position 16pb + m)
+        auto state_product = [&](int slot, int pb) __attribute__((always_inline)) {  // out^T tiles (columns 16jt + 4g .. + 3, position 16pb + m)
 #pragma unroll
             for (int jw = 0; jw < NJW; ++jw) {
                 f32x4 o1 = {0.f, 0.f, 0.f, 0.f}, o2 = o1;
@@ -453,7 +453,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
             }
         };
         u32x4 bf[2][4];
-        auto read_c = [&]() {
+        auto read_c = [&]() __attribute__((always_inline)) {
 #pragma unroll
             for (int jw = 0; jw < NJW; ++jw)
 #pragma unroll
@@ -461,7 +461,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
                     cf[jw][kb] = cat(lds_read_tr16(cC + (32 * kb + 4 * g + (m >> 2)) * TL::CS + 16 * (NJW * w + jw) + 4 * (m & 3)),
                                      lds_read_tr16(cC + (32 * kb + 16 + 4 * g + (m >> 2)) * TL::CS + 16 * (NJW * w + jw) + 4 * (m & 3)));
         };
-        auto read_b = [&](int slot, int kb, int it0) {  // B^T fragments of row tiles it0 .. it0 + 3, rows interleaved
+        auto read_b = [&](int slot, int kb, int it0) __attribute__((always_inline)) {  // B^T fragments of row tiles it0 .. it0 + 3, rows interleaved
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int it = it0 + e;
@@ -470,7 +470,7 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
                                   lds_read_tr16(cB + (32 * kb + 16 + 4 * g + (m >> 2)) * TL::BS + c));
             }
         };
-        auto update = [&](int slot, int kb, int it0) {  // S += B_c^T C_c (complement form: -=)
+        auto update = [&](int slot, int kb, int it0) __attribute__((always_inline)) {  // S += B_c^T C_c (complement form: -=)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const u32x4 b = bf[slot][e] ^ u32x4{flip, flip, flip, flip};

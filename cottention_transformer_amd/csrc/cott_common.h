@@ -82,6 +82,13 @@ typedef __amdgpu_buffer_rsrc_t rsrc_t;
 __device__ __forceinline__ rsrc_t make_rsrc(const void *p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
 }
+// The same for a pointer that is wavefront-uniform but was computed in vector registers (64-bit address arithmetic):
+// a descriptor left there makes every load through it a loop over the distinct values found in the lanes.
+__device__ __forceinline__ rsrc_t make_rsrc_uniform(const void *p, uint32_t bytes) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return make_rsrc(reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo), __builtin_amdgcn_readfirstlane(bytes));
+}
 // NT: non-temporal load, for data that no other workgroup reads and that is not read again before the caches have
 // turned over (long sequences): such loads do not displace other lines and stream about a third faster.  Stores
 // are never non-temporal: the 8-byte pieces of a row have to meet in L2 before the line goes to memory.

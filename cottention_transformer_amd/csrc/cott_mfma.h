@@ -400,17 +400,17 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
     const bool scaled = PREP && prep.cnt != nullptr && prep.sig != nullptr;
     const float sig = scaled ? prep.sig[wi.bh % prep.H] : 0.f;
     const bool has_pos = PREP && prep.pos != nullptr && prep.rot != nullptr;
-    const rsrc_t rPos = make_rsrc(has_pos ? prep.pos + tok0 : nullptr, has_pos ? (uint32_t)N * 8u : 0u);
+    const rsrc_t rPos = make_rsrc_uniform(has_pos ? prep.pos + tok0 : nullptr, has_pos ? (uint32_t)N * 8u : 0u);
     const rsrc_t rKeep = make_rsrc(PREP && prep.keep ? prep.keep + tok0 : nullptr, PREP && prep.keep ? (uint32_t)N : 0u);
     const rsrc_t rCnt = make_rsrc(scaled ? prep.cnt + tok0 : nullptr, scaled ? (uint32_t)N * 4u : 0u);
     const bool rotary = PREP && prep.rot != nullptr;
     const rsrc_t rRot = make_rsrc(rotary ? prep.rot : nullptr, rotary ? (uint32_t)prep.table_rows * prep.R * 4u : 0u);
     u32x2 pnext[NB];
-    auto row0_of = [&](int p) {
+    auto row0_of = [&](int p) __attribute__((always_inline)) {
         const int pc = min(p, p1 - 1);
         return (reversed ? nchunks - 1 - pc : pc) * kChunk;
     };
-    auto fetch_positions = [&](int p) {
+    auto fetch_positions = [&](int p) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
@@ -418,7 +418,7 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
             pnext[u] = __builtin_amdgcn_raw_buffer_load_b64(rPos, (int)((uint32_t)srow * 8u), 0, 0);
         }
     };
-    auto load_side = [&](int p) {  // side inputs of chunk p (uses the positions fetched one call earlier)
+    auto load_side = [&](int p) __attribute__((always_inline)) {  // side inputs of chunk p (uses the positions fetched one call earlier)
         const int row0 = row0_of(p);
         int trow[NB];
 #pragma unroll
@@ -444,13 +444,13 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
             cnt_c[u] = bitcast<float>(__builtin_amdgcn_raw_buffer_load_b32(rCnt, srow * 4, 0, 0));
         }
     };
-    auto load_chunk = [&](int s, int p) {
+    auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
         load_tile<DI, kThreads, STREAM>(rb[s], rB, row0, ldb, tid);
         load_tile<DJ, kThreads, STREAM>(rc[s], rC, row0, ldc, tid);
     };
     // registers of stage s -> LDS tiles tb, tc
-    auto stage = [&](int s, u16 *tb, u16 *tc) {
+    auto stage = [&](int s, u16 *tb, u16 *tc) __attribute__((always_inline)) {
         if constexpr (!PREP) {
             store_tile<DI, TL::BS>(tb, rb[s], di, tid);
             store_tile<DJ, TL::CS>(tc, rc[s], dj, tid);
@@ -473,7 +473,7 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
             }
         }
     };
-    auto finish = [&]() {
+    auto finish = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) slot[(w * TL::TPW + u) * 64 + l] = S[u];
     };
@@ -487,7 +487,7 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
     if constexpr (PREP) load_side(p0 + 1);
     load_chunk(0, p0 + PF);
     __syncthreads();
-    run_rounds<PF>(p0, p1, [&](int s, int p) {
+    run_rounds<PF>(p0, p1, [&](int s, int p) __attribute__((always_inline)) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - p0) & 1;
         stage(s1, sB + (buf ^ 1) * SB, sC + (buf ^ 1) * SC);
@@ -587,7 +587,7 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
     const rsrc_t rB = make_rsrc(B_head, ((uint32_t)(r.N - 1) * ldb + di) * 2u);
     const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 2u);
     // the staged tile(s) of chunk p (scan order): 16-byte row segments, rows past N dropped by the range check
-    auto write_out = [&](int p) {
+    auto write_out = [&](int p) __attribute__((always_inline)) {
         const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -605,7 +605,7 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
         }
     };
     u32x4 rb[PF][8 * DI / LT], rc[PF][8 * DJ / LT];
-    auto load_chunk = [&](int s, int p) {
+    auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
         const int pc = min(p, r.p1 - 1);
         const int row0 = (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
         load_tile<DI, LT, STREAM>(rb[s], rB, row0, ldb, tid);
@@ -617,7 +617,7 @@ __device__ __forceinline__ void loader_role(const u16 *B_head, const u16 *C_head
     store_tile<DJ, TL::CS, LT>(sC, rc[0], dj, tid);
     load_chunk(0, r.p0 + PF);
     __syncthreads();
-    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) __attribute__((always_inline)) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - r.p0) & 1;
         // stage chunk p+1 (its loads were issued PF-1 chunks ago) and refill the register stage
@@ -656,7 +656,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
     const size_t tok0 = (size_t)(bh / ps.H) * r.N;
     const bool scaled = ps.cnt != nullptr && ps.sig != nullptr;
     const float sig = scaled ? ps.sig[bh % ps.H] : 0.f;
-    auto write_out = [&](int p) {
+    auto write_out = [&](int p) __attribute__((always_inline)) {
         const int row0 = (r.reversed ? r.nchunks - 1 - p : p) * kChunk;
         const rsrc_t rO = make_rsrc(so->O[0], ((uint32_t)(r.N - 1) * so->ld[0] + so->dj[0]) * 2u);
         const u16 *tile = so->sO + (((p - r.p0) & 1) * 2) * SO;
@@ -674,7 +674,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
     u32x4 ra[PF][NB], rb[PF][NB], rc[PF][NC];
     f32x4 sn[PF][NB], cs[PF][NB];
     float keep_ab[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
-    auto row0_of = [&](int p) {
+    auto row0_of = [&](int p) __attribute__((always_inline)) {
         const int pc = min(p, r.p1 - 1);
         return (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
     };
@@ -683,9 +683,9 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
     // chunks are loaded in walking order, so the next call is the next chunk.  A descriptor of zero bytes stands in
     // when there are none: the loads return zero and the row is pos0 + s.
     const bool has_pos = ps.pos != nullptr && ps.rot != nullptr;
-    const rsrc_t rPos = make_rsrc(has_pos ? ps.pos + tok0 : nullptr, has_pos ? (uint32_t)r.N * 8u : 0u);
+    const rsrc_t rPos = make_rsrc_uniform(has_pos ? ps.pos + tok0 : nullptr, has_pos ? (uint32_t)r.N * 8u : 0u);
     u32x2 pnext[NB];
-    auto fetch_positions = [&](int p) {
+    auto fetch_positions = [&](int p) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
@@ -694,7 +694,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
         }
     };
     fetch_positions(r.p0);
-    auto load_chunk = [&](int s, int p) {
+    auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
         int trow[NB];
 #pragma unroll
@@ -729,7 +729,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
         }
     };
     // registers of stage s (chunk p) -> prepared tiles in the LDS buffers ta, tb, tc and in qo / ko / vo
-    auto stage = [&](int s, int p, u16 *ta, u16 *tb, u16 *tc) {
+    auto stage = [&](int s, int p, u16 *ta, u16 *tb, u16 *tc) __attribute__((always_inline)) {
         const int row0 = row0_of(p);
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
@@ -759,7 +759,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
     stage(0, r.p0, sA, sB, sC);
     load_chunk(0, r.p0 + PF);
     __syncthreads();
-    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) __attribute__((always_inline)) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - r.p0) & 1;
         stage(s1, p + 1, sA + (buf ^ 1) * SB, sB + (buf ^ 1) * SB, sC + (buf ^ 1) * SC);
@@ -803,7 +803,7 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
     // 16-byte load per lane) and turned through a 1 KiB piece of LDS of this wavefront's own: 64 scattered 4-byte
     // loads per lane took several microseconds per workgroup.  The piece lies in the second buffer of the B tile,
     // which nobody writes before the first barrier.
-    auto add_transposed = [&](const float *src, int src_njt) {
+    auto add_transposed = [&](const float *src, int src_njt) __attribute__((always_inline)) {
         float *scr = reinterpret_cast<float *>(const_cast<u16 *>(sB) + SB) + w * 256;
         f32x4 tile[TL::TPW];
 #pragma unroll
@@ -840,7 +840,7 @@ __device__ __forceinline__ void state_role(const float *seed, bool seed_transpos
         }
     }
     if (io.ext != nullptr) add_transposed(io.ext, io.njt);  // the state the forward pass saved is this one's transpose
-    auto put_state = [&](u16 *dst) {
+    auto put_state = [&](u16 *dst) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < TL::TPW; ++u) {
             const int t = w * TL::TPW + u;
@@ -911,16 +911,16 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     static_assert(SKIP == 0 || (SKIP <= 4 ? IB == 2 : (IB == 1 && SKIP <= 12)), "block pairing needs two blocks per wavefront");
     // block (16 positions of the chunk) number `ib` of this wavefront; whether its score tile against key tile jt
     // can hold anything (SKIP: keys >= queries are kept)
-    auto blk = [&](int ib) {
+    auto blk = [&](int ib) __attribute__((always_inline)) {
         if constexpr (SKIP >= 5) return (SKIP - 5) & 3;
         else return SKIP == 0 ? blk0 + ib : ((SKIP & 1) ? (ib == 0 ? 0 : 3) : (ib == 0 ? 1 : 2));
     };
-    auto live = [&](int ib, int jt) {
+    auto live = [&](int ib, int jt) __attribute__((always_inline)) {
         if constexpr (SKIP == 0) return true;
         else if constexpr (SKIP <= 4) return SKIP <= 2 ? jt >= blk(ib) : jt <= blk(ib);
         else return SKIP <= 8 ? jt >= SKIP - 5 : jt <= SKIP - 9;
     };
-    auto live_step = [&](int kb) {  // whether any block of this wavefront uses keys 32 kb .. 32 kb + 31
+    auto live_step = [&](int kb) __attribute__((always_inline)) {  // whether any block of this wavefront uses keys 32 kb .. 32 kb + 31
         bool any = false;
 #pragma unroll
         for (int ib = 0; ib < IB; ++ib) any = any || live(ib, 2 * kb) || live(ib, 2 * kb + 1);
@@ -931,7 +931,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     const int reversed = r.reversed;
     const bool mask_rev = r.mask_rev != 0, comp = r.comp != 0;
     u32x4 qn[PF][IB][TL::KS], qc[IB][TL::KS];
-    auto load_q = [&](int s, int p) {
+    auto load_q = [&](int s, int p) __attribute__((always_inline)) {
         if constexpr (!PREP) {
             const int pc = min(p, r.p1 - 1);
             const int row = (reversed ? r.nchunks - 1 - pc : pc) * kChunk + m;
@@ -947,7 +947,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
     __syncthreads();
     // (the large tiles keep the exit test inside the round: with 8 column tiles and 4 contraction steps per block
     // the single-exit form measured 8 % slower there, at D = 128 on long sequences)
-    run_rounds<PF, (DI * DJ > 64 * 64)>(r.p0, r.p1, [&](int s, int p) {
+    run_rounds<PF, (DI * DJ > 64 * 64)>(r.p0, r.p1, [&](int s, int p) __attribute__((always_inline)) {
         {
             const int buf = (p - r.p0) & 1;
             const u16 *cB = sB + buf * SB, *cC = sC + buf * SC, *cS = sS + buf * SSZ;
@@ -974,7 +974,7 @@ __device__ __forceinline__ void output_role(const u16 *A_head, u16 *O_head, int 
             constexpr int JB = (JBmax / TL::KS < 1) ? 1 : ((JBmax / TL::KS < TL::NJT) ? (JBmax / TL::KS) : TL::NJT);
             constexpr int NBATCH = TL::NJT / JB;
             u32x4 vf[2][JB][2], sf[2][JB][TL::KS];
-            auto read_batch = [&](int slot, int j0) {
+            auto read_batch = [&](int slot, int j0) __attribute__((always_inline)) {
 #pragma unroll
                 for (int jj = 0; jj < JB; ++jj) {
                     const int jt = j0 + jj;
@@ -1349,7 +1349,7 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
         }
     }
     u32x4 qn[PF][TL::KS];
-    auto load_q = [&](int s, int p) {
+    auto load_q = [&](int s, int p) __attribute__((always_inline)) {
         const int row = min(p, p1 - 1) * kChunk + 16 * w + m;
 #pragma unroll
         for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * lda + 32 * ks + 8 * g) * 2u);
@@ -1363,7 +1363,7 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
 #pragma unroll
         for (int ks = 0; ks < TL::KS; ++ks)
             sf[jt][ks] = *reinterpret_cast<const u32x4 *>(sS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
-    run_rounds<PF>(p0, p1, [&](int s, int p) {
+    run_rounds<PF>(p0, p1, [&](int s, int p) __attribute__((always_inline)) {
         {
             u32x4 qc[TL::KS];
 #pragma unroll
@@ -1425,7 +1425,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
 
     u32x4 qn[PF2][TL::KS];
     float keep_q[PF2];
-    auto load_q = [&](int s, int p) {
+    auto load_q = [&](int s, int p) __attribute__((always_inline)) {
         const int row = min(p, nchunks - 1) * kChunk + 16 * w + m;
 #pragma unroll
         for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * lda + 32 * ks + 8 * g) * 2u);
@@ -1439,7 +1439,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
     {
         u32x4 rb[PF][NB], rc[PF][NC];
         float keep_b[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
-        auto load_chunk = [&](int s, int p) {
+        auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
             const int row0 = min(p, nchunks - 1) * kChunk;
             load_tile<DI>(rb[s], rB, row0, ldb, tid);
             load_tile<DJ>(rc[s], rC, row0, ldc, tid);
@@ -1458,7 +1458,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
             }
         };
         // registers of stage s (chunk p) -> LDS tiles tb, tc; PREP: prepared on the way, and out to ko / vo
-        auto stage = [&](int s, int p, u16 *tb, u16 *tc) {
+        auto stage = [&](int s, int p, u16 *tb, u16 *tc) __attribute__((always_inline)) {
             if constexpr (!PREP) {
                 store_tile<DI, TL::BS>(tb, rb[s], di, tid);
                 store_tile<DJ, TL::CS>(tc, rc[s], dj, tid);
@@ -1511,7 +1511,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
         stage(0, 0, sB, sC);
         load_chunk(0, PF);
         __syncthreads();
-        run_rounds<PF>(0, nchunks, [&](int s, int p) {
+        run_rounds<PF>(0, nchunks, [&](int s, int p) __attribute__((always_inline)) {
             const int s1 = (s + 1) % PF;
             const int buf = p & 1;
             stage(s1, p + 1, sB + (buf ^ 1) * SB, sC + (buf ^ 1) * SC);
@@ -1542,7 +1542,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
             sf[jt][ks] = *reinterpret_cast<const u32x4 *>(sS + (16 * jt + m) * TL::SS + 32 * ks + 8 * g);
 
     // ---- pass 2: out_c = A_c S
-    run_rounds<PF2>(0, nchunks, [&](int s, int p) {
+    run_rounds<PF2>(0, nchunks, [&](int s, int p) __attribute__((always_inline)) {
         {
             u32x4 qc[TL::KS];
 #pragma unroll

@@ -123,18 +123,18 @@ __global__ __launch_bounds__(kThreads) void group_state_split_kernel(ProblemSetF
         return;
     }
     u32x4 rb[PF][DI / 32][2], rc[PF][DJ / 32][2];
-    auto load_chunk = [&](int s, int p) {
+    auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
         const int pc = min(p, p1 - 1);
         const int row0 = (reversed ? nchunks - 1 - pc : pc) * kChunk;
         load_tile_f<DI, kThreads, false>(rb[s], rB, row0, ldb, tid);
         load_tile_f<DJ, kThreads, false>(rc[s], rC, row0, ldc, tid);
     };
-    auto stage = [&](int s, int buf) {
+    auto stage = [&](int s, int buf) __attribute__((always_inline)) {
         store_tile_split<DI, TL::BS, kThreads>(sBh + buf * SB, sBl + buf * SB, rb[s], di, tid);
         store_tile_split<DJ, TL::CS, kThreads>(sCh + buf * SC, sCl + buf * SC, rc[s], dj, tid);
     };
     // S[i][j] += sum over the 64 positions of B[tok][i] C[tok][j] for the tiles this wavefront owns (see state_update)
-    auto update = [&](int buf) {
+    auto update = [&](int buf) __attribute__((always_inline)) {
         constexpr int ROWS = (TL::TPW + TL::NJT - 1) / TL::NJT;
         constexpr int COLS = TL::TPW < TL::NJT ? TL::TPW : TL::NJT;
         const u16 *bh = sBh + buf * SB, *bl = sBl + buf * SB, *ch = sCh + buf * SC, *cl = sCl + buf * SC;
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kThreads) void group_state_split_kernel(ProblemSetF
     stage(0, 0);
     load_chunk(0, p0 + PF);
     __syncthreads();
-    run_rounds<PF>(p0, p1, [&](int s, int p) {
+    run_rounds<PF>(p0, p1, [&](int s, int p) __attribute__((always_inline)) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - p0) & 1;
         stage(s1, buf ^ 1);
@@ -189,7 +189,7 @@ __device__ __forceinline__ void split_loader_role(const float *A_head, const flo
     const rsrc_t rB = make_rsrc(B_head, ((uint32_t)(r.N - 1) * ldb + di) * 4u);
     const rsrc_t rC = make_rsrc(C_head, ((uint32_t)(r.N - 1) * ldc + dj) * 4u);
     u32x4 ra[PF][8 * DI / LT][2], rb[PF][8 * DI / LT][2], rc[PF][8 * DJ / LT][2];
-    auto load_chunk = [&](int s, int p) {
+    auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
         const int pc = min(p, r.p1 - 1);
         const int row0 = (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
         load_tile_f<DI, LT, false>(ra[s], rA, row0, lda, tid);
@@ -197,7 +197,7 @@ __device__ __forceinline__ void split_loader_role(const float *A_head, const flo
         load_tile_f<DJ, LT, false>(rc[s], rC, row0, ldc, tid);
     };
     // LDS: [hi | lo] x [2 buffers] per operand
-    auto stage = [&](int s, int buf) {
+    auto stage = [&](int s, int buf) __attribute__((always_inline)) {
         store_tile_split<DI, TL::BS, LT>(sA + buf * CT::SA, sA + (2 + buf) * CT::SA, ra[s], di, tid);
         store_tile_split<DI, TL::BS, LT>(sB + buf * CT::SA, sB + (2 + buf) * CT::SA, rb[s], di, tid);
         store_tile_split<DJ, TL::CS, LT>(sC + buf * CT::SC, sC + (2 + buf) * CT::SC, rc[s], dj, tid);
@@ -207,7 +207,7 @@ __device__ __forceinline__ void split_loader_role(const float *A_head, const flo
     stage(0, 0);
     load_chunk(0, r.p0 + PF);
     __syncthreads();
-    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) {
+    run_rounds<PF>(r.p0, r.p1, [&](int s, int p) __attribute__((always_inline)) {
         const int s1 = (s + 1) % PF;
         const int buf = (p - r.p0) & 1;
         stage(s1, buf ^ 1);
@@ -228,7 +228,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
     static_assert(NIT == 2 * KS && NIT % 4 == 0, "two row tiles per contraction step, row tiles in batches of four");
     const int g = l >> 4, m = l & 15;
     const bool mask_rev = r.mask_rev != 0;
-    auto live = [&](int pb, int jt) { return FUT ? jt >= pb : jt <= pb; };
+    auto live = [&](int pb, int jt) __attribute__((always_inline)) { return FUT ? jt >= pb : jt <= pb; };
     const rsrc_t rO = make_rsrc(O_head, ((uint32_t)(r.N - 1) * ldo + dj) * 4u);
     int spb[3], sjt[3];  // the three score tiles of this wavefront (see col_compute_role)
     {
@@ -274,7 +274,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
                 }
     }
     u32x4 soph[KS][NJW], sopl[KS][NJW];
-    auto pack_state = [&]() {
+    auto pack_state = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -295,7 +295,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
     f32x4 o[4][NJW];
     u32x4 cfh[NJW][2], cfl[NJW][2], pfh[4][2], pfl[4][2];
     int pbuf = 0;  // score buffer written in the current chunk
-    auto read_scores_of_previous = [&]() {
+    auto read_scores_of_previous = [&]() __attribute__((always_inline)) {
         const int base = (pbuf ^ 1) * 16 * 64;
 #pragma unroll
         for (int pb = 0; pb < 4; ++pb)
@@ -309,7 +309,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
                 }
             }
     };
-    auto finish_previous = [&](int pprev) {
+    auto finish_previous = [&](int pprev) __attribute__((always_inline)) {
         const int row0 = (r.reversed ? r.nchunks - 1 - pprev : pprev) * kChunk;
         f32x4 acc2[4][NJW];
 #pragma unroll
@@ -345,7 +345,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
         const u16 *cBh = sB + buf * CT::SA, *cBl = sB + (2 + buf) * CT::SA;
         const u16 *cCh = sC + buf * CT::SC, *cCl = sC + (2 + buf) * CT::SC;
         u32x4 sqh[2][KS], sql[2][KS], skh[2][KS], skl[2][KS];
-        auto read_score = [&](int slot, int t) {
+        auto read_score = [&](int slot, int t) __attribute__((always_inline)) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const int qa = (16 * spb[t] + m) * TL::BS + 32 * ks + 8 * g, ka = (16 * sjt[t] + m) * TL::BS + 32 * ks + 8 * g;
@@ -355,7 +355,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
                 skl[slot][ks] = ld128(cBl + ka);
             }
         };
-        auto score_tile = [&](int slot, int t) {
+        auto score_tile = [&](int slot, int t) __attribute__((always_inline)) {
             f32x4 acc[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) acc[ks] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -378,14 +378,14 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
             sPl[pbuf * 16 * 64 + (spb[t] * 4 + sjt[t]) * 64 + l] = lo;
         };
         u32x4 qfh[2][KS], qfl[2][KS];
-        auto read_q = [&](int slot, int pb) {
+        auto read_q = [&](int slot, int pb) __attribute__((always_inline)) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 qfh[slot][ks] = ld128(cAh + (16 * pb + m) * TL::BS + 32 * ks + 8 * g);
                 qfl[slot][ks] = ld128(cAl + (16 * pb + m) * TL::BS + 32 * ks + 8 * g);
             }
         };
-        auto state_product = [&](int slot, int pb) {
+        auto state_product = [&](int slot, int pb) __attribute__((always_inline)) {
 #pragma unroll
             for (int jw = 0; jw < NJW; ++jw) {
                 f32x4 acc[KS];
@@ -402,7 +402,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
             }
         };
         u32x4 bfh[2][4], bfl[2][4];
-        auto read_c = [&]() {
+        auto read_c = [&]() __attribute__((always_inline)) {
 #pragma unroll
             for (int jw = 0; jw < NJW; ++jw)
 #pragma unroll
@@ -412,7 +412,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
                     cfl[jw][kb] = cat(lds_read_tr16(cCl + a0), lds_read_tr16(cCl + a1));
                 }
         };
-        auto read_b = [&](int slot, int kb, int it0) {
+        auto read_b = [&](int slot, int kb, int it0) __attribute__((always_inline)) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int it = it0 + e;
@@ -421,7 +421,7 @@ __device__ __forceinline__ void split_compute_role(const ColStateIO &io, float *
                 bfl[slot][e] = cat(lds_read_tr16(cBl + a0), lds_read_tr16(cBl + a1));
             }
         };
-        auto update = [&](int slot, int kb, int it0) {
+        auto update = [&](int slot, int kb, int it0) __attribute__((always_inline)) {
 #pragma unroll
             for (int t = 0; t < 3; ++t)
 #pragma unroll

@@ -303,7 +303,7 @@ def causal_dot_product_prepared(q, k, v, keep=None, cnt=None, sig=None, rotary=N
 
 
 def noncausal_fused_preparation_supported(dtype, b, h, n, dk, dv):
-    """Whether noncausal_dot_product_prepared has a kernel for the shape: bf16 / fp16, head dims 32..64 in steps of
+    """Whether noncausal_dot_product_prepared has a kernel for the shape: bf16 / fp16, head dims 32..128 in steps of
     16, enough heads that a head is handled by one workgroup (cott_noncausal_fwd_prep_supported)."""
     if dtype not in (torch.bfloat16, torch.float16):
         return False

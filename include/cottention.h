@@ -283,7 +283,7 @@ COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, v
  * above without a rotation (BERT_Trainer/BertCosAttention.py:162-178 mask / normalise / scale in front of :249; there
  * cnt is the number of real tokens of the batch element at every position).  q_out, k_out, v_out receive the
  * prepared tensors for the backward pass (cott_noncausal_bwd on them, then cott_prep_ex_bwd).  bf16 / fp16, head
- * dims 32..64 in steps of 16, and a head must fit one workgroup (no sequence groups: B*H at least about the number
+ * dims 32..128 in steps of 16, and a head must fit one workgroup (no sequence groups: B*H at least about the number
  * of CUs): cott_noncausal_fwd_prep_supported() says whether a shape qualifies; otherwise COTT_ERR_UNSUPPORTED.
  * Needs no workspace. */
 COTT_API int cott_noncausal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype);

@@ -869,6 +869,9 @@ NC_FUSED_PREP_CASES = [
     (16, 16, 130, 64, 32, BF, True, True),     # one workgroup per head, narrower values
     (64, 8, 63, 32, 64, BF, False, False),     # no mask, a single partial chunk, per-head layout
     (48, 8, 200, 48, 48, HF, False, True),     # padded head dims
+    (16, 16, 300, 128, 128, BF, True, True),   # 128-wide heads
+    (20, 16, 200, 128, 64, HF, False, True),   # wide q / k rows, narrower values
+    (24, 12, 130, 80, 112, BF, True, False),   # padded to 128 on both sides
 ]
 
 
@@ -926,7 +929,7 @@ def test_non_causal_fused_preparation_is_refused_where_not_built(ct):
     assert not ct.noncausal_fused_preparation_supported(F32, 32, 12, 512, 64, 64)
     assert not ct.noncausal_fused_preparation_supported(BF, 1, 2, 4096, 64, 64)      # few heads: sequence groups
     q = torch.randn(1, 2, 4096, 64, device=DEV, dtype=BF)
-    assert not ct.noncausal_fused_preparation_supported(BF, 16, 16, 512, 128, 128)   # wide heads: the two kernels
+    assert ct.noncausal_fused_preparation_supported(BF, 16, 16, 512, 128, 128)       # wide heads
     with pytest.raises(RuntimeError, match="one workgroup"):
         ct.noncausal_dot_product_prepared(q, q, q)
 

@@ -158,7 +158,7 @@ def test_c_abi_argument_errors_without_a_gpu():
     assert L.cott_causal_fwd_prep_preferred(8, 16, 256, 128, 128, _loader.BF16, 64) == 0
     assert L.cott_causal_fwd_prep_preferred(1, 16, 65536, 64, 64, _loader.BF16, 64) == 0       # sequence groups
     assert L.cott_causal_fwd_prep_preferred(8, 16, 2048, 64, 64, _loader.F32, 0) == 0
-    # ... and inside the non-causal kernel: 16-bit, head dims of at most 64, a head must fit one workgroup
+    # ... and inside the non-causal kernel: 16-bit, a head must fit one workgroup
     ncprep = lambda *shape_dtype, cnt=None, sig=None: L.cott_noncausal_fwd_prep(
         16, 16, 16, 16, None, None, None, None, cnt, sig, 1, 1, *shape_dtype, None)
     assert ncprep(32, 12, 512, 64, 64, _loader.F32) == _loader.ERR_UNSUPPORTED
@@ -167,9 +167,9 @@ def test_c_abi_argument_errors_without_a_gpu():
     assert "cnt and sig" in _loader.last_error()
     assert ncprep(1, 2, 4096, 64, 64, _loader.BF16) == _loader.ERR_UNSUPPORTED
     assert "one workgroup" in _loader.last_error()
-    assert ncprep(16, 16, 512, 128, 128, _loader.BF16) == _loader.ERR_UNSUPPORTED
     assert ncprep(0, 12, 512, 64, 64, _loader.BF16) == _loader.OK
     assert L.cott_noncausal_fwd_prep_supported(32, 12, 512, 64, 64, _loader.BF16) == 1
+    assert L.cott_noncausal_fwd_prep_supported(16, 16, 512, 128, 128, _loader.BF16) == 1
     assert L.cott_noncausal_fwd_prep_supported(32, 12, 512, 64, 64, _loader.F32) == 0
     assert L.cott_noncausal_fwd_prep_supported(1, 2, 4096, 64, 64, _loader.BF16) == 0
 
@@ -315,5 +315,5 @@ def test_plan_queries_stay_sane_over_random_shapes():
             assert dt != _loader.F32 and dk <= 128
         sup = L.cott_noncausal_fwd_prep_supported(b, h, n, dk, dv, dt)
         if sup:
-            assert dt != _loader.F32 and dk <= 64 and dv <= 64
+            assert dt != _loader.F32 and dk <= 128 and dv <= 128
             assert L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, dt) == 0
