@@ -52,6 +52,8 @@ SIGNATURES = {
     "cott_profile_read": (_i, [_i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_long)]),
     "cott_kernel_name": (ctypes.c_char_p, [_i]),
     "cott_stream_probe": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp]),
+    "cott_plan_geometry": (_i, [_i, _i]),
+    "cott_plan_describe": (_i, [_i] * 8 + [ctypes.POINTER(_i), ctypes.POINTER(_i)]),
 }
 
 KERNEL_IDS = {"group_state": 0, "state_prefix": 1, "scan": 2, "apply": 3, "scan_grad": 4, "generic": 5, "decode": 6,

@@ -6,6 +6,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -45,7 +46,7 @@ ProfScope::~ProfScope() {
 // Scratch memory of cott_causal_fwd_noalloc: the group-state slots that the other entry points take from the
 // caller's workspace.  Every device the library runs on holds its own copy of this array until the process ends.
 // In host code the name is only a handle for hipGetSymbolAddress; kernels receive the address it returns.
-#define COTT_SCRATCH_BYTES (32u << 20)
+#define COTT_SCRATCH_BYTES (48u << 20)
 static __device__ __align__(256) unsigned char scratch[COTT_SCRATCH_BYTES];
 
 namespace {
@@ -87,7 +88,10 @@ int exp_int(const char *name, int dflt) {
 // throughput to these LDS-heavy kernels, so grids just above the CU count run almost twice as long).
 // CUs of the current device, asked once per process (256 on an unpartitioned MI355X; the fallback when the query
 // fails).  A partitioned device reports fewer and gets correspondingly smaller launch plans.
+std::atomic<int> g_cus_given{0}, g_xcds_given{0};  // cott_plan_geometry: > 0 replaces the device's answer
+
 int device_cus() {
+    if (const int given = g_cus_given.load(std::memory_order_relaxed)) return given;
     static const int v = [] {
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess) return 256;
@@ -97,6 +101,7 @@ int device_cus() {
     return v;
 }
 int device_xcds() {
+    if (const int given = g_xcds_given.load(std::memory_order_relaxed)) return given;
     static const int v = [] {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) != hipSuccess) return 8;
@@ -106,8 +111,8 @@ int device_xcds() {
     return v;
 }
 int target_workgroups() {
-    static const int v = [] { const int x = exp_int("COTT_TARGET_WGS", 0); return x > 0 ? x : device_cus(); }();
-    return v;
+    static const int given = exp_int("COTT_TARGET_WGS", 0);
+    return given > 0 ? given : device_cus();
 }
 // -1 auto, 0 never, 1 always split the output columns of each op in two.
 int split_policy() {
@@ -951,6 +956,60 @@ int cott_causal_saved_plan(int B, int H, int N, int Dk, int Dv, int dtype, int *
         return fail(COTT_ERR_INVALID, "%s: bad shape or dtype", fn);
     if (saved_states_plan((long)B * H, N, Dk, Dv, dtype, chunks_per_cut, ncuts, bwd_workspace_bytes))
         *slot_floats = cott::mfma_pad(Dk) * cott::mfma_pad(Dv);
+    return COTT_OK;
+}
+
+int cott_plan_geometry(int cus, int xcds) {
+    if (cus < 0 || xcds < 0 || (cus > 0 && xcds > 0 && cus % xcds != 0))
+        return fail(COTT_ERR_INVALID, "cott_plan_geometry: %d CUs in %d XCDs", cus, xcds);
+    g_cus_given.store(cus, std::memory_order_relaxed);
+    g_xcds_given.store(xcds, std::memory_order_relaxed);
+    return COTT_OK;
+}
+
+int cott_plan_describe(int which, int with_saved_states, int B, int H, int N, int Dk, int Dv, int dtype, int *sets,
+                       int *nsets) {
+    const char *fn = "cott_plan_describe";
+    if (!sets || !nsets || which < 0 || which > 3) return fail(COTT_ERR_INVALID, "%s: bad argument", fn);
+    *nsets = 0;
+    if (elem_size(dtype) == 0 || B < 0 || H < 0 || N < 0 || Dk < 1 || Dv < 1)
+        return fail(COTT_ERR_INVALID, "%s: bad shape or dtype", fn);
+    const bool causal = which < 2, grads = (which & 1) != 0;
+    if ((long)B * H * N == 0 || !use_mfma(dtype, Dk, Dv, N) || (grads && !use_mfma(dtype, Dv, Dk, N))) return COTT_OK;
+    Op ops[3];
+    int n = 1;
+    char tag[8];  // distinct stand-in addresses, never dereferenced: the layout only compares operands
+    if (grads) {
+        grad_ops(ops, tag + 0, tag + 1, tag + 2, tag + 3, tag + 4, tag + 5, tag + 6, Dk, Dv, causal);
+        n = 3;
+        if (with_saved_states && causal) {
+            int cpc = 0, cuts = 0;
+            if (saved_states_plan((long)B * H, N, Dk, Dv, dtype, &cpc, &cuts, nullptr)) {
+                ops[0].ext = tag + 7;
+                ops[0].save_cpg = cpc;
+                ops[0].save_n = cuts;
+            }
+        }
+    } else {
+        ops[0] = Op{tag + 0, tag + 1, tag + 2, tag + 3, Dk, Dv, 0};
+    }
+    int members[8][8], counts[8];
+    const int ns = form_sets(ops, n, (long)B * H, N, dtype, causal, members, counts);
+    for (int s = 0; s < ns; ++s) {
+        const SetLayout L = layout_set(ops, n, members[s], counts[s], (long)B * H, N, dtype, causal);
+        int *o = sets + 8 * s;
+        const int per_unit = L.pair ? 2 : counts[s] * L.p.halves;
+        o[0] = counts[s];
+        o[1] = L.p.halves;
+        o[2] = L.p.G;
+        o[3] = L.p.cpg;
+        o[4] = L.p.sub;
+        o[5] = L.pair ? 1 : 0;
+        o[6] = L.complement ? 1 : 0;
+        const long x = device_xcds();  // (head, group) units rounded up to whole rounds of the XCDs, as the launchers do
+        o[7] = (int)((((long)B * H * L.p.G + x - 1) / x) * x * per_unit);
+    }
+    *nsets = ns;
     return COTT_OK;
 }
 

@@ -68,7 +68,8 @@ COTT_API int cott_causal_fwd_may_alias_v(int B, int H, int N, int Dk, int Dv, in
  * instead of caller memory.  It has no counterpart in the reference; it is for callers that cannot allocate
  * device memory around the call: code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  Same arguments, results (bit for bit) and errors as cott_causal_fwd; a shape whose slots exceed
- * cott_noalloc_scratch_bytes() (32 MiB, enough for every plan this build makes) returns COTT_ERR_WORKSPACE.
+ * cott_noalloc_scratch_bytes() (48 MiB, enough for every plan this build makes on a part of up to 256 CUs)
+ * returns COTT_ERR_WORKSPACE.
  * The array's address is looked up once per device (hipGetSymbolAddress): by cott_noalloc_scratch_bytes() when a
  * device is current, else by the first call of the entry point on that device.  Call cott_noalloc_scratch_bytes()
  * before a stream capture starts, so that the lookup does not happen inside it.  No call allocates or frees.
@@ -315,6 +316,20 @@ COTT_API int cott_causal_fwd_prep_save(const void *q, const void *k, const void 
 COTT_API int cott_profile_enable(int on);
 COTT_API int cott_profile_read(int kernel_id, double *total_ms, long *launches);
 COTT_API const char *cott_kernel_name(int kernel_id);
+
+/* ---- launch plans (pure host functions, for tests and tools) -----------------------------------
+ * No counterpart in the reference.  The launch plans depend on the device's CU and XCD counts (asked once per process;
+ * 256 / 8 when no device answers).  cott_plan_geometry(cus, xcds) replaces them for every later call of this process
+ * (0, 0: back to the device's), so that the plans of another part can be examined on any host; cus must be a multiple of xcds.
+ * cott_plan_describe: the launches behind `which` = 0 causal forward, 1 causal gradients (with_saved_states: as
+ * cott_causal_bwd_saved runs them where cott_causal_saved_plan has a plan), 2 non-causal forward, 3 non-causal
+ * gradients, for a shape: *nsets launches (at most 8; 0 when the shape takes the plain-FMA path) and per launch eight
+ * ints in sets[8 * s ..]: ops, column halves, sequence groups G, chunks per group, pieces of the group-state pass,
+ * whether dK and dV share pair workgroups, whether ops that sum over the past run in complement form, and the
+ * workgroups of the scan's grid. */
+COTT_API int cott_plan_geometry(int cus, int xcds);
+COTT_API int cott_plan_describe(int which, int with_saved_states, int B, int H, int N, int Dk, int Dv, int dtype,
+                                int *sets, int *nsets);
 
 /* ---- streaming probe (measurement aid) ---------------------------------------------------------
  * No counterpart in the reference.  Launches a kernel with the launch shape of the scan kernels and none of their

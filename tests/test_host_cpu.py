@@ -181,13 +181,15 @@ def test_no_alloc_entry_point_checks_and_its_scratch_symbol(tmp_path):
     import subprocess
     from cottention_transformer_amd import _loader
     L = _loader.lib()
-    assert L.cott_noalloc_scratch_bytes() == 32 << 20
+    assert L.cott_noalloc_scratch_bytes() == 48 << 20
     assert L.cott_causal_fwd_noalloc(16, 16, 16, 16, 1, 1, 8, 24, 32, _loader.F32, 0, None) == _loader.ERR_INVALID
     assert "divisible by 16" in _loader.last_error()
     assert L.cott_causal_fwd_noalloc(None, 16, 16, 16, 1, 1, 8, 64, 64, _loader.F32, 0, None) == _loader.ERR_INVALID
     assert L.cott_causal_fwd_noalloc(None, None, None, None, 0, 4, 128, 64, 64, _loader.BF16, 0, None) == _loader.OK
-    # every plan of the forward pass fits the built-in scratch (at most one 64 KiB slot per workgroup of a full chip)
-    for shape in ((1, 16, 65536, 128, 128), (1, 1, 1 << 20, 128, 128), (3, 5, 30000, 64, 128)):
+    # every plan of the forward pass fits the built-in scratch: at most two group-state workgroups per CU with a
+    # 64 KiB slot each, plus the slots of the last group, which no workgroup fills (G / (G - 1) <= 3 / 2 with pieces)
+    # (test_launch_plans_over_device_geometries sweeps random shapes)
+    for shape in ((1, 16, 65536, 128, 128), (1, 1, 1 << 20, 128, 128), (3, 5, 30000, 64, 128), (5, 16, 16384, 128, 128)):
         for dt in (_loader.BF16, _loader.F32):
             assert L.cott_causal_workspace_bytes(*shape, dt) <= L.cott_noalloc_scratch_bytes()
     objdump, readelf = "/opt/rocm/llvm/bin/llvm-objdump", "/opt/rocm/llvm/bin/llvm-readelf"
@@ -201,7 +203,7 @@ def test_no_alloc_entry_point_checks_and_its_scratch_symbol(tmp_path):
             out = subprocess.run([readelf, "-s", "--wide", str(tmp_path / f)], check=True, capture_output=True, text=True).stdout
             rows += [l for l in out.splitlines() if l.split()[-1:] == ["_ZL7scratch"]]
     assert rows, "scratch array not found in the device code objects"
-    assert all("GLOBAL" in l and str(32 << 20) in l for l in rows), rows
+    assert all("GLOBAL" in l and str(48 << 20) in l for l in rows), rows
 
 
 def test_saved_states_plan_and_argument_checks():
@@ -317,3 +319,73 @@ def test_plan_queries_stay_sane_over_random_shapes():
         if sup:
             assert dt != _loader.F32 and dk <= 128 and dv <= 128
             assert L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, dt) == 0
+
+
+@pytest.mark.parametrize("cus,xcds", [(256, 8), (304, 8), (128, 4), (64, 2), (32, 1), (80, 8)])
+def test_launch_plans_over_device_geometries(cus, xcds):
+    """The launch planner's rules were measured on one part (256 CUs in 8 XCDs) but follow the CU and XCD counts of the
+    device.  With those counts given (cott_plan_geometry), over seeded random shapes: every grid is a whole number of
+    XCD rounds and stays within a few workgroups per CU unless the heads alone exceed that; groups cover the sequence;
+    the cuts cott_causal_saved_plan names are the groups the gradient launch that takes the states is cut into; the
+    workspace sizes follow from the plan (one padded state per head, group, piece and op with sums of its own at most);
+    and on parts of up to 256 CUs every forward plan fits the built-in array of cott_causal_fwd_noalloc."""
+    import ctypes
+    import random
+    from cottention_transformer_amd import _loader
+    L = _loader.lib()
+    assert L.cott_plan_geometry(7, 2) == _loader.ERR_INVALID
+    assert L.cott_plan_geometry(cus, xcds) == _loader.OK
+    try:
+        rnd = random.Random(cus * 31 + xcds)
+        sets, nsets = (ctypes.c_int * 64)(), ctypes.c_int(0)
+        pad = lambda d: 32 if d <= 32 else (64 if d <= 64 else 128)
+        seen_groups = seen_pair = seen_comp = 0
+        for _ in range(300):
+            b = rnd.choice([1, 2, 3, 5, 8, 32, 100]); h = rnd.choice([1, 2, 8, 12, 16])
+            n = rnd.choice([1, 63, 64, 65, 512, 2048, 4097, 16384, 65536])
+            dk = rnd.choice([32, 48, 64, 96, 128]); dv = rnd.choice([32, 64, 80, 128])
+            dt = rnd.choice([_loader.BF16, _loader.F16, _loader.F32])
+            bh, nchunks = b * h, (n + 63) // 64
+            cpc, cuts, slot, wsb = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
+            assert L.cott_causal_saved_plan(b, h, n, dk, dv, dt, ctypes.byref(cpc), ctypes.byref(cuts),
+                                            ctypes.byref(slot), ctypes.byref(wsb)) == _loader.OK
+            for which, saved in ((0, 0), (1, 0), (1, 1), (2, 0), (3, 0)):
+                assert L.cott_plan_describe(which, saved, b, h, n, dk, dv, dt, sets, ctypes.byref(nsets)) == _loader.OK
+                assert 1 <= nsets.value <= 3, (which, b, h, n, dk, dv, dt)
+                ops_total, slots = 0, 0
+                for s in range(nsets.value):
+                    cnt, halves, G, cpg, sub, pair, comp, grid = sets[8 * s: 8 * s + 8]
+                    case = (cus, xcds, which, saved, b, h, n, dk, dv, dt, s, tuple(sets[8 * s: 8 * s + 8]))
+                    ops_total += cnt
+                    assert halves in (1, 2) and 1 <= G <= nchunks and 1 <= sub <= 4, case
+                    assert (G - 1) * cpg < nchunks <= G * cpg, case           # the groups cover the sequence, none is empty
+                    per_unit = 2 if pair else cnt * halves
+                    assert grid % (xcds * per_unit) == 0 and grid >= bh * G * per_unit, case
+                    assert grid < (bh * G + xcds) * per_unit, case             # less than one XCD round of padding
+                    # cutting into groups never pushes a launch past two workgroups per CU (the fp32 matrix-pipe
+                    # kernels aim at two per CU); what exceeds that is heads times ops alone
+                    if G > 1:
+                        assert bh * per_unit * G <= 2 * cus, case
+                        seen_groups += 1
+                    seen_pair += pair
+                    seen_comp += comp
+                    slots += cnt * halves * bh * G * sub
+                    if which == 1 and saved and cuts.value > 0 and (pair or comp):
+                        assert (G, cpg) == (cuts.value, cpc.value), case     # the forward pass cuts where this launch does
+                assert ops_total == (3 if which in (1, 3) else 1)
+                if which == 2:
+                    nc_slots = slots
+                    continue
+                if which == 3:  # one query serves the non-causal forward and gradients: the larger of the two
+                    ws, slots = L.cott_noncausal_workspace_bytes(b, h, n, dk, dv, dt), max(slots, nc_slots)
+                elif which == 1:
+                    ws = wsb.value if (saved and cuts.value > 0) else L.cott_causal_bwd_workspace_bytes(b, h, n, dk, dv, dt)
+                else:
+                    ws = L.cott_causal_workspace_bytes(b, h, n, dk, dv, dt)
+                # (a column half's slot is half a padded state; ops that take their states from elsewhere have none)
+                assert ws % 16 == 0 and ws <= slots * pad(dk) * pad(dv) * 4, (cus, which, saved, b, h, n, dk, dv, dt, ws)
+                if which == 0 and cus <= 256:
+                    assert ws <= L.cott_noalloc_scratch_bytes(), (cus, b, h, n, dk, dv, dt, ws)
+        assert seen_groups > 50 and seen_pair > 5 and seen_comp > 5
+    finally:
+        assert L.cott_plan_geometry(0, 0) == _loader.OK

@@ -42,9 +42,10 @@ def both(L, q, k, v, code, rev=0):
 def test_no_alloc_entry_point_equals_workspace_entry_point(L, oracle, dt):
     from cottention_transformer_amd import _loader
     code = _loader.BF16 if dt == BF else _loader.F32
-    assert L.cott_noalloc_scratch_bytes() == 32 << 20
-    # first a long sequence in many groups of 128-wide heads, then a smaller, ragged one: both use the scratch
-    for (b, h, n, d, rev) in ((1, 4, 8192, 128, 0), (1, 2, 1023, 64, 0), (1, 2, 1023, 64, 1)):
+    assert L.cott_noalloc_scratch_bytes() == 48 << 20
+    # first long sequences in many groups of 128-wide heads, then a smaller, ragged one: all use the scratch
+    # (the first shape, 80 heads in three groups of three pieces each, has the largest slot array of all plans: 45 MiB)
+    for (b, h, n, d, rev) in ((5, 16, 16384, 128, 0), (1, 4, 8192, 128, 0), (1, 2, 1023, 64, 0), (1, 2, 1023, 64, 1)):
         print("no-alloc", (b, h, n, d, rev, dt), flush=True)
         q, k, v, _ = inputs(b, h, n, d, d, dt, seed=n + rev)
         want, got, need = both(L, q.to(DEV), k.to(DEV), v.to(DEV), code, rev)
@@ -67,7 +68,7 @@ def test_no_alloc_entry_point_in_a_hip_graph(L):
     assert L.cott_causal_workspace_bytes(b, h, n, d, d, _loader.BF16) > 0, "the shape must use group-state slots"
     q, k, v, _ = (x.to(DEV) for x in inputs(b, h, n, d, d, BF, seed=7))
     out = torch.full_like(v, float("nan"))
-    assert L.cott_noalloc_scratch_bytes() == 32 << 20            # resolves the symbol, outside the capture
+    assert L.cott_noalloc_scratch_bytes() == 48 << 20            # resolves the symbol, outside the capture
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     graph = torch.cuda.CUDAGraph()
