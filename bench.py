@@ -25,7 +25,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # `bench.py --calibration-copy` (counters scaled by their reading for the 256 MiB copy in the same run).
 # A counter run cannot be made from inside this script; the figures and commands are in
 # profiles/headline_kernels_hbm_traffic_pmc.txt.
-MEASURED_TRAFFIC_BYTES = {"scan": 127.25 * 2**20, "scan_grad": 223.18 * 2**20}
+MEASURED_TRAFFIC_BYTES = {"scan": 127.26 * 2**20, "scan_grad": 223.16 * 2**20}
 
 
 def parse():
@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--long-only", type=int, default=0, metavar="N",
                     help="run only the long-context configuration B1 H16 D128 bf16 at sequence length N (fwd and bwd "
                          "separately, per-kernel durations) for --steps steps: for profiling")
+    ap.add_argument("--cold-only", action="store_true",
+                    help="run only the headline forward and gradient launches with cold caches (and the streaming-only "
+                         "kernel of their launch shape): for counter runs whose per-dispatch averages are cold launches")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -137,6 +140,13 @@ def main():
         return
     B, H, N, D = 8, 16, 2048, 64
     q, k, v, do = make_inputs(torch, B, H, N, D, D, torch.bfloat16, dev)
+    if args.cold_only:
+        def fwd_saving():
+            return ct.causal_dot_product_saving(q, k, v)
+        saved = fwd_saving()[1]
+        print(json.dumps({"cold_cache_headline": cold_cache_kernel_times(
+            torch, fwd_saving, lambda: ct.causal_backward(q, k, v, do, saved=saved), dev, B * H * N * D * 2, 256)}))
+        return
 
     # The step as CustomAttention runs it on 16-bit tensors: the forward pass leaves the state dQ starts from (here one
     # 16 KiB slot per head, the sum over the whole sequence) and the backward pass takes it, so that dQ walks the
