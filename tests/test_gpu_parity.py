@@ -812,8 +812,12 @@ def test_input_preparation_inside_the_forward_kernel(ct, oracle, case):
         assert got.shape == ref.shape and rel_l2(got, ref.numpy()) <= 2e-2, name
 
 
-@pytest.mark.parametrize("case", [(8, 16, 256, 64, 64, BF, 64, True), (4, 32, 1000, 64, 128, HF, 16, False)],
-                         ids=["8x16x256-bf16-bnhd", "4x32x1000-fp16"])
+@pytest.mark.parametrize("case", [(8, 16, 256, 64, 64, BF, 64, True), (4, 32, 1000, 64, 128, HF, 16, False),
+                                  (10, 16, 300, 128, 128, BF, 32, True),      # 128-wide rows: the column-owner scan
+                                  (2, 8, 700, 128, 128, HF, 128, False),      # ... cut into groups (preparing group-state pass)
+                                  (1, 4, 3000, 64, 64, BF, 64, True)],        # 64-wide rows in groups
+                         ids=["8x16x256-bf16-bnhd", "4x32x1000-fp16", "10x16x300x128-bf16-bnhd", "2x8x700x128-fp16-groups",
+                              "1x4x3000-bf16-bnhd-groups"])
 def test_fused_preparation_with_position_ids(ct, oracle, case):
     """cott_causal_fwd_prep with the block's own position_ids tensor (GPT_Trainer/GPTCosAttention.py:458): ids that are
     neither consecutive nor equal across the batch, one row repeated for the whole batch as GPT-J's model passes them,
