@@ -648,14 +648,16 @@ int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtyp
 int cott_causal_fwd_prep_preferred(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim) {
     if (!cott_causal_fwd_prep_supported(B, H, N, Dk, Dv, dtype, rotary_dim)) return 0;
     if ((long)B * H * N == 0) return 1;
-    // The preparation is vector-ALU work of the loader wavefronts, which hides behind the other roles only for rows of
-    // up to 64 columns of heads that are one group.  Measured in a loop over one shape, rotary 32 with position ids,
-    // mask and value scaling (one launch against cott_prep_ex_fwd + cott_causal_fwd): B8 H16 N2048 D64 87 against 63 us
-    // (inside the GPT block, where the tensors come from memory, 74 against 71 us and one launch less: the block's step
-    // 741 against 770 us); D128 248 against 160 us; B4 H16 N8192 D128 508 against 351 us; B1 H16 N65536 D128 1002
-    // against 720 us (group-state pass 352 us, scan 643 us); B2 H12 N16384 D64 274 against 140 us.
+    // Heads that are one group: the one launch wins at every width.  Measured in a loop over one shape, rotary 32 with
+    // position ids, mask and value scaling, one launch against cott_prep_ex_fwd + cott_causal_fwd: B16 H16 N2048 D64
+    // 111 against 138 us, D128 210 against 278; B32 H16 N2048 D128 416 against 564; in column halves B8 H16 N2048 D64
+    // 60 against 59..67 from run to run, N8192 281 against 306, D128 N2048 137 against 159, N8192
+    // 499 against 628.  Heads cut into sequence groups: even as whole problems (B1 H16 N65536 D128 682 against 723, D64
+    // 328 against 341, N32768 D128 365 against 371, B4 H16 N8192 D128 353 against 343, B2 H12 N32768 D128 548 against
+    // 522), slower as column halves in groups, where both halves of a head prepare its q and k rows and so does the
+    // group-state pass (B2 H12 N8192 D64 90 against 65, D128 194 against 150; B1 H16 N8192 D128 119 against 91).
     const SetPlan p = plan_set((long)B * H, N, 1, Dk, Dv, true, dtype);
-    return cott::mfma_pad(Dk) <= 64 && p.G == 1;
+    return p.G == 1;
 }
 
 namespace {

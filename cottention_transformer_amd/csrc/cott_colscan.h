@@ -155,7 +155,8 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
     };
     u32x4 ra[PF][NB], rb[PF][NB], rc[PF][NC];
     f32x4 sn[PF][NB], cs[PF][NB];
-    float keep_ab[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
+    uint32_t keep_ab[PF][NB], keep_c[PF][NC];  // the bytes as loaded: converting them here would wait for the load
+    float cnt_c[PF][NC];
     auto row0_of = [&](int p) __attribute__((always_inline)) {
         const int pc = min(p, r.p1 - 1);
         return (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
@@ -189,7 +190,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
             ra[s][u] = buf_load16(rA, (uint32_t)(row * lda + col) * 2u);
             rb[s][u] = buf_load16(rB, (uint32_t)(row * ldb + col) * 2u);
             const int srow = min(row, r.N - 1);
-            keep_ab[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            keep_ab[s][u] = ps.keep != nullptr ? (uint32_t)ps.keep[tok0 + srow] : 1u;
             if (ps.rot != nullptr && col < ps.R) {
                 const float *t = ps.rot + (size_t)trow[u] * ps.R + col / 2;
                 sn[s][u] = *reinterpret_cast<const f32x4 *>(t);
@@ -202,7 +203,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
             const int row = row0 + v / (DJ / 8), col = (v % (DJ / 8)) * 8;
             rc[s][u] = buf_load16(rC, (uint32_t)(row * ldc + col) * 2u);
             const int srow = min(row, r.N - 1);
-            keep_c[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            keep_c[s][u] = ps.keep != nullptr ? (uint32_t)ps.keep[tok0 + srow] : 1u;
             cnt_c[s][u] = scaled ? ps.cnt[tok0 + srow] : 0.f;
         }
     };
@@ -214,8 +215,8 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
             const int v = tid + LT * u;
             const int lrow = v / (DI / 8), col = (v % (DI / 8)) * 8;
             const bool rotate = ps.rot != nullptr && col < ps.R;
-            const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
-            const u32x4 yb = prep_qk_piece<TR, DI / 8>(rb[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
+            const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], (float)keep_ab[s][u], ps.eps);
+            const u32x4 yb = prep_qk_piece<TR, DI / 8>(rb[s][u], col, di, rotate, sn[s][u], cs[s][u], (float)keep_ab[s][u], ps.eps);
             *reinterpret_cast<u32x4 *>(ta + lrow * TL::BS + col) = ya;
             *reinterpret_cast<u32x4 *>(tb + lrow * TL::BS + col) = yb;
             const uint32_t off = (col < di && p < r.p1) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
@@ -226,7 +227,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
         for (int u = 0; u < NC; ++u) {
             const int v = tid + LT * u;
             const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
-            const u32x4 y = prep_v_piece<TR>(rc[s][u], col < dj, keep_c[s][u], cnt_c[s][u], sig, scaled);
+            const u32x4 y = prep_v_piece<TR>(rc[s][u], col < dj, (float)keep_c[s][u], cnt_c[s][u], sig, scaled);
             *reinterpret_cast<u32x4 *>(tc + lrow * TL::CS + col) = y;
             const uint32_t off = (col < dj && p < r.p1) ? (uint32_t)((row0 + lrow) * ps.dv + col) * 2u : kOobOffset;
             __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);

@@ -395,7 +395,8 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
     // and issued before that iteration's tile loads, so that waiting for them does not wait for those.  Position ids
     // are fetched one step earlier still, since the table entries' addresses depend on them.
     f32x4 sn[NB], cs[NB];
-    float keep_b[NB], keep_c[NC], cnt_c[NC];
+    uint32_t keep_b[NB], keep_c[NC];  // the bytes as loaded: converting them at once would wait for the load
+    float cnt_c[NC];
     const size_t tok0 = PREP ? (size_t)(wi.bh / prep.H) * N : 0;
     const bool scaled = PREP && prep.cnt != nullptr && prep.sig != nullptr;
     const float sig = scaled ? prep.sig[wi.bh % prep.H] : 0.f;
@@ -432,7 +433,7 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
         for (int u = 0; u < NB; ++u) {
             const int v = tid + kThreads * u;
             const int srow = min(row0 + v / (DI / 8), N - 1), col = (v % (DI / 8)) * 8;
-            keep_b[u] = prep.keep != nullptr ? (float)__builtin_amdgcn_raw_buffer_load_b8(rKeep, srow, 0, 0) : 1.f;
+            keep_b[u] = prep.keep != nullptr ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(rKeep, srow, 0, 0) : 1u;
             const uint32_t toff = (rotary && col < prep.R) ? (uint32_t)(trow[u] * prep.R + col / 2) * 4u : kOobOffset;
             sn[u] = bitcast<f32x4>(__builtin_amdgcn_raw_buffer_load_b128(rRot, (int)toff, 0, 0));
             cs[u] = bitcast<f32x4>(__builtin_amdgcn_raw_buffer_load_b128(rRot, (int)toff, prep.R * 2, 0));
@@ -440,7 +441,7 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
 #pragma unroll
         for (int u = 0; u < NC; ++u) {
             const int srow = min(row0 + (tid + kThreads * u) / (DJ / 8), N - 1);
-            keep_c[u] = prep.keep != nullptr ? (float)__builtin_amdgcn_raw_buffer_load_b8(rKeep, srow, 0, 0) : 1.f;
+            keep_c[u] = prep.keep != nullptr ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(rKeep, srow, 0, 0) : 1u;
             cnt_c[u] = bitcast<float>(__builtin_amdgcn_raw_buffer_load_b32(rCnt, srow * 4, 0, 0));
         }
     };
@@ -460,7 +461,7 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
                 const int v = tid + kThreads * u;
                 const int col = (v % (DI / 8)) * 8;
                 *reinterpret_cast<u32x4 *>(tb + (v / (DI / 8)) * TL::BS + col) = prep_qk_piece<TR, DI / 8>(
-                    rb[s][u], col, di, rotary && col < prep.R, sn[u], cs[u], keep_b[u], prep.eps);
+                    rb[s][u], col, di, rotary && col < prep.R, sn[u], cs[u], (float)keep_b[u], prep.eps);
                 __builtin_amdgcn_sched_barrier(0);  // one piece at a time: eight unpacked columns each are enough registers
             }
 #pragma unroll
@@ -468,7 +469,7 @@ __global__ __launch_bounds__(kThreads, 2) void group_state_kernel(ProblemSet set
                 const int v = tid + kThreads * u;
                 const int col = (v % (DJ / 8)) * 8;
                 *reinterpret_cast<u32x4 *>(tc + (v / (DJ / 8)) * TL::CS + col) =
-                    prep_v_piece<TR>(rc[s][u], col < dj, keep_c[u], cnt_c[u], sig, scaled);
+                    prep_v_piece<TR>(rc[s][u], col < dj, (float)keep_c[u], cnt_c[u], sig, scaled);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -673,7 +674,8 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
     };
     u32x4 ra[PF][NB], rb[PF][NB], rc[PF][NC];
     f32x4 sn[PF][NB], cs[PF][NB];
-    float keep_ab[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
+    uint32_t keep_ab[PF][NB], keep_c[PF][NC];  // the bytes as loaded: converting them here would wait for the load
+    float cnt_c[PF][NC];
     auto row0_of = [&](int p) __attribute__((always_inline)) {
         const int pc = min(p, r.p1 - 1);
         return (r.reversed ? r.nchunks - 1 - pc : pc) * kChunk;
@@ -711,7 +713,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
             ra[s][u] = buf_load16(rA, (uint32_t)(row * lda + col) * 2u);
             rb[s][u] = buf_load16(rB, (uint32_t)(row * ldb + col) * 2u);
             const int srow = min(row, r.N - 1);
-            keep_ab[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            keep_ab[s][u] = ps.keep != nullptr ? (uint32_t)ps.keep[tok0 + srow] : 1u;
             if (ps.rot != nullptr && col < ps.R) {
                 const float *t = ps.rot + (size_t)trow[u] * ps.R + col / 2;
                 sn[s][u] = *reinterpret_cast<const f32x4 *>(t);
@@ -724,7 +726,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
             const int row = row0 + v / (DJ / 8), col = (v % (DJ / 8)) * 8;
             rc[s][u] = buf_load16(rC, (uint32_t)(row * ldc + col) * 2u);
             const int srow = min(row, r.N - 1);
-            keep_c[s][u] = ps.keep != nullptr ? (float)ps.keep[tok0 + srow] : 1.f;
+            keep_c[s][u] = ps.keep != nullptr ? (uint32_t)ps.keep[tok0 + srow] : 1u;
             cnt_c[s][u] = scaled ? ps.cnt[tok0 + srow] : 0.f;
         }
     };
@@ -736,8 +738,8 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
             const int v = tid + LT * u;
             const int lrow = v / (DI / 8), col = (v % (DI / 8)) * 8;
             const bool rotate = ps.rot != nullptr && col < ps.R;
-            const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
-            const u32x4 yb = prep_qk_piece<TR, DI / 8>(rb[s][u], col, di, rotate, sn[s][u], cs[s][u], keep_ab[s][u], ps.eps);
+            const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], (float)keep_ab[s][u], ps.eps);
+            const u32x4 yb = prep_qk_piece<TR, DI / 8>(rb[s][u], col, di, rotate, sn[s][u], cs[s][u], (float)keep_ab[s][u], ps.eps);
             *reinterpret_cast<u32x4 *>(ta + lrow * TL::BS + col) = ya;
             *reinterpret_cast<u32x4 *>(tb + lrow * TL::BS + col) = yb;
             const uint32_t off = (col < di) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
@@ -748,7 +750,7 @@ __device__ __forceinline__ void loader_role_prep(const u16 *A_head, const u16 *B
         for (int u = 0; u < NC; ++u) {
             const int v = tid + LT * u;
             const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
-            const u32x4 y = prep_v_piece<TR>(rc[s][u], col < dj, keep_c[s][u], cnt_c[s][u], sig, scaled);
+            const u32x4 y = prep_v_piece<TR>(rc[s][u], col < dj, (float)keep_c[s][u], cnt_c[s][u], sig, scaled);
             *reinterpret_cast<u32x4 *>(tc + lrow * TL::CS + col) = y;
             const uint32_t off = (col < dj) ? (uint32_t)((row0 + lrow) * ps.dv + col) * 2u : kOobOffset;
             __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);
@@ -1424,12 +1426,12 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
     const float sig = scaled ? prep.sig[wi.bh % prep.H] : 0.f;
 
     u32x4 qn[PF2][TL::KS];
-    float keep_q[PF2];
+    uint32_t keep_q[PF2];
     auto load_q = [&](int s, int p) __attribute__((always_inline)) {
         const int row = min(p, nchunks - 1) * kChunk + 16 * w + m;
 #pragma unroll
         for (int ks = 0; ks < TL::KS; ++ks) qn[s][ks] = buf_load16(rA, (uint32_t)(row * lda + 32 * ks + 8 * g) * 2u);
-        if constexpr (PREP) keep_q[s] = prep.keep != nullptr ? (float)prep.keep[tok0 + min(row, N - 1)] : 1.f;
+        if constexpr (PREP) keep_q[s] = prep.keep != nullptr ? (uint32_t)prep.keep[tok0 + min(row, N - 1)] : 1u;
     };
 
     // ---- pass 1: S = sum over all chunks of B_c^T C_c
@@ -1438,7 +1440,8 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
     for (int u = 0; u < TL::TPW; ++u) S[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     {
         u32x4 rb[PF][NB], rc[PF][NC];
-        float keep_b[PF][NB], keep_c[PF][NC], cnt_c[PF][NC];
+        uint32_t keep_b[PF][NB], keep_c[PF][NC];  // the bytes as loaded: converting them at once would wait for the load
+        float cnt_c[PF][NC];
         auto load_chunk = [&](int s, int p) __attribute__((always_inline)) {
             const int row0 = min(p, nchunks - 1) * kChunk;
             load_tile<DI>(rb[s], rB, row0, ldb, tid);
@@ -1447,12 +1450,12 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
 #pragma unroll
                 for (int u = 0; u < NB; ++u) {
                     const int srow = min(row0 + (tid + kThreads * u) / (DI / 8), N - 1);
-                    keep_b[s][u] = prep.keep != nullptr ? (float)prep.keep[tok0 + srow] : 1.f;
+                    keep_b[s][u] = prep.keep != nullptr ? (uint32_t)prep.keep[tok0 + srow] : 1u;
                 }
 #pragma unroll
                 for (int u = 0; u < NC; ++u) {
                     const int srow = min(row0 + (tid + kThreads * u) / (DJ / 8), N - 1);
-                    keep_c[s][u] = prep.keep != nullptr ? (float)prep.keep[tok0 + srow] : 1.f;
+                    keep_c[s][u] = prep.keep != nullptr ? (uint32_t)prep.keep[tok0 + srow] : 1u;
                     cnt_c[s][u] = scaled ? prep.cnt[tok0 + srow] : 0.f;
                 }
             }
@@ -1478,7 +1481,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
                     }
                     ss = lane_group_sum<DI / 8>(ss);
                     const float nrm = __builtin_amdgcn_sqrtf(ss);
-                    const float mul = keep_b[s][u] * __builtin_amdgcn_rcpf(nrm > prep.eps ? nrm : prep.eps);
+                    const float mul = (float)keep_b[s][u] * __builtin_amdgcn_rcpf(nrm > prep.eps ? nrm : prep.eps);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) x[e] *= mul;
                     const u32x4 y = pack8<TR>(x);
@@ -1492,7 +1495,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
                     const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
                     float x[8];
                     unpack8<TR>(rc[s][u], x);
-                    const float mul = (col < dj) ? value_scale(keep_c[s][u], cnt_c[s][u], sig, scaled) : 0.f;
+                    const float mul = (col < dj) ? value_scale((float)keep_c[s][u], cnt_c[s][u], sig, scaled) : 0.f;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) x[e] *= mul;
                     const u32x4 y = (col < dj) ? pack8<TR>(x) : u32x4{0u, 0u, 0u, 0u};
@@ -1561,7 +1564,7 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
                 ss += __shfl_xor(ss, 16, 64);
                 ss += __shfl_xor(ss, 32, 64);
                 const float nrm = __builtin_amdgcn_sqrtf(ss);
-                const float mul = keep_q[s] * __builtin_amdgcn_rcpf(nrm > prep.eps ? nrm : prep.eps);
+                const float mul = (float)keep_q[s] * __builtin_amdgcn_rcpf(nrm > prep.eps ? nrm : prep.eps);
 #pragma unroll
                 for (int ks = 0; ks < TL::KS; ++ks) {
 #pragma unroll
