@@ -648,16 +648,17 @@ int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtyp
 int cott_causal_fwd_prep_preferred(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim) {
     if (!cott_causal_fwd_prep_supported(B, H, N, Dk, Dv, dtype, rotary_dim)) return 0;
     if ((long)B * H * N == 0) return 1;
-    // Heads that are one group: the one launch wins at every width.  Measured in a loop over one shape, rotary 32 with
-    // position ids, mask and value scaling, one launch against cott_prep_ex_fwd + cott_causal_fwd: B16 H16 N2048 D64
-    // 111 against 138 us, D128 210 against 278; B32 H16 N2048 D128 416 against 564; in column halves B8 H16 N2048 D64
-    // 60 against 59..67 from run to run, N8192 281 against 306, D128 N2048 137 against 159, N8192
-    // 499 against 628.  Heads cut into sequence groups: even as whole problems (B1 H16 N65536 D128 682 against 723, D64
-    // 328 against 341, N32768 D128 365 against 371, B4 H16 N8192 D128 353 against 343, B2 H12 N32768 D128 548 against
-    // 522), slower as column halves in groups, where both halves of a head prepare its q and k rows and so does the
-    // group-state pass (B2 H12 N8192 D64 90 against 65, D128 194 against 150; B1 H16 N8192 D128 119 against 91).
+    // Measured in a loop over one shape, rotary 32 with position ids, mask and value scaling, one launch against
+    // cott_prep_ex_fwd + cott_causal_fwd.  Heads that are one group: B16 H16 N2048 D64 113 against 137 us, D128 210
+    // against 275; B32 H16 N2048 D128 413 against 563; in column halves B8 H16 N2048 D64 61 against 60..67, N8192 282
+    // against 306, D128 N2048 143 against 160, N8192 509 against 628.  Whole problems in sequence groups (the sums of
+    // 64- and 128-wide rows by colsum_prep_kernel): B1 H16 N65536 D128 567 against 722, N32768 312 against 372, B4 H16
+    // N8192 D128 305 against 338, B2 H12 N32768 D128 460 against 522; D64 even or a little ahead (B4 H16 N32768 598
+    // against 650, N8192 166 against 161, B1 H16 N32768 170 against 169).  Column halves in groups are slower: both
+    // halves of a head prepare its q and k rows and so does the group-state pass (B2 H12 N8192 D64 92 against 65, D128
+    // 183 against 149; B1 H16 N8192 D128 112 against 92).
     const SetPlan p = plan_set((long)B * H, N, 1, Dk, Dv, true, dtype);
-    return p.G == 1;
+    return p.G == 1 || p.halves == 1;
 }
 
 namespace {

@@ -120,7 +120,9 @@ __device__ __forceinline__ void col_loader_role(const u16 *A_head, const u16 *B_
 // and share their rotary table entries.  Side inputs (keep, count, table entries) travel with the pieces, PF chunks
 // ahead; position ids one call earlier than the table entries they select.  first_half: this workgroup writes qo and
 // ko (the two column halves of a head prepare the same q and k rows).
-template <class TR, int DI, int DJ, int PF, int LT>
+// SUMS: the group-state pass of such a forward (colsum_prep_kernel): only the B and C tiles are loaded, prepared and staged,
+// nothing is written to memory (the scan that follows leaves the prepared rows).
+template <class TR, int DI, int DJ, int PF, int LT, bool SUMS = false>
 __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u16 *B_head, const u16 *C_head, u16 *O_head,
                                                      int di, int dj, int lda, int ldb, int ldc, int ldo, const ScanRange &r,
                                                      int tid, u16 *sA, u16 *sB, u16 *sC, const u16 *sO, const PrepSide &ps,
@@ -187,7 +189,7 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
         for (int u = 0; u < NB; ++u) {
             const int v = tid + LT * u;
             const int row = row0 + v / (DI / 8), col = (v % (DI / 8)) * 8;
-            ra[s][u] = buf_load16(rA, (uint32_t)(row * lda + col) * 2u);
+            if constexpr (!SUMS) ra[s][u] = buf_load16(rA, (uint32_t)(row * lda + col) * 2u);
             rb[s][u] = buf_load16(rB, (uint32_t)(row * ldb + col) * 2u);
             const int srow = min(row, r.N - 1);
             keep_ab[s][u] = ps.keep != nullptr ? (uint32_t)ps.keep[tok0 + srow] : 1u;
@@ -215,13 +217,15 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
             const int v = tid + LT * u;
             const int lrow = v / (DI / 8), col = (v % (DI / 8)) * 8;
             const bool rotate = ps.rot != nullptr && col < ps.R;
-            const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], (float)keep_ab[s][u], ps.eps);
             const u32x4 yb = prep_qk_piece<TR, DI / 8>(rb[s][u], col, di, rotate, sn[s][u], cs[s][u], (float)keep_ab[s][u], ps.eps);
-            *reinterpret_cast<u32x4 *>(ta + lrow * TL::BS + col) = ya;
             *reinterpret_cast<u32x4 *>(tb + lrow * TL::BS + col) = yb;
-            const uint32_t off = (col < di && p < r.p1) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
-            __builtin_amdgcn_raw_buffer_store_b128(ya, rQo, (int)off, 0, 0);
-            __builtin_amdgcn_raw_buffer_store_b128(yb, rKo, (int)off, 0, 0);
+            if constexpr (!SUMS) {
+                const u32x4 ya = prep_qk_piece<TR, DI / 8>(ra[s][u], col, di, rotate, sn[s][u], cs[s][u], (float)keep_ab[s][u], ps.eps);
+                *reinterpret_cast<u32x4 *>(ta + lrow * TL::BS + col) = ya;
+                const uint32_t off = (col < di && p < r.p1) ? (uint32_t)((row0 + lrow) * di + col) * 2u : kOobOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(ya, rQo, (int)off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(yb, rKo, (int)off, 0, 0);
+            }
         }
 #pragma unroll
         for (int u = 0; u < NC; ++u) {
@@ -229,8 +233,10 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
             const int lrow = v / (DJ / 8), col = (v % (DJ / 8)) * 8;
             const u32x4 y = prep_v_piece<TR>(rc[s][u], col < dj, (float)keep_c[s][u], cnt_c[s][u], sig, scaled);
             *reinterpret_cast<u32x4 *>(tc + lrow * TL::CS + col) = y;
-            const uint32_t off = (col < dj && p < r.p1) ? (uint32_t)((row0 + lrow) * ps.dv + col) * 2u : kOobOffset;
-            __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);
+            if constexpr (!SUMS) {
+                const uint32_t off = (col < dj && p < r.p1) ? (uint32_t)((row0 + lrow) * ps.dv + col) * 2u : kOobOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(y, rVo, (int)off, 0, 0);
+            }
         }
     };
 #pragma unroll
@@ -243,12 +249,15 @@ __device__ __forceinline__ void col_loader_role_prep(const u16 *A_head, const u1
         const int buf = (p - r.p0) & 1;
         stage(s1, p + 1, sA + (buf ^ 1) * CT::SA, sB + (buf ^ 1) * CT::SA, sC + (buf ^ 1) * CT::SC);
         load_chunk(s1, p + 1 + PF);
-        if (p > r.p0 + 1) write_out(p - 2);
+        if constexpr (!SUMS)
+            if (p > r.p0 + 1) write_out(p - 2);
         chunk_barrier();
     });
-    if (r.p1 > r.p0 + 1) write_out(r.p1 - 2);
+    if constexpr (!SUMS)
+        if (r.p1 > r.p0 + 1) write_out(r.p1 - 2);
     __syncthreads();
-    if (r.p1 > r.p0) write_out(r.p1 - 1);
+    if constexpr (!SUMS)
+        if (r.p1 > r.p0) write_out(r.p1 - 1);
 }
 
 // Where the compute wavefront `w` of a workgroup finds and leaves its state (all pointers already at this head, and
@@ -260,6 +269,7 @@ struct ColStateIO {
     const float *sin = nullptr;       // row-major [di][lds] hand-over state to start from
     float *sout = nullptr;            // ... and to leave at the end (last group only)
     int lds = 0;
+    float *sums = nullptr;            // SUMS: where the sum of B^T C over the chunks walked goes, plain tile layout
     float *save = nullptr;            // states for a backward pass (ProblemT::save): first slot of this head
     int save_njt = 0, save_jt0 = 0, save_slot = 0, save_cpg = 1, save_n = 0;
 };
@@ -276,7 +286,8 @@ struct ColStateIO {
 // pays the full LDS latency some forty times per chunk).
 __device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 
-template <class TR, int DI, int DJ, bool FUT>
+// SUMS: only the state update runs, from a zero state, and the sum is left in io.sums (colsum_prep_kernel).
+template <class TR, int DI, int DJ, bool FUT, bool SUMS = false>
 __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, int dj, const ScanRange &r, int w, int l,
                                                    const u16 *sA, const u16 *sB, const u16 *sC, u16 *sO, u32x2 *sP) {
     using TL = Tiling<DI, DJ>;
@@ -480,6 +491,21 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
             }
         };
 
+        if constexpr (SUMS) {
+            read_c();
+            read_b(0, 0, 0);
+            sched_fence();
+            constexpr int NBS = 2 * (NIT / 4);
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) {
+                if (b + 1 < NBS) read_b((b + 1) & 1, (b + 1) / (NIT / 4), 4 * ((b + 1) % (NIT / 4)));
+                sched_fence();
+                update(b & 1, b / (NIT / 4), 4 * (b % (NIT / 4)));
+                sched_fence();
+            }
+            chunk_barrier();
+            continue;
+        }
         if (p > r.p0) finish(buf ^ 1);
         read_score(0, 0);
         sched_fence();
@@ -528,10 +554,17 @@ __device__ __forceinline__ void col_compute_role(const ColStateIO &io, int di, i
         }
         chunk_barrier();
     }
-    if (r.p1 > r.p0) {
-        finish((r.p1 - 1 - r.p0) & 1);
+    if constexpr (!SUMS) {
+        if (r.p1 > r.p0) finish((r.p1 - 1 - r.p0) & 1);
     }
     __syncthreads();  // (the loader wavefronts send the last tile out after this)
+    if constexpr (SUMS) {
+        f32x4 *dst = reinterpret_cast<f32x4 *>(io.sums);
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int jw = 0; jw < NJW; ++jw) dst[plain_index(it, NJW * w + jw, TL::NJT)] = S[it][jw];
+    }
     if (io.sout != nullptr) {
 #pragma unroll
         for (int it = 0; it < NIT; ++it)
@@ -618,6 +651,52 @@ __global__ __launch_bounds__(512) void colscan_kernel(ProblemSet set, int BH, in
         col_compute_role<TR, DI, DJ, true>(io, di, dj, r, wv, l, sA, sB, sC, sO, sP);
     else
         col_compute_role<TR, DI, DJ, false>(io, di, dj, r, wv, l, sA, sB, sC, sO, sP);
+}
+
+// The group-state pass of a forward that prepares its inputs itself, for 128-wide q / k rows: sum of k_hat^T v_hat over
+// each piece of each group of chunks, with the roles of colscan_kernel: four loader wavefronts prepare and stage the k and
+// v tiles, four compute wavefronts each keep a quarter of the sum's columns.  Same grid, pieces and slots as
+// group_state_kernel, whose single role does all of this (N = 65536, 16 heads: 299 us there).
+template <class TR, int DI, int DJ, int PF>
+__global__ __launch_bounds__(512) void colsum_prep_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G,
+                                                          int ngroups, PrepSide prep) {
+    using TL = Tiling<DI, DJ>;
+    using CT = ColTiling<DI, DJ>;
+    __shared__ __attribute__((aligned(16))) u16 sB[2 * CT::SA];
+    __shared__ __attribute__((aligned(16))) u16 sC[2 * CT::SC];
+    const int l = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int sub = set.sub;
+    const WorkItem wi = decode_workgroup(set.nact * sub, BH, set.xcds);
+    if (wi.grp >= ngroups) return;
+    const Problem &pr = set.p[set.act[wi.prob / sub]];
+    const int grp = wi.grp, piece = wi.prob % sub;
+    if (grp == G - 1 && ngroups == G && !pr.comp) return;
+    if (pr.seed_from >= 0 || pr.ext != nullptr) return;
+    const int cps = (cpg + sub - 1) / sub;  // chunks per piece
+    ScanRange r;
+    r.N = N;
+    r.nchunks = nchunks;
+    r.p0 = grp * cpg + piece * cps;
+    r.p1 = min(r.p0 + cps, min((grp + 1) * cpg, nchunks));
+    r.reversed = pr.reversed;
+    r.mask_rev = pr.mask_rev;
+    r.comp = 0;
+    float *slot = pr.gstate + (((size_t)wi.bh * G + grp) * sub + piece) * TL::STATE_FLOATS;
+    if (r.p1 <= r.p0) {  // a piece past the end of its group: its slot is zero
+        for (int e = threadIdx.x; e < TL::STATE_FLOATS / 4; e += 512) reinterpret_cast<f32x4 *>(slot)[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+        return;
+    }
+    if (wv >= 4) {
+        col_loader_role_prep<TR, DI, DJ, PF, 256, true>(nullptr, pr.B + head_base(pr.bsB, pr.hsB, pr.H, wi.bh),
+                                                        pr.C + head_base(pr.bsC, pr.hsC, pr.H, wi.bh), nullptr, pr.di, pr.dj,
+                                                        pr.lda, pr.ldb, pr.ldc, pr.ldo, r, (int)threadIdx.x - 256, nullptr, sB,
+                                                        sC, nullptr, prep, wi.bh, pr.c0, false);
+        return;
+    }
+    ColStateIO io;
+    io.sums = slot;
+    col_compute_role<TR, DI, DJ, false, true>(io, pr.di, pr.dj, r, wv, l, nullptr, sB, sC, nullptr, nullptr);
 }
 
 }  // namespace cott

@@ -230,9 +230,9 @@ def fused_preparation_supported(dtype, b, h, n, dk, dv, rotary_dim=0):
 
 
 def fused_preparation_preferred(dtype, b, h, n, dk, dv, rotary_dim=0):
-    """Whether the one launch of causal_dot_product_prepared is also the faster form for the shape (heads that are not
-    cut into sequence groups: cott_causal_fwd_prep_preferred); the modules take prepare_inputs + causal_dot_product
-    elsewhere."""
+    """Whether the one launch of causal_dot_product_prepared is also the faster form for the shape (all but those planned
+    as column halves in sequence groups: cott_causal_fwd_prep_preferred); the modules take prepare_inputs +
+    causal_dot_product elsewhere."""
     if dtype not in (torch.bfloat16, torch.float16):
         return False
     key = ("preferred", dtype, b, h, n, dk, dv, rotary_dim)

@@ -269,10 +269,9 @@ COTT_API int cott_prep_ex_bwd(const void *q, const void *k, const void *v,
  * same shape (cott_causal_workspace_bytes; sequences cut into groups, whose group sums are then formed from rows
  * prepared the same way; NULL / 0 when that is 0). */
 COTT_API int cott_causal_fwd_prep_supported(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim);
-/* 1 where the one launch has also measured faster than cott_prep_ex_fwd followed by cott_causal_fwd (heads that are
- * not cut into sequence groups, at every width; in groups the two forms are about even as whole problems and the one
- * launch is slower as column halves), else 0: the rule the modules of this package follow when they choose between
- * the two forms.  Pure host function. */
+/* 1 where the one launch has also measured faster than cott_prep_ex_fwd followed by cott_causal_fwd (every shape but
+ * those planned as column halves in sequence groups: few heads, medium sequence lengths), else 0: the rule the
+ * modules of this package follow when they choose between the two forms.  Pure host function. */
 COTT_API int cott_causal_fwd_prep_preferred(int B, int H, int N, int Dk, int Dv, int dtype, int rotary_dim);
 COTT_API int cott_causal_fwd_prep(const void *q, const void *k, const void *v, void *o,
                          void *q_out, void *k_out, void *v_out,

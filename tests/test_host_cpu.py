@@ -156,8 +156,9 @@ def test_c_abi_argument_errors_without_a_gpu():
     # the form the modules choose: only where the one launch has measured faster
     assert L.cott_causal_fwd_prep_preferred(8, 16, 2048, 64, 64, _loader.BF16, 64) == 1
     assert L.cott_causal_fwd_prep_preferred(8, 16, 256, 128, 128, _loader.BF16, 64) == 1
-    assert L.cott_causal_fwd_prep_preferred(2, 12, 8192, 128, 128, _loader.BF16, 64) == 0      # sequence groups
-    assert L.cott_causal_fwd_prep_preferred(1, 16, 65536, 64, 64, _loader.BF16, 64) == 0       # sequence groups
+    assert L.cott_causal_fwd_prep_preferred(1, 16, 65536, 128, 128, _loader.BF16, 64) == 1
+    assert L.cott_causal_fwd_prep_preferred(2, 12, 8192, 128, 128, _loader.BF16, 64) == 0      # column halves in groups
+    assert L.cott_causal_fwd_prep_preferred(1, 16, 65536, 64, 64, _loader.BF16, 64) == 1       # whole problems in groups
     assert L.cott_causal_fwd_prep_preferred(8, 16, 2048, 64, 64, _loader.F32, 0) == 0
     # ... and inside the non-causal kernel: 16-bit, a head must fit one workgroup
     ncprep = lambda *shape_dtype, cnt=None, sig=None: L.cott_noncausal_fwd_prep(
