@@ -548,6 +548,27 @@ def run_extras(torch, ct, dev):
     ex["noncausal_fwd_with_preparation_B32_H12_N512_D64"] = {"one_launch_us": s_nf * 1e6,
                                                              "separate_pass_plus_kernel_us": s_n2 * 1e6}
     del bq, bk, bv, bkeep, bcnt, bsig
+    # the GPT block's preparation (rotary with position ids, normalisation, value scaling, mask) inside the causal
+    # forward (cott_causal_fwd_prep) on the projections' (B,S,H,D) tensors, next to the separate pass followed by the
+    # plain forward: the headline shape and the GPT-1.2B head shape at the long-context length
+    for (cb, ch, cn, cd) in ((8, 16, 2048, 64), (1, 16, 65536, 128)):
+        cq, ck, cv = (torch.randn(cb, cn, ch, cd, device=dev).bfloat16() for _ in range(3))
+        ckeep = torch.rand(cb, cn, device=dev) > 0.1
+        ccnt = ckeep.float().cumsum(-1).contiguous()
+        csig = torch.sigmoid(torch.randn(ch, device=dev))
+        ctab = torch.randn(cn, 32, device=dev)
+        cpos = torch.arange(cn, device=dev).expand(cb, cn).contiguous()
+
+        def c_two_kernels():
+            p = ct.prepare_inputs(cq, ck, cv, ckeep, ccnt, csig, rotary=(ctab, cpos), bnhd=True, check_positions=False)
+            return ct.causal_dot_product(*p, merged_heads=True)
+        s_cf = time_region(torch, lambda: ct.causal_dot_product_prepared(cq, ck, cv, ckeep, ccnt, csig, rotary=(ctab, cpos),
+                                                                         bnhd=True, merged_heads=True), 30, 5)
+        s_c2 = time_region(torch, c_two_kernels, 30, 5)
+        ex[f"causal_fwd_with_preparation_B{cb}_H{ch}_N{cn}_D{cd}"] = {
+            "one_launch_us": s_cf * 1e6, "separate_pass_plus_kernel_us": s_c2 * 1e6,
+            "modules_take_the_one_launch": bool(ct.fused_preparation_preferred(torch.bfloat16, cb, ch, cn, cd, cd, 32))}
+        del cq, ck, cv, ckeep, ccnt, csig, ctab, cpos
     # whole GPT attention block (projections, rotary, preparation, attention, output projection), fwd+bwd under
     # bf16 autocast at the GPT-300M shape; second figure: same block with rotary / head permute as torch ops
     block_step = gpt_block_step(torch, dev)
