@@ -745,6 +745,11 @@ FUSED_PREP_CASES = [
     (2, 2, 2500, 48, 80, HF, 16, False, True),     # padded, per-head layout
     (1, 16, 4100, 128, 128, BF, 64, True, True),   # 128-wide: column halves in groups, ragged tail
     (1, 3, 6000, 128, 128, BF, 32, False, True),   # 128-wide: whole tiles in many groups
+    # whole problems in groups (the plans of many heads on long sequences): the group sums come from the kernel with
+    # loader and compute wavefronts
+    (1, 64, 4100, 128, 128, BF, 64, True, True),   # 128 x 128 tiles, four groups, ragged tail
+    (4, 16, 8200, 64, 64, HF, 32, False, True),    # 64 x 64 tiles
+    (2, 32, 4096, 64, 128, BF, 16, True, False),   # 64-wide rows, 128-wide values
 ]
 
 
