@@ -133,3 +133,35 @@ def test_decode_on_a_state_beyond_the_last_level_cache(ct, oracle):
     assert rel_l2(state[sub], ref_state) <= 1e-6
     total = s0.double() + torch.einsum("tbhi,tbhj->bhij", ks.double(), vs.double())
     assert float((state.double() - total).norm() / total.norm()) <= 1e-6
+
+
+@pytest.mark.parametrize("case", [(8, 16, 2048, 64, 64, BF, 64), (1, 16, 65536, 128, 128, BF, 32)],
+                         ids=["8x16x2048x64", "1x16x65536x128"])
+def test_one_launch_forward_with_preparation_at_benchmark_sizes(ct, oracle, case):
+    """cott_causal_fwd_prep at the two shapes the benchmark times it on (the headline shape: column halves, one group;
+    the long-context shape: whole 128 x 128 problems in 16 groups, the group sums by the kernel with loader and
+    compute wavefronts), on the projections' (B,N,H,D) tensors with a mask, value scaling and the rotation by position
+    ids: the prepared tensors against the CPU statement of GPT_Trainer/GPTCosAttention.py:229-248, 462-476 (elementwise,
+    the counts as a running sum of the mask) and the outputs against the causal oracle on those, per 64-row block."""
+    from oracle import torch_forms as tf
+    b, h, n, dk, dv, dt, rdim = case
+    say("one-launch forward with preparation", case)
+    g = torch.Generator().manual_seed(n + dk)
+    q, k, v = (torch.randn(b, n, h, d, generator=g).to(dt) for d in (dk, dk, dv))
+    keep = torch.rand(b, n, generator=g) > 0.1
+    sig = torch.sigmoid(torch.randn(h, generator=g))
+    table = tf.gptj_sinusoid_table(n, rdim).float()
+    ids = torch.arange(n)[None, :].expand(b, n)
+    cnt = keep.double().cumsum(-1)                                                # kept keys at positions <= s (:241)
+    sin, cos = torch.split(table.double()[ids], rdim // 2, dim=-1)
+    rot = lambda x: torch.cat([tf.gptj_rotate(x[..., :rdim], sin, cos), x[..., rdim:]], -1)   # (B,N,H,D) layout
+    m = keep[:, :, None, None].double()
+    rq = (torch.nn.functional.normalize(rot(q.double()), dim=-1, p=2) * m).permute(0, 2, 1, 3)
+    rk = (torch.nn.functional.normalize(rot(k.double()), dim=-1, p=2) * m).permute(0, 2, 1, 3)
+    scale = (cnt[:, :, None, None] ** sig.double().reshape(1, 1, h, 1)).clamp(min=1)
+    rv = (v.double() / scale * m).permute(0, 2, 1, 3)
+    o, prepared = ct.causal_dot_product_prepared(q.to(DEV), k.to(DEV), v.to(DEV), keep=keep.to(DEV), cnt=cnt.float().to(DEV),
+                                                 sig=sig.to(DEV), rotary=(table.to(DEV), ids.contiguous().to(DEV)), bnhd=True)
+    for name, got, ref in zip(("q_hat", "k_hat", "v_hat"), prepared, (rq, rk, rv)):
+        check(name, got, ref.numpy(), TOL[dt])
+    check("O", o, oracle.causal(rq.contiguous(), rk.contiguous(), rv.contiguous()), TOL[dt])
