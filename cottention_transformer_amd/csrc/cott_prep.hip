@@ -173,8 +173,11 @@ __device__ __forceinline__ void split_row(long row, const PrepArgs &a, int &s, i
 // limited by instruction issue, not by bytes: the per-row work (index split, norm, division) is repeated by
 // every lane of the row, so two groups per lane (half as many wavefronts) are faster than one, while more
 // rows or groups per lane only cost registers.
-template <class ACC, bool BACKWARD, int NV, int R, bool ALL_BF16 = false>
+// PAIRED (with ALL_BF16, NV == 2, row widths multiples of 8): the two groups of a lane are neighbours, columns 8 l .. 8 l + 7,
+// and travel as one 16-byte load or store instead of two 8-byte ones (the kernel is bound by instruction issue).
+template <class ACC, bool BACKWARD, int NV, int R, bool ALL_BF16 = false, bool PAIRED = false>
 __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
+    static_assert(!PAIRED || (ALL_BF16 && NV == 2), "paired groups: bf16 tensors, two groups per lane");
     // ALL_BF16: every tensor is bf16, known at compile time: no type dispatch around the loads and stores (the block's
     // shapes, B8 H16 N2048 D64 in the projections' layout with rotary, mask and scale: forward 48.5 -> 44.8 us,
     // backward 97.8 -> 91.5 us per call)
@@ -186,6 +189,16 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
     const int rpb = kPrepThreads / lpr;
     const long row0 = ((long)blockIdx.x * R) * rpb + threadIdx.x / lpr;
     const int lane = threadIdx.x % lpr;
+    auto col_of = [&](int c) __attribute__((always_inline)) { return PAIRED ? 4 * (lane * NV + c) : 4 * (lane + c * lpr); };
+    auto unpack_pair = [&](u32x4 v, Vec4<ACC> &lo, Vec4<ACC> &hi) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            lo.x[2 * i] = (ACC)Bf16::to_float((u16)(v[i] & 0xffffu));
+            lo.x[2 * i + 1] = (ACC)Bf16::to_float((u16)(v[i] >> 16));
+            hi.x[2 * i] = (ACC)Bf16::to_float((u16)(v[2 + i] & 0xffffu));
+            hi.x[2 * i + 1] = (ACC)Bf16::to_float((u16)(v[2 + i] >> 16));
+        }
+    };
 
     Vec4<ACC> x[R][NV], g[R][NV];
     long rr[R];
@@ -214,9 +227,20 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
     }
 #pragma unroll
     for (int u = 0; u < R; ++u) {
+        if constexpr (PAIRED) {
+            const int col = col_of(0);
+            u32x4 xv = {0u, 0u, 0u, 0u}, gv = xv;
+            if (act[u] && col < D) {
+                xv = *reinterpret_cast<const u32x4 *>(static_cast<const u16 *>(a.x[t]) + xoff[u] + col);
+                if (BACKWARD) gv = *reinterpret_cast<const u32x4 *>(static_cast<const u16 *>(a.g[t]) + (size_t)rr[u] * D + col);
+            }
+            unpack_pair(xv, x[u][0], x[u][NV - 1]);
+            if (BACKWARD) unpack_pair(gv, g[u][0], g[u][NV - 1]);
+            continue;
+        }
 #pragma unroll
         for (int c = 0; c < NV; ++c) {
-            const int col = 4 * (lane + c * lpr);
+            const int col = col_of(c);
             if (act[u] && col < D) {
                 x[u][c] = load4<ACC>(a.x[t], x_dtype, xoff[u] + col);
                 if (BACKWARD) g[u][c] = load4<ACC>(a.g[t], g_dtype, (size_t)rr[u] * D + col);
@@ -239,7 +263,7 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
             const float *sc = a.rot + (size_t)tp * a.R;
 #pragma unroll
             for (int c = 0; c < NV; ++c) {
-                const int col = 4 * (lane + c * lpr);
+                const int col = col_of(c);
                 if (col < a.R) {
                     sn[u][c] = *reinterpret_cast<const f32x2 *>(sc + col / 2);
                     cs[u][c] = *reinterpret_cast<const f32x2 *>(sc + col / 2 + a.R / 2);
@@ -257,7 +281,7 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
         if (rotary) {
 #pragma unroll
             for (int c = 0; c < NV; ++c) {
-                const int col = 4 * (lane + c * lpr);
+                const int col = col_of(c);
                 if (col < a.R) rotate4(x[u][c], sn[u][c], cs[u][c], false);
             }
         }
@@ -306,17 +330,28 @@ __global__ __launch_bounds__(kPrepThreads) void prep_kernel(PrepArgs a) {
                 }
             }
         }
+        u32x4 ypair;
 #pragma unroll
         for (int c = 0; c < NV; ++c) {
-            const int col = 4 * (lane + c * lpr);
+            const int col = col_of(c);
             if (act[u] && col < D) {
                 Vec4<ACC> y;
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     y.x[i] = BACKWARD ? mul_g * g[u][c].x[i] + mul_x * x[u][c].x[i] : mul_x * x[u][c].x[i];
                 if (BACKWARD && rotary && col < a.R) rotate4(y, sn[u][c], cs[u][c], true);
-                store4<ACC>(a.y[t], BACKWARD ? x_dtype : y_dtype, (BACKWARD ? xoff[u] : (size_t)r * D) + col, y);
+                if constexpr (PAIRED) {
+                    ypair[2 * c] = Bf16::pack2((float)y.x[0], (float)y.x[1]);
+                    ypair[2 * c + 1] = Bf16::pack2((float)y.x[2], (float)y.x[3]);
+                } else {
+                    store4<ACC>(a.y[t], BACKWARD ? x_dtype : y_dtype, (BACKWARD ? xoff[u] : (size_t)r * D) + col, y);
+                }
             }
+        }
+        if constexpr (PAIRED) {
+            const int col = col_of(0);
+            if (act[u] && col < D)
+                *reinterpret_cast<u32x4 *>(static_cast<u16 *>(a.y[t]) + (BACKWARD ? xoff[u] : (size_t)r * D) + col) = ypair;
         }
     }
 }
@@ -371,9 +406,13 @@ hipError_t launch_prep(bool backward, const void *const x[3], const void *const 
     const dim3 grid((unsigned)blocks, 3), blk(kPrepThreads);
     const bool f64 = x_dtype == COTT_F64;
     const bool all_bf16 = x_dtype == COTT_BF16 && y_dtype == COTT_BF16 && (!backward || g_dtype == COTT_BF16);
+    // rows whose lanes can take 16 bytes each: widths multiples of 8 (16-byte aligned rows in either layout) that fill
+    // the two groups of every lane, or leave whole lanes empty
+    const bool paired = dk % 8 == 0 && dv % 8 == 0;
 #define COTT_PREP(ACC, BWD) \
     do { \
         if (wide) prep_kernel<ACC, BWD, kMaxVec, 1><<<grid, blk, 0, stream>>>(a); \
+        else if (nv == 2 && all_bf16 && paired) prep_kernel<float, BWD, 2, 2, true, true><<<grid, blk, 0, stream>>>(a); \
         else if (nv == 2 && all_bf16) prep_kernel<ACC, BWD, 2, 2, true><<<grid, blk, 0, stream>>>(a); \
         else if (nv == 2) prep_kernel<ACC, BWD, 2, 2><<<grid, blk, 0, stream>>>(a); \
         else prep_kernel<ACC, BWD, 1, 2><<<grid, blk, 0, stream>>>(a); \
