@@ -449,10 +449,25 @@ def run_extras(torch, ct, dev):
     cf = cold_kernel_us(torch, lambda: ct.noncausal_dot_product(q, k, v), "apply", big)
     cb = cold_kernel_us(torch, lambda: ct.noncausal_backward(q, k, v, do), "apply", big)
     tb = b * h * n * d * 2
+    # beside them the kernel that only streams the same tensors in a launch of as many workgroups as there are heads
+    # (cott_stream_probe; the non-causal kernels read k, v and then q in two passes, the probe in one)
+    from cottention_transformer_amd import _loader
+    src = torch.ones(4 * tb // 4, dtype=torch.int32, device=dev)
+    dst = torch.zeros(3 * tb // 4, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def probe(nr, nw):
+        def fn():
+            if _loader.lib().cott_stream_probe(src.data_ptr(), dst.data_ptr(), tb, nr, nw, b * h, 8192, stream) != _loader.OK:
+                raise RuntimeError("cott_stream_probe refused the launch")
+        return fn
     ex["noncausal_cold_cache_B32_H12_N512_D64"] = {
         "fwd_kernel_us": cf, "fwd_frac_hbm": 4 * tb / (cf * 1e-6) / 1e9 / HBM_PEAK_GBS, "fwd_tokens_per_s": b * n / (cf * 1e-6),
-        "bwd_kernel_us": cb, "bwd_frac_hbm": 7 * tb / (cb * 1e-6) / 1e9 / HBM_PEAK_GBS}
-    del q, k, v, do, big
+        "bwd_kernel_us": cb, "bwd_frac_hbm": 7 * tb / (cb * 1e-6) / 1e9 / HBM_PEAK_GBS,
+        "streaming_only": {"workgroups": b * h, "block_bytes": 8192,
+                           "fwd_shape_3_reads_1_write_us": cold_kernel_us(torch, probe(3, 1), "stream_probe", big),
+                           "grad_shape_4_reads_3_writes_us": cold_kernel_us(torch, probe(4, 3), "stream_probe", big)}}
+    del q, k, v, do, big, src, dst
     # recurrent decode, state (256,16,128,128) fp32, 512 consecutive steps with fresh q,k,v per step
     b, h, d, steps = 256, 16, 128, 512
     g = torch.Generator(device=dev).manual_seed(0)
