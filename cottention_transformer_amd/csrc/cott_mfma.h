@@ -1576,14 +1576,24 @@ __global__ __launch_bounds__(kThreads) void noncausal_kernel(ProblemSet set, int
                 }
             }
             if (PF2 == PF || p + PF2 < nchunks) load_q(s, p + PF2);
+            // The 16 output rows of this wavefront go through its own staging rows in the first C tile (free since the
+            // hand-over) and leave as 16-byte pieces of whole rows: 8-byte accumulator pieces written straight to
+            // memory are quarter cache lines that have to meet in L2.  (One wavefront's LDS accesses execute in order.)
+            u16 *sW = sC + (16 * w) * TL::CS;
 #pragma unroll
             for (int jt = 0; jt < TL::NJT; ++jt) {
                 f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jt][ks], qc[ks], o);
-                const int col = 16 * jt + 4 * g;
-                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldo + col) * 2u : kOobOffset;
-                buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
+                *reinterpret_cast<u32x2 *>(sW + m * TL::CS + 16 * jt + 4 * g) = u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
+            }
+            constexpr int PPR = DJ / 8;  // 16-byte pieces per row
+#pragma unroll
+            for (int u = 0; u < DJ / 32; ++u) {
+                const int v = l + 64 * u, lrow = v / PPR, col = (v % PPR) * 8;
+                const u32x4 val = *reinterpret_cast<const u32x4 *>(sW + lrow * TL::CS + col);
+                const uint32_t off = (col < dj) ? (uint32_t)((p * kChunk + 16 * w + lrow) * ldo + col) * 2u : kOobOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(val, rO, (int)off, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the next chunk's waits out of this one
         }
