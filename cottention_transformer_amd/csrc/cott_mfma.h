@@ -1329,6 +1329,7 @@ template <class TR, int DI, int DJ, int PF>
 __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH, int N, int nchunks, int cpg, int G) {
     using TL = Tiling<DI, DJ>;
     __shared__ __attribute__((aligned(16))) u16 sS[DJ * TL::SS];
+    __shared__ __attribute__((aligned(16))) u16 sOw[kChunk * TL::CS];  // 16 staging rows per wavefront for its outputs
     const int tid = threadIdx.x, l = tid & 63, g = l >> 4, m = l & 15;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const WorkItem wi = decode_workgroup(set.count, BH, set.xcds);
@@ -1371,15 +1372,22 @@ __global__ __launch_bounds__(kThreads) void apply_kernel(ProblemSet set, int BH,
 #pragma unroll
             for (int ks = 0; ks < TL::KS; ++ks) qc[ks] = (32 * ks + 8 * g < di) ? qn[s][ks] : u32x4{0u, 0u, 0u, 0u};
             load_q(s, p + PF);
-            const int orow = p * kChunk + 16 * w + m;
+            // (outputs staged per wavefront and stored as 16-byte pieces of whole rows, as in noncausal_kernel)
+            u16 *sW = sOw + (16 * w) * TL::CS;
 #pragma unroll
             for (int jt = 0; jt < TL::NJT; ++jt) {
                 f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < TL::KS; ++ks) o = TR::mfma(sf[jt][ks], qc[ks], o);
-                const int col = 16 * jt + 4 * g;
-                const uint32_t off = (col < dj) ? (uint32_t)(orow * ldo + col) * 2u : kOobOffset;
-                buf_store8(rO, off, u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])});
+                *reinterpret_cast<u32x2 *>(sW + m * TL::CS + 16 * jt + 4 * g) = u32x2{TR::pack2(o[0], o[1]), TR::pack2(o[2], o[3])};
+            }
+            constexpr int PPR = DJ / 8;  // 16-byte pieces per row
+#pragma unroll
+            for (int u = 0; u < DJ / 32; ++u) {
+                const int v = l + 64 * u, lrow = v / PPR, col = (v % PPR) * 8;
+                const u32x4 val = *reinterpret_cast<const u32x4 *>(sW + lrow * TL::CS + col);
+                const uint32_t off = (col < dj) ? (uint32_t)((p * kChunk + 16 * w + lrow) * ldo + col) * 2u : kOobOffset;
+                __builtin_amdgcn_raw_buffer_store_b128(val, rO, (int)off, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the next chunk's waits out of this one
         }
