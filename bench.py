@@ -25,7 +25,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # `bench.py --calibration-copy` (counters scaled by their reading for the 256 MiB copy in the same run).
 # A counter run cannot be made from inside this script; the figures and commands are in
 # profiles/headline_kernels_hbm_traffic_pmc.txt.
-MEASURED_TRAFFIC_BYTES = {"scan": 127.21 * 2**20, "scan_grad": 223.43 * 2**20}
+MEASURED_TRAFFIC_BYTES = {"scan": 127.19 * 2**20, "scan_grad": 223.05 * 2**20}
 
 
 def parse():
